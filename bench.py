@@ -1,0 +1,180 @@
+#!/usr/bin/env python3
+"""Benchmark of the bandwidth-bound low-memory operators at ResNet-50 batch-184
+shapes (fp32) on one MI355X.
+
+A "step" is one pass of the hot path over one synthetic batch:
+  1. BatchNorm backward from the in-place OUTPUT on [184,256,56,56]
+  2. ReLU backward from the 1-bit mask on [184,256,56,56]
+  3. max-pool 3x3/s2/p1 backward from 4-bit indices, [184,64,56,56] -> [184,64,112,112]
+All inputs are resident in HBM before the timed region.  `value` is the
+algorithmic bytes of one step (each operand read once, each result written
+once) divided by the measured time per step.  Each operator is also timed on
+its own with events recorded on the launch stream; the BatchNorm backward
+(the dominant one) is reported in `roofline`, the others in `kernels`.
+
+The same operators are timed on the host's cores through the stock PyTorch
+CPU path on a slice of the batch (`cpu_baseline`).
+
+Prints one JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth, GB/s
+
+N, C, H, W = 184, 256, 56, 56          # BN / ReLU tensor
+PN, PC, PH_IN, PW_IN = 184, 64, 112, 112  # max-pool input
+E = N * C * H * W
+BYTES_BN = 3 * E * 4                    # read dy, read y, write dx
+BYTES_RELU = 2 * E * 4 + E // 8         # read dy, read mask, write dx
+BYTES_POOL = E * 4 + (E // 4) * 4 + (E // 4) // 2  # write dx, read dy, read packed idx
+BYTES_STEP = BYTES_BN + BYTES_RELU + BYTES_POOL
+
+
+def gpu_bench(steps, warmup):
+    import torch
+
+    import monet_amd.lm_ops as lm_ops
+    from monet_amd.lm_ops import bn as bn_ops
+    from monet_amd.lm_ops import pool as pool_ops
+    from monet_amd.lm_ops import relu as relu_ops
+
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    # --- BN-from-output inputs: y = BN_train(x), dy ~ N(0,1)
+    x = torch.randn(N, C, H, W, device=dev)
+    gamma = torch.rand(C, device=dev) + 0.5
+    beta = torch.randn(C, device=dev) * 0.1
+    y, save_mean, save_invstd = bn_ops.bn_forward_train(x, gamma, beta, None, None, 0.1, 1e-5)
+    dy = torch.randn(N, C, H, W, device=dev)
+    # --- ReLU mask of an N(0,1) tensor; the backward runs in place on its own gradient copy
+    _, mask = relu_ops.relu_forward_with_mask(x, want_output=False)
+    g_relu = torch.randn(N, C, H, W, device=dev)
+    del x
+    # --- max-pool indices of an N(0,1) tensor
+    px = torch.randn(PN, PC, PH_IN, PW_IN, device=dev)
+    _, idx4, geo = pool_ops.max_pool2d_with_packed_indices(px, 3, 2, 1, 1, False)
+    pdy = torch.randn(PN, PC, PH_IN // 2, PW_IN // 2, device=dev)
+    in_shape = list(px.shape)
+    del px
+    torch.cuda.synchronize()
+
+    def op_bn():
+        return bn_ops.bn_backward_from_output(dy, y, gamma, beta, save_invstd)
+
+    def op_relu():
+        return relu_ops.relu_backward_from_mask(g_relu, mask)
+
+    def op_pool():
+        return pool_ops.max_pool2d_backward_from_packed_indices(pdy, idx4, geo, in_shape)
+
+    ops = [("bn_bwd_from_output", op_bn, BYTES_BN), ("relu_bwd_mask", op_relu, BYTES_RELU),
+           ("maxpool_bwd_idx", op_pool, BYTES_POOL)]
+    for _ in range(warmup):
+        for _, fn, _ in ops:
+            fn()
+    torch.cuda.synchronize()
+    ev = {name: [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+                 for _ in range(steps)] for name, _, _ in ops}
+    t0 = time.perf_counter()
+    for k in range(steps):
+        for name, fn, _ in ops:
+            a, b = ev[name][k]
+            a.record()
+            fn()
+            b.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / steps
+    kernels = {}
+    for name, _, nbytes in ops:
+        ms = sum(a.elapsed_time(b) for a, b in ev[name]) / steps
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        kernels[name] = {"ms": round(ms, 4), "bytes": nbytes, "GB/s": round(gbs, 1),
+                         "frac": round(gbs / HBM_PEAK_GBS, 4)}
+    return ms_per_step, kernels
+
+
+def cpu_baseline(sample_n=23, reps=5):
+    """Stock PyTorch CPU operators on `sample_n` of the 184 images, all host threads."""
+    import torch
+
+    from oracle import cpu_path
+
+    threads = torch.get_num_threads()
+    torch.manual_seed(0)
+    x = torch.randn(sample_n, C, H, W)
+    gamma = torch.rand(C) + 0.5
+    beta = torch.randn(C) * 0.1
+    y, mean, invstd = cpu_path.bn_forward(x, gamma, beta)
+    dy = torch.randn_like(x)
+    px = torch.randn(sample_n, PC, PH_IN, PW_IN)
+    py, pidx = cpu_path.maxpool_forward(px, 3, 2, 1)
+    pdy = torch.randn_like(py)
+
+    def step():
+        cpu_path.bn_backward(dy, x, gamma, mean, invstd)
+        cpu_path.relu_backward(dy, y)
+        cpu_path.maxpool_backward(pdy, px, 3, 2, 1, pidx)
+
+    step()  # warm-up
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        step()
+        times.append(time.perf_counter() - t0)
+    med = sorted(times)[len(times) // 2]
+    nbytes = BYTES_STEP * sample_n / N
+    return {"value": round(nbytes / med / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"{sample_n} of {N} images of the same three operators through stock PyTorch "
+                      f"CPU ops (torch {torch.__version__}), 1 warm-up + median of {reps}"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    ms_per_step, kernels = gpu_bench(args.steps, args.warmup)
+    value = BYTES_STEP / (ms_per_step * 1e-3) / 1e9
+    bn = kernels["bn_bwd_from_output"]
+    out = {
+        "metric": "lm_ops HBM GB/s (algorithmic bytes / time; BN-from-output bwd + ReLU-mask bwd "
+                  "+ maxpool-index bwd at ResNet-50 bs184 shapes)",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "isolated bandwidth-bound lm_ops at ResNet-50 bs184 shapes, fp32: "
+                               "BN bwd from output [184,256,56,56]; ReLU 1-bit-mask bwd "
+                               "[184,256,56,56]; maxpool3x3s2 bwd [184,64,56,56]->[184,64,112,112]",
+                   "bytes_per_step": BYTES_STEP},
+        "roofline": {"bound": "hbm", "kernel": "bn_bwd_from_output (reduce + apply launches)",
+                     "achieved": bn["GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": bn["frac"], "traffic": None},
+        "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

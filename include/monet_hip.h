@@ -1,0 +1,163 @@
+/*
+ * monet_hip.h - C ABI of libmonet_hip.so, the gfx950 (MI355X) kernels behind
+ * the low-memory operator library (the lm_ops op classes).
+ *
+ * Conventions shared by every entry point
+ *   - Every pointer is a raw DEVICE pointer into memory owned by the caller
+ *     (inputs, outputs and workspaces).  The library never allocates, frees or
+ *     caches device memory and keeps no mutable global state, so it is
+ *     re-entrant; the caller's allocator sees every byte that is used.
+ *   - `stream` is a hipStream_t passed as void*; all work is enqueued on it and
+ *     no entry point synchronises with the host.
+ *   - Return value: MN_OK (0) or one of the MN_E* codes below.  Nothing throws
+ *     or exits across the boundary.  mn_status_string() names a code.
+ *   - Tensors are dense, row-major (NCHW for 4-D), fp32 unless the name says
+ *     otherwise.  "In place" is allowed exactly where a comment says so.
+ *
+ * Each declaration cites the function of the reference implementation
+ * (utsaslab/MONeT, paths relative to its root) whose role it takes over.
+ */
+#ifndef MONET_HIP_H
+#define MONET_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MN_OK 0
+#define MN_EINVAL 1       /* null pointer, negative size, misaligned operand, ws too small */
+#define MN_EUNSUPPORTED 2 /* shape / variant / dtype this build has no kernel for */
+#define MN_ELAUNCH 3      /* hipGetLastError() reported a failed launch */
+
+typedef void* mn_stream_t;
+
+/* ABI version of this header; bumped on any signature change. */
+int mn_abi_version(void);
+const char* mn_status_string(int status);
+
+/* ------------------------------------------------------------------ pack --
+ * 1-bit pack: n bytes (each 0 or 1) -> (n+7)/8 bytes, first element in bit 7
+ * of byte 0, tail bits zero.  Replaces pack / pack_ (monet/lm_ops/pack.cpp:72-98,
+ * kernel monet/lm_ops/pack.cu:22-31). */
+int mn_pack_bits(const uint8_t* bools, uint8_t* packed, size_t n, mn_stream_t stream);
+/* Inverse: writes n bytes of 0/1.  Replaces unpack (pack.cpp:99-111, pack.cu:32-40). */
+int mn_unpack_bits(const uint8_t* packed, uint8_t* bools, size_t n, mn_stream_t stream);
+/* r[i] = bit(i) * v[i]; r may alias v.  Replaces unpack_multiply
+ * (pack.cpp:112-131, pack.cu:41-50). */
+int mn_unpack_bits_mul_f32(const uint8_t* packed, const float* v, float* r, size_t n,
+                           mn_stream_t stream);
+/* 4-bit pack: n bytes (each < 16) -> (n+1)/2 bytes, element 2j in the high
+ * nibble of byte j, 2j+1 in the low nibble, tail nibble zero.  Replaces
+ * pack_two (pack.cpp:38-54, pack.cu:3-12). */
+int mn_pack_nibbles(const uint8_t* u, uint8_t* packed, size_t n, mn_stream_t stream);
+/* Inverse: writes n bytes.  Replaces unpack_two (pack.cpp:55-70, pack.cu:13-21). */
+int mn_unpack_nibbles(const uint8_t* packed, uint8_t* u, size_t n, mn_stream_t stream);
+
+/* ------------------------------------------------------------------ relu --
+ * Fused y = max(x, 0) (NaN propagates) and mask = pack(x > 0) in one pass.
+ * y may alias x (in-place ReLU); y may be NULL to produce the mask only.
+ * Replaces the clamp_min + (x > 0) + pack sequence of BinaryActReLU.forward /
+ * .intermediate (monet/lm_ops/relu.py:100-107). */
+int mn_relu_fwd_mask_f32(const float* x, float* y, uint8_t* mask, size_t n, mn_stream_t stream);
+/* dx[i] = bit(i) ? grad[i] : grad[i] * 0 (so NaN/inf and the sign of zero
+ * behave like the multiply in the reference).  dx may alias grad.  Replaces
+ * unpack + in-place multiply of BinaryActReLU.backward (relu.py:109-118). */
+int mn_relu_bwd_mask_f32(const float* grad, const uint8_t* mask, float* dx, size_t n,
+                         mn_stream_t stream);
+/* dx[i] = ref[i] > threshold ? grad[i] : 0 with ref the stored ReLU input or
+ * output.  dx may alias grad.  Replaces relu_backward / threshold_kernel
+ * (monet/lm_ops/lrrelu.cpp:11-20, lrrelu.cu:4-15). */
+int mn_relu_bwd_ref_f32(const float* grad, const float* ref, float threshold, float* dx, size_t n,
+                        mn_stream_t stream);
+
+/* --------------------------------------------------------------- maxpool --
+ * Geometry of a 2-D max pool over an NCHW tensor.  PH/PW are the output sizes
+ * (mn_pool_out_size gives them). */
+typedef struct mn_pool2d {
+  int32_t N, C, H, W;
+  int32_t kH, kW, sH, sW, pH, pW, dH, dW;
+  int32_t PH, PW;
+} mn_pool2d;
+
+/* Output extent along one axis; the rule of pooling_output_shape
+ * (monet/lm_ops/maxpool.cpp:54-75).  Returns -1 on invalid arguments. */
+int64_t mn_pool_out_size(int64_t in, int64_t k, int64_t pad, int64_t stride, int64_t dil,
+                         int ceil_mode);
+/* y = max over each window; idx4 = the window-relative argmax ch*kW+cw (rows
+ * and columns counted from the unclipped window origin, first maximum in
+ * row-major order wins, a NaN always wins) packed two per byte like
+ * mn_pack_nibbles over the flat NCHW output order.  Needs kH*kW <= 16.
+ * Replaces max_pool2d_with_indices_cuda + pack_two of
+ * IndicesActMaxPool2D.forward (monet/lm_ops/pool.py:43-53,
+ * maxpool.cpp:369-405, kernel maxpool.cu:26-72). */
+int mn_maxpool_fwd_idx_f32(const mn_pool2d* g, const float* x, float* y, uint8_t* idx4,
+                           mn_stream_t stream);
+/* dx[n,c,h,w] = sum of dy over the windows that cover (h,w) and whose stored
+ * index names it (window rows outer, columns inner).  Writes every element of
+ * dx, so dx needs no clearing.  Replaces unpack_two + zeros +
+ * max_pool2d_with_indices_backward_out_cuda of IndicesActMaxPool2D.backward
+ * (pool.py:55-69, maxpool.cpp:407-435, kernel maxpool.cu:81-131). */
+int mn_maxpool_bwd_idx_f32(const mn_pool2d* g, const float* dy, const uint8_t* idx4, float* dx,
+                           mn_stream_t stream);
+
+/* ------------------------------------------------------------- batchnorm --
+ * All BN entry points view the tensor as [N, C, HW] and reduce over N and HW.
+ * Bytes of caller-provided workspace the BN entry points need for a tensor of
+ * this shape (cross-workgroup partial sums). */
+size_t mn_bn_ws_bytes(int64_t N, int64_t C, int64_t HW);
+/* Training forward: batch mean / biased variance per channel, y = (x - mean) *
+ * invstd * gamma + beta, running_mean/var updated in place with `momentum`
+ * (unbiased variance), save_mean / save_invstd written.  gamma / beta may be
+ * NULL (1 / 0); running_* may be NULL.  y may alias x.  Replaces do_forward
+ * -> cudnn_batch_norm (monet/lm_ops/lrbn.cpp:21-41). */
+int mn_bn_fwd_train_f32(const float* x, const float* gamma, const float* beta, float* running_mean,
+                        float* running_var, float* y, float* save_mean, float* save_invstd,
+                        int64_t N, int64_t C, int64_t HW, double momentum, double eps, void* ws,
+                        size_t ws_bytes, mn_stream_t stream);
+/* Recompute forward from saved statistics: y = (x - mean) * invstd * gamma +
+ * beta.  y may alias x.  Takes the role of the F.batch_norm call in
+ * InputActBatchNorm.forward when params are set (monet/lm_ops/bn.py:32-34). */
+int mn_bn_fwd_apply_f32(const float* x, const float* mean, const float* invstd, const float* gamma,
+                        const float* beta, float* y, int64_t N, int64_t C, int64_t HW,
+                        mn_stream_t stream);
+/* Backward from the INPUT x: dgamma = sum dy*xhat, dbeta = sum dy,
+ * dx = (dy - xhat*dgamma/M - dbeta/M) * invstd * gamma, xhat = (x-mean)*invstd.
+ * dx may alias dy.  Replaces do_cudnn_backward -> cudnn_batch_norm_backward
+ * (monet/lm_ops/lrbn.cpp:43-70). */
+int mn_bn_bwd_from_x_f32(const float* dy, const float* x, const float* gamma, const float* mean,
+                         const float* invstd, float* dx, float* dgamma, float* dbeta, int64_t N,
+                         int64_t C, int64_t HW, void* ws, size_t ws_bytes, mn_stream_t stream);
+/* Backward from the OUTPUT y (the input is never read): gsum = sum dy,
+ * dot = sum dy*(y-beta); dbeta = gsum, dgamma = dot/gamma,
+ * dx = (dy - (y-beta)*dot/(M*gamma^2) - gsum/M) * invstd * gamma.  Undefined
+ * for gamma == 0, like the reference.  dx may alias dy.  Replaces
+ * output_activated_bn_backward (monet/lm_ops/lrbn.cpp:154-172, kernel
+ * batch_norm_backward_kernel1 monet/lm_ops/lrbn.cu:138-209). */
+int mn_bn_bwd_from_y_f32(const float* dy, const float* y, const float* gamma, const float* beta,
+                         const float* invstd, float* dx, float* dgamma, float* dbeta, int64_t N,
+                         int64_t C, int64_t HW, void* ws, size_t ws_bytes, mn_stream_t stream);
+
+/* --------------------------------------------------------------- softmax --
+ * The tensor is viewed as [outer, dim, inner]; softmax runs over `dim`.
+ * Replaces softmax_forward (monet/lm_ops/softmax.cpp:11-15). */
+int mn_softmax_fwd_f32(const float* x, float* y, int64_t outer, int64_t dim, int64_t inner,
+                       mn_stream_t stream);
+/* dx = dy*y - y * sum_dim(dy*y), without materialising dy*y.  dx may alias dy.
+ * Replaces softmax_backward1 (monet/lm_ops/softmax.cpp:17-33). */
+int mn_softmax_bwd_f32(const float* dy, const float* y, float* dx, int64_t outer, int64_t dim,
+                       int64_t inner, mn_stream_t stream);
+/* Fused backward of mean-reduced softmax cross-entropy over [outer, dim,
+ * inner] logits with int64 labels [outer, inner]:
+ * dlogits = (softmax(logits) - onehot(label)) * scale.  The reference applies
+ * the loss outside its operator library with the stock nn.CrossEntropyLoss
+ * (examples/imagenet.py:199,327); this is the fused kernel for that step. */
+int mn_xent_bwd_f32(const float* logits, const int64_t* labels, float* dlogits, int64_t outer,
+                    int64_t dim, int64_t inner, float scale, mn_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MONET_HIP_H */

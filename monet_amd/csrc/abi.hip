@@ -1,0 +1,23 @@
+// ABI bookkeeping entry points of libmonet_hip.so.
+#include "common.h"
+
+extern "C" {
+
+int mn_abi_version(void) { return 1; }
+
+const char* mn_status_string(int status) {
+  switch (status) {
+    case MN_OK:
+      return "ok";
+    case MN_EINVAL:
+      return "invalid argument (null pointer, bad size, misaligned operand or workspace too small)";
+    case MN_EUNSUPPORTED:
+      return "unsupported shape, variant or dtype";
+    case MN_ELAUNCH:
+      return "kernel launch failed";
+    default:
+      return "unknown status";
+  }
+}
+
+}  // extern "C"

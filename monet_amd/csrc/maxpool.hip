@@ -1,0 +1,262 @@
+// Max-pool forward with 4-bit window-relative argmax indices, and the
+// backward that gathers from them.  Index of a window element =
+// ch*kW + cw, where (ch, cw) count rows / columns from the UNCLIPPED window
+// origin (ph*sH - pH, pw*sW - pW) in steps of the dilation.
+#include "common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+
+// Geometry with compile-time constants (K == kernel, S == stride, P == pad,
+// dilation 1) or, for the generic case, run-time fields.
+template <int K, int S, int P>
+struct CtGeo {
+  __device__ __forceinline__ int kH() const { return K; }
+  __device__ __forceinline__ int kW() const { return K; }
+  __device__ __forceinline__ int sH() const { return S; }
+  __device__ __forceinline__ int sW() const { return S; }
+  __device__ __forceinline__ int pH() const { return P; }
+  __device__ __forceinline__ int pW() const { return P; }
+  __device__ __forceinline__ int dH() const { return 1; }
+  __device__ __forceinline__ int dW() const { return 1; }
+};
+struct RtGeo {
+  int kh, kw, sh, sw, ph, pw, dh, dw;
+  __device__ __forceinline__ int kH() const { return kh; }
+  __device__ __forceinline__ int kW() const { return kw; }
+  __device__ __forceinline__ int sH() const { return sh; }
+  __device__ __forceinline__ int sW() const { return sw; }
+  __device__ __forceinline__ int pH() const { return ph; }
+  __device__ __forceinline__ int pW() const { return pw; }
+  __device__ __forceinline__ int dH() const { return dh; }
+  __device__ __forceinline__ int dW() const { return dw; }
+};
+
+// One output element: scan the window row-major; a strictly larger value or a
+// NaN takes over.  If nothing does (window of -inf) the first valid element
+// is reported.
+template <class G>
+__device__ __forceinline__ void pool_one(const G g, const float* __restrict__ xp, int H, int W,
+                                         int ph, int pw, float& best, uint32_t& bidx) {
+  int hstart = ph * g.sH() - g.pH();
+  int wstart = pw * g.sW() - g.pW();
+  const int hend = min(hstart + (g.kH() - 1) * g.dH() + 1, H);
+  const int wend = min(wstart + (g.kW() - 1) * g.dW() + 1, W);
+  int ch0 = 0, cw0 = 0;
+  while (hstart < 0) {
+    hstart += g.dH();
+    ++ch0;
+  }
+  while (wstart < 0) {
+    wstart += g.dW();
+    ++cw0;
+  }
+  float maxval = -INFINITY;
+  uint32_t maxidx = ch0 * g.kW() + cw0;
+  int ch = ch0;
+  for (int h = hstart; h < hend; h += g.dH(), ++ch) {
+    int cw = cw0;
+    for (int w = wstart; w < wend; w += g.dW(), ++cw) {
+      const float val = xp[(size_t)h * W + w];
+      if (val > maxval || val != val) {
+        maxidx = ch * g.kW() + cw;
+        maxval = val;
+      }
+    }
+  }
+  best = maxval;
+  bidx = maxidx;
+}
+
+// One thread per PAIR of consecutive outputs in flat NCHW order = one index
+// byte.  `total` = N*C*PH*PW.
+template <class G>
+__global__ __launch_bounds__(kThreads) void maxpool_fwd_idx_kernel(
+    const G g, const float* __restrict__ x, float* __restrict__ y, uint8_t* __restrict__ idx4,
+    int H, int W, int PH, int PW, size_t total) {
+  const size_t j = (size_t)blockIdx.x * kThreads + threadIdx.x;
+  const size_t o0 = 2 * j;
+  if (o0 >= total) return;
+  const uint32_t plane_sz = (uint32_t)PH * PW;
+  size_t plane = o0 / plane_sz;
+  uint32_t r = (uint32_t)(o0 - plane * plane_sz);
+  int ph = r / PW;
+  int pw = r - ph * PW;
+  float v0, v1 = 0.f;
+  uint32_t i0, i1 = 0;
+  pool_one(g, x + plane * (size_t)H * W, H, W, ph, pw, v0, i0);
+  y[o0] = v0;
+  if (o0 + 1 < total) {
+    if (++pw == PW) {
+      pw = 0;
+      if (++ph == PH) {
+        ph = 0;
+        ++plane;
+      }
+    }
+    pool_one(g, x + plane * (size_t)H * W, H, W, ph, pw, v1, i1);
+    y[o0 + 1] = v1;
+  }
+  idx4[j] = (uint8_t)(((i0 & 15u) << 4) | (i1 & 15u));
+}
+
+// Range of windows along one axis that cover input coordinate `c`.
+template <class G>
+__device__ __forceinline__ void cover(int c, int pad, int k, int dil, int stride, int pooled,
+                                      int& lo, int& hi) {
+  const int ext = (k - 1) * dil + 1;
+  lo = (c + pad < ext) ? 0 : (c + pad - ext) / stride + 1;
+  hi = min((c + pad) / stride + 1, pooled);
+}
+
+template <class G>
+__device__ __forceinline__ float pool_bwd_one(const G g, const float* __restrict__ dyp,
+                                              const uint8_t* __restrict__ idx4, size_t obase,
+                                              int PH, int PW, int h, int w) {
+  int ph0, ph1, pw0, pw1;
+  cover<G>(h, g.pH(), g.kH(), g.dH(), g.sH(), PH, ph0, ph1);
+  cover<G>(w, g.pW(), g.kW(), g.dW(), g.sW(), PW, pw0, pw1);
+  float grad = 0.f;
+  for (int ph = ph0; ph < ph1; ++ph) {
+    const int oh = h - ph * g.sH() + g.pH();
+    if (g.dH() != 1 && oh % g.dH() != 0) continue;
+    for (int pw = pw0; pw < pw1; ++pw) {
+      const int ow = w - pw * g.sW() + g.pW();
+      if (g.dW() != 1 && ow % g.dW() != 0) continue;
+      const uint32_t rel = (oh / g.dH()) * g.kW() + ow / g.dW();
+      const size_t o = obase + (size_t)ph * PW + pw;
+      const uint32_t b = idx4[o >> 1];
+      const uint32_t stored = (o & 1) ? (b & 15u) : (b >> 4);
+      if (stored == rel) grad += dyp[(size_t)ph * PW + pw];
+    }
+  }
+  return grad;
+}
+
+// grid = (chunks of a plane, planes); VEC consecutive w per thread.
+template <class G, int VEC>
+__global__ __launch_bounds__(kThreads) void maxpool_bwd_idx_kernel(
+    const G g, const float* __restrict__ dy, const uint8_t* __restrict__ idx4,
+    float* __restrict__ dx, int H, int W, int PH, int PW, uint32_t planes) {
+  const int WV = W / VEC;
+  const uint32_t per_plane = (uint32_t)H * WV;
+  const uint32_t t = blockIdx.x * kThreads + threadIdx.x;
+  if (t >= per_plane) return;
+  const int h = t / WV;
+  const int w0 = (t - h * WV) * VEC;
+  for (uint32_t plane = blockIdx.y; plane < planes; plane += gridDim.y) {
+    const size_t obase = (size_t)plane * PH * PW;
+    const float* dyp = dy + obase;
+    float r[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) r[v] = pool_bwd_one(g, dyp, idx4, obase, PH, PW, h, w0 + v);
+    float* out = dx + ((size_t)plane * H + h) * W + w0;
+    if (VEC == 4) {
+      float4_t q = {r[0], r[1], r[2], r[3]};
+      st_stream(reinterpret_cast<float4_t*>(out), q);
+    } else {
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) out[v] = r[v];
+    }
+  }
+}
+
+int check_geo(const mn_pool2d* g) {
+  if (!g) return MN_EINVAL;
+  if (g->N < 0 || g->C < 0 || g->H <= 0 || g->W <= 0 || g->PH <= 0 || g->PW <= 0) return MN_EINVAL;
+  if (g->kH <= 0 || g->kW <= 0 || g->sH <= 0 || g->sW <= 0 || g->dH <= 0 || g->dW <= 0)
+    return MN_EINVAL;
+  if (g->pH < 0 || g->pW < 0 || 2 * g->pH > g->kH || 2 * g->pW > g->kW) return MN_EINVAL;
+  if (g->kH * g->kW > 16) return MN_EUNSUPPORTED;  // index must fit a nibble
+  // every window must start inside the padded image and hold >= 1 real element
+  if ((int64_t)(g->PH - 1) * g->sH >= (int64_t)g->H + g->pH) return MN_EINVAL;
+  if ((int64_t)(g->PW - 1) * g->sW >= (int64_t)g->W + g->pW) return MN_EINVAL;
+  if ((int64_t)g->H * g->W >= (1ll << 31) || (int64_t)g->PH * g->PW >= (1ll << 31))
+    return MN_EUNSUPPORTED;
+  return MN_OK;
+}
+
+template <class G>
+void launch_fwd(const G geo, const mn_pool2d* g, const float* x, float* y, uint8_t* idx4,
+                hipStream_t s) {
+  const size_t total = (size_t)g->N * g->C * g->PH * g->PW;
+  const size_t pairs = (total + 1) / 2;
+  const unsigned blocks = (unsigned)((pairs + kThreads - 1) / kThreads);
+  maxpool_fwd_idx_kernel<G><<<blocks, kThreads, 0, s>>>(geo, x, y, idx4, g->H, g->W, g->PH, g->PW,
+                                                        total);
+}
+
+template <class G>
+void launch_bwd(const G geo, const mn_pool2d* g, const float* dy, const uint8_t* idx4, float* dx,
+                hipStream_t s) {
+  const uint32_t planes = (uint32_t)g->N * g->C;
+  const bool vec = (g->W % 4 == 0) && mn_aligned(dx, 16);
+  const uint32_t per_plane = (uint32_t)g->H * (vec ? g->W / 4 : g->W);
+  dim3 grid((per_plane + kThreads - 1) / kThreads, planes < 65535u ? planes : 65535u);
+  if (vec)
+    maxpool_bwd_idx_kernel<G, 4><<<grid, kThreads, 0, s>>>(geo, dy, idx4, dx, g->H, g->W, g->PH,
+                                                           g->PW, planes);
+  else
+    maxpool_bwd_idx_kernel<G, 1><<<grid, kThreads, 0, s>>>(geo, dy, idx4, dx, g->H, g->W, g->PH,
+                                                           g->PW, planes);
+}
+
+bool is_ct(const mn_pool2d* g, int k, int s, int p) {
+  return g->kH == k && g->kW == k && g->sH == s && g->sW == s && g->pH == p && g->pW == p &&
+         g->dH == 1 && g->dW == 1;
+}
+
+RtGeo rt(const mn_pool2d* g) {
+  return RtGeo{g->kH, g->kW, g->sH, g->sW, g->pH, g->pW, g->dH, g->dW};
+}
+
+}  // namespace
+
+extern "C" {
+
+int64_t mn_pool_out_size(int64_t in, int64_t k, int64_t pad, int64_t stride, int64_t dil,
+                         int ceil_mode) {
+  if (in <= 0 || k <= 0 || stride <= 0 || dil <= 0 || pad < 0) return -1;
+  const int64_t num = in + 2 * pad - dil * (k - 1) - 1 + (ceil_mode ? stride - 1 : 0);
+  // floor division (num may be negative)
+  int64_t q = num / stride;
+  if ((num % stride != 0) && ((num < 0) != (stride < 0))) --q;
+  int64_t out = q + 1;
+  if (pad && (out - 1) * stride >= in + pad) --out;  // last window must start inside the image
+  return out;
+}
+
+int mn_maxpool_fwd_idx_f32(const mn_pool2d* g, const float* x, float* y, uint8_t* idx4,
+                           mn_stream_t stream) {
+  const int st = check_geo(g);
+  if (st != MN_OK) return st;
+  if ((size_t)g->N * g->C == 0) return MN_OK;
+  if (!x || !y || !idx4) return MN_EINVAL;
+  hipStream_t s = mn_stream(stream);
+  if (is_ct(g, 3, 2, 1))
+    launch_fwd(CtGeo<3, 2, 1>{}, g, x, y, idx4, s);
+  else if (is_ct(g, 2, 2, 0))
+    launch_fwd(CtGeo<2, 2, 0>{}, g, x, y, idx4, s);
+  else
+    launch_fwd(rt(g), g, x, y, idx4, s);
+  return mn_launch_status();
+}
+
+int mn_maxpool_bwd_idx_f32(const mn_pool2d* g, const float* dy, const uint8_t* idx4, float* dx,
+                           mn_stream_t stream) {
+  const int st = check_geo(g);
+  if (st != MN_OK) return st;
+  if ((size_t)g->N * g->C == 0) return MN_OK;
+  if (!dy || !dx || !idx4) return MN_EINVAL;
+  hipStream_t s = mn_stream(stream);
+  if (is_ct(g, 3, 2, 1))
+    launch_bwd(CtGeo<3, 2, 1>{}, g, dy, idx4, dx, s);
+  else if (is_ct(g, 2, 2, 0))
+    launch_bwd(CtGeo<2, 2, 0>{}, g, dy, idx4, dx, s);
+  else
+    launch_bwd(rt(g), g, dy, idx4, dx, s);
+  return mn_launch_status();
+}
+
+}  // extern "C"

@@ -1,0 +1,141 @@
+"""BatchNorm operator implementations (reference: monet/lm_ops/bn.py).
+
+  InputActBatchNorm    backward from the stored INPUT   (bn.py:12-54)
+  OutputActBatchNorm   backward from the stored OUTPUT  (bn.py:96-140), so an
+                       in-place consumer chain can drop the input.
+
+Both share the forward: the first forward of an iteration computes batch
+statistics, updates the running statistics and records
+`params = (training, eps, save_mean, save_invstd, reserve)`; a forward on an
+instance whose `params` are already set is a RECOMPUTATION and re-applies the
+saved statistics without touching the running ones.  The recomputation uses
+the saved invstd as is, so it reproduces the first forward bit for bit
+(the reference's F.batch_norm call at bn.py:32-34 adds eps a second time).
+"""
+import torch
+
+from .. import _lib
+from .base import OP, InputStorage, OutputStorage, implements
+
+
+def _as_nchw(t, name):
+    _lib.require_gpu_tensor(t, name, torch.float32)
+    if t.dim() < 2:
+        raise RuntimeError("batch_norm expects at least a 2-D input")
+    tc = t if t.is_contiguous() else t.contiguous()
+    N, C = tc.shape[0], tc.shape[1]
+    HW = tc.numel() // (N * C) if N * C else 0
+    return tc, N, C, HW
+
+
+def _workspace(N, C, HW, device):
+    nbytes = _lib.load().mn_bn_ws_bytes(N, C, HW)
+    return torch.empty(max(nbytes, 4), dtype=torch.uint8, device=device), nbytes
+
+
+def bn_forward_train(x, weight, bias, running_mean, running_var, momentum, eps, out=None):
+    """Training forward -> (y, save_mean, save_invstd)."""
+    xc, N, C, HW = _as_nchw(x, "input")
+    y = torch.empty_like(xc) if out is None else out
+    save_mean = torch.empty(C, dtype=torch.float32, device=x.device)
+    save_invstd = torch.empty(C, dtype=torch.float32, device=x.device)
+    ws, nbytes = _workspace(N, C, HW, x.device)
+    _lib.call("mn_bn_fwd_train_f32", _lib.ptr(xc), _lib.ptr(weight), _lib.ptr(bias),
+              _lib.ptr(running_mean), _lib.ptr(running_var), _lib.ptr(y), _lib.ptr(save_mean),
+              _lib.ptr(save_invstd), N, C, HW, float(momentum), float(eps), _lib.ptr(ws), nbytes,
+              _lib.stream_ptr(x.device))
+    return y, save_mean, save_invstd
+
+
+def bn_forward_apply(x, mean, invstd, weight, bias):
+    """y = (x - mean) * invstd * weight + bias with given per-channel vectors."""
+    xc, N, C, HW = _as_nchw(x, "input")
+    y = torch.empty_like(xc)
+    _lib.call("mn_bn_fwd_apply_f32", _lib.ptr(xc), _lib.ptr(mean), _lib.ptr(invstd),
+              _lib.ptr(weight), _lib.ptr(bias), _lib.ptr(y), N, C, HW, _lib.stream_ptr(x.device))
+    return y
+
+
+def _bn_backward(entry, grad, t, weight, shift, invstd):
+    tc, N, C, HW = _as_nchw(t, "stored activation")
+    g = grad if grad.is_contiguous() else grad.contiguous()
+    _lib.require_gpu_tensor(g, "grad_output", torch.float32)
+    if g.shape != tc.shape:
+        raise RuntimeError("grad_output and the stored activation differ in shape")
+    dx = torch.empty_like(tc)
+    dw = torch.empty(C, dtype=torch.float32, device=t.device)
+    db = torch.empty(C, dtype=torch.float32, device=t.device)
+    ws, nbytes = _workspace(N, C, HW, t.device)
+    _lib.call(entry, _lib.ptr(g), _lib.ptr(tc), _lib.ptr(weight), _lib.ptr(shift),
+              _lib.ptr(invstd), _lib.ptr(dx), _lib.ptr(dw), _lib.ptr(db), N, C, HW, _lib.ptr(ws),
+              nbytes, _lib.stream_ptr(t.device))
+    return dx, dw, db
+
+
+def bn_backward_from_input(grad, x, weight, save_mean, save_invstd):
+    return _bn_backward("mn_bn_bwd_from_x_f32", grad, x, weight, save_mean, save_invstd)
+
+
+def bn_backward_from_output(grad, y, weight, bias, save_invstd):
+    return _bn_backward("mn_bn_bwd_from_y_f32", grad, y, weight, bias, save_invstd)
+
+
+class _BatchNormForward(OP):
+    params = None   # (training, eps, save_mean, save_invstd, reserve)
+    running_mean = None
+    running_var = None
+
+    def forward(self, input_, weight, bias, running_mean, running_var,
+                training=False, momentum=0.1, eps=1e-5, *args, **kwargs):
+        with torch.no_grad():
+            if self.running_mean is None and running_mean is not None:
+                self.running_mean = running_mean.requires_grad_(False)
+                self.running_var = running_var.requires_grad_(False)
+            if self.params is None:
+                if training:
+                    out, save_mean, save_invstd = bn_forward_train(
+                        input_, weight, bias, self.running_mean, self.running_var, momentum, eps)
+                else:
+                    # inference statistics: normalise with the running ones
+                    save_mean = self.running_mean
+                    save_invstd = torch.rsqrt(self.running_var + eps)
+                    out = bn_forward_apply(input_, save_mean, save_invstd, weight, bias)
+                self.params = bool(training), eps, save_mean, save_invstd, None
+            else:
+                _, _, save_mean, save_invstd, _ = self.params
+                out = bn_forward_apply(input_, save_mean, save_invstd, weight, bias)
+            return out
+
+
+@implements(['aten::batch_norm'],
+            ['normal', 'multiway', 'newnode', 'multiway_newnode', 'conv_multiway_newnode',
+             'conv_normal'])
+class InputActBatchNorm(_BatchNormForward):
+    backward_storage = InputStorage(0, 1, 2, 3, 4)
+
+    def backward(self, grad_output, stored, nodel=False):
+        with torch.no_grad():
+            input_, weight, bias, running_mean, running_var = stored
+            training, eps, save_mean, save_invstd, _ = self.params
+            if not training:
+                raise NotImplementedError
+            di, dw, db = bn_backward_from_input(grad_output, input_, weight, save_mean, save_invstd)
+            if not nodel:
+                del stored[4], stored[3], stored[2], stored[1], stored[0]
+            return di, dw, db, None, None
+
+
+@implements(['aten::batch_norm'], ['multiway', 'multiway_newnode', 'conv_multiway_newnode'])
+class OutputActBatchNorm(_BatchNormForward):
+    backward_storage = [InputStorage(1, 2, 3, 4), OutputStorage()]
+
+    def backward(self, grad_output, stored, nodel=False):
+        with torch.no_grad():
+            weight, bias, running_mean, running_var, output = stored
+            training, eps, save_mean, save_invstd, _ = self.params
+            if not training:
+                raise NotImplementedError
+            di, dw, db = bn_backward_from_output(grad_output, output, weight, bias, save_invstd)
+            if not nodel:
+                del stored[4], stored[3], stored[2], stored[1], stored[0]
+            return di, dw, db, None, None

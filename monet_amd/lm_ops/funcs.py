@@ -1,0 +1,56 @@
+"""Residual add and adaptive average pooling (reference:
+monet/lm_ops/funcs.py:7-59).  Bandwidth-bound but stock: they call PyTorch."""
+import torch
+
+from .base import OP, implements
+
+_ALL = ['normal', 'multiway', 'newnode', 'multiway_newnode', 'conv_multiway_newnode', 'conv_normal']
+
+
+@implements(['aten::adaptive_avg_pool2d'], _ALL)
+class AdaptiveAvgPool2D(OP):
+    params = None
+
+    def forward(self, x, output_size):
+        with torch.no_grad():
+            self.params = x.shape, x.device, x.dtype
+            return torch._C._nn.adaptive_avg_pool2d(x, output_size)
+
+    def backward(self, grad_output, stored, nodel=False):
+        assert len(stored) == 0
+        with torch.no_grad():
+            shape, device, dtype = self.params
+            # the aten backward only reads the shape of its second argument
+            like = torch.empty(1, dtype=dtype, device=device).expand(list(shape))
+            return torch.ops.aten._adaptive_avg_pool2d_backward(grad_output.contiguous(), like)
+
+
+class _AddBase(OP):
+    backward_storage = None
+    params = None
+
+    def backward(self, grad_output, stored, nodel=False):
+        assert len(stored) == 0
+        with torch.no_grad():
+            s = self.params
+            return grad_output, (grad_output if s == 1 else grad_output * s)
+
+
+@implements(['aten::add'], _ALL)
+class Add(_AddBase):
+    def forward(self, a, b, s):
+        with torch.no_grad():
+            self.params = s
+            return torch.add(a, b, alpha=s)
+
+
+@implements(['aten::add_'], _ALL)
+class AddIP(_AddBase):
+    inplace = False
+
+    def forward(self, a, b, s):
+        with torch.no_grad():
+            self.params = s
+            if self.inplace:
+                return a.add_(b, alpha=s)
+            return torch.add(a, b, alpha=s)
