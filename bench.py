@@ -166,7 +166,7 @@ def main():
                                "BN bwd from output [184,256,56,56]; ReLU 1-bit-mask bwd "
                                "[184,256,56,56]; maxpool3x3s2 bwd [184,64,56,56]->[184,64,112,112]",
                    "bytes_per_step": BYTES_STEP},
-        "roofline": {"bound": "hbm", "kernel": "bn_bwd_from_output (reduce + apply launches)",
+        "roofline": {"bound": "hbm", "kernel": "bn_bwd_from_output (bn_prepare_kernel + bn_resident_kernel launches)",
                      "achieved": bn["GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": bn["frac"], "traffic": None},
         "kernels": kernels,

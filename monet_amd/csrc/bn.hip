@@ -1,13 +1,32 @@
 // BatchNorm kernels over an [N, C, HW] view (NCHW): training forward, forward
 // from saved statistics, backward from the input and backward from the output.
 //
-// Work decomposition (all kernels): channel c owns N*HW elements, visited as
-// the flat sequence j = n*HWV + i (HWV = HW / VEC vectors per image slab).
-// That sequence is cut into S equal pieces, one workgroup each, so the grid is
-// C*S workgroups whatever the shape; workgroup b handles channel b / S, piece
-// b % S.  Reductions are two-level and atomic-free: every workgroup writes one
-// partial pair to the workspace, and the consumer kernel re-adds the S partials
-// of its channel in a fixed order, so results are reproducible.
+// Work decomposition: channel c owns N*HW elements, visited as the flat
+// sequence j = n*HWV + i (HWV = HW / VEC vectors per image slab).  That
+// sequence is cut into S equal pieces, one workgroup each.  Reductions are
+// two-level and free of floating-point atomics: every workgroup writes one
+// partial pair to the workspace and the S partials of a channel are re-added
+// in a fixed order, so results are reproducible.
+//
+// The statistics-then-apply operators (training forward, both backwards) need
+// every element twice.  Re-reading it costs a second trip through the memory
+// fabric whether or not a cache holds it, so the main formulation keeps it ON
+// CHIP: a piece is sized to fit the registers of one workgroup (kKeep vectors
+// per thread and tensor).  A workgroup loads its piece once, reduces it,
+// publishes the partial, waits until the other workgroups of its channel have
+// published theirs, then computes the result from the registers it still
+// holds.  HBM traffic is the algorithmic minimum: each operand read once, the
+// result written once.
+//
+// Why the wait always ends: workgroups take their work item from a ticket
+// counter when they start, so the items of a channel are held by workgroups
+// that are all running or about to be started in ticket order; the lowest
+// unfinished channel can always complete because at most S <= 256 workgroups
+// are needed at once and the device holds more than that.  A spin bound turns
+// a broken launch into wrong numbers instead of a hang.
+//
+// Channels too large for S <= 256 resident pieces fall back to two launches
+// (reduce, then apply) that read the operands twice.
 #include "common.h"
 
 namespace mn_bn {
@@ -16,6 +35,7 @@ constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / MN_WAVE;
 constexpr int kMaxSplit = 64;
 constexpr int kU = 4;  // vectors in flight per thread per tensor
+
 
 template <int VEC>
 struct Vec;
@@ -37,24 +57,25 @@ struct Shape {
   uint64_t tot;  // vectors per channel = N * HWV
 };
 
-// Walks the vectors of one piece with a stride of kThreads, keeping (n, i)
+// Walks the vectors of one piece with a stride of STRIDE (= workgroup size), keeping (n, i)
 // without a division per step.
-struct Cursor {
+template <int STRIDE>
+struct CursorT {
   uint64_t j, jend;
   uint32_t n, i, qstep, rstep, HWV;
-  __device__ __forceinline__ Cursor(const Shape& sh, int piece) {
+  __device__ __forceinline__ CursorT(const Shape& sh, int piece) {
     HWV = sh.HWV;
     const uint64_t j0 = (uint64_t)piece * sh.L;
     jend = min(j0 + sh.L, sh.tot);
     j = j0 + threadIdx.x;
     n = (uint32_t)(j / HWV);
     i = (uint32_t)(j - (uint64_t)n * HWV);
-    qstep = kThreads / HWV;
-    rstep = kThreads - qstep * HWV;
+    qstep = STRIDE / HWV;
+    rstep = STRIDE - qstep * HWV;
   }
   __device__ __forceinline__ bool valid() const { return j < jend; }
   __device__ __forceinline__ void next() {
-    j += kThreads;
+    j += STRIDE;
     n += qstep;
     i += rstep;
     if (i >= HWV) {
@@ -69,6 +90,8 @@ struct Cursor {
   }
 };
 
+typedef CursorT<kThreads> Cursor;
+
 template <int VEC>
 __device__ __forceinline__ typename Vec<VEC>::type ldv(const float* p) {
   return ld_stream(reinterpret_cast<const typename Vec<VEC>::type*>(p));
@@ -82,26 +105,39 @@ __device__ __forceinline__ float comp(const float& v, int) { return v; }
 __device__ __forceinline__ void setc(float4_t& v, int k, float a) { v[k] = a; }
 __device__ __forceinline__ void setc(float& v, int, float a) { v = a; }
 
+enum Mode { BWD_FROM_X = 0, BWD_FROM_Y = 1, FWD_TRAIN = 2 };
+
+// Everything a statistics-then-apply operator needs.
+//   backward: a = dy, b = x or y, shift = mean or beta, out = dx
+//   forward : b = x, out = y
+struct Args {
+  Shape sh;
+  const float* a;
+  const float* b;
+  const float* gamma;
+  const float* shift;   // backward: mean (from x) / beta (from y); forward: beta
+  const float* invstd;  // backward only
+  float* out;
+  float* vec0;          // backward: dgamma; forward: save_mean
+  float* vec1;          // backward: dbeta;  forward: save_invstd
+  float* running_mean;  // forward only
+  float* running_var;
+  float* partial;       // [C][S][2]
+  float* pivot;         // [C], forward only
+  uint32_t* ticket;     // resident launch only
+  float inv_m, unbias, momentum, eps;
+};
+
 // ---------------------------------------------------------------- reduce --
-// partial[c][piece] = ( sum a , sum a*(b - shift[c]) )       (backward)
-//                  or ( sum (b - K) , sum (b - K)^2 )         (STATS: forward)
-// with K = first element of the channel (also stored in pivot[c]).
-template <int VEC, bool STATS>
-__global__ __launch_bounds__(kThreads) void bn_reduce_kernel(const Shape sh, const float* a,
-                                                             const float* b, const float* shift,
-                                                             float* partial, float* pivot) {
-  __shared__ float lds[2 * kWaves];
+// (s0, s1) = ( sum a , sum a*(b - shift) )   backward
+//          = ( sum (b - K) , sum (b - K)^2 ) forward, K = first element of the channel
+template <int VEC, int MODE>
+__device__ __forceinline__ void reduce_piece(const Args& A, int c, int piece, float sft, float& s0,
+                                             float& s1) {
   typedef typename Vec<VEC>::type V;
-  const int c = blockIdx.x / sh.S;
-  const int piece = blockIdx.x - c * sh.S;
-  float sft;
-  if (STATS) {
-    sft = b[(size_t)c * sh.HW];
-    if (piece == 0 && threadIdx.x == 0) pivot[c] = sft;
-  } else {
-    sft = shift ? shift[c] : 0.f;
-  }
-  float s0 = 0.f, s1 = 0.f;
+  const Shape& sh = A.sh;
+  s0 = 0.f;
+  s1 = 0.f;
   Cursor cur(sh, piece);
   while (cur.valid()) {
     V va[kU], vb[kU];
@@ -111,8 +147,8 @@ __global__ __launch_bounds__(kThreads) void bn_reduce_kernel(const Shape sh, con
       ok[u] = cur.valid();
       if (ok[u]) {
         const size_t o = cur.off<VEC>(sh.C, c, sh.HW);
-        vb[u] = ldv<VEC>(b + o);
-        if (!STATS) va[u] = ldv<VEC>(a + o);
+        vb[u] = ldv<VEC>(A.b + o);
+        if (MODE != FWD_TRAIN) va[u] = ldv<VEC>(A.a + o);
       }
       cur.next();
     }
@@ -122,7 +158,7 @@ __global__ __launch_bounds__(kThreads) void bn_reduce_kernel(const Shape sh, con
 #pragma unroll
         for (int k = 0; k < VEC; ++k) {
           const float d = comp(vb[u], k) - sft;
-          if (STATS) {
+          if (MODE == FWD_TRAIN) {
             s0 += d;
             s1 += d * d;
           } else {
@@ -134,207 +170,489 @@ __global__ __launch_bounds__(kThreads) void bn_reduce_kernel(const Shape sh, con
       }
     }
   }
-  block_sum2<kWaves>(s0, s1, lds);
-  if (threadIdx.x == 0) {
-    partial[2 * (size_t)blockIdx.x] = s0;
-    partial[2 * (size_t)blockIdx.x + 1] = s1;
+}
+
+template <int MODE>
+__device__ __forceinline__ float reduce_shift(const Args& A, int c) {
+  if (MODE == FWD_TRAIN) return A.b[(size_t)c * A.sh.HW];
+  return A.shift ? A.shift[c] : 0.f;
+}
+
+// ----------------------------------------------------------------- apply --
+// out = (a - (b - sft)*proj - gmean) * gscale     backward
+// out = (b - mean) * scale + bias                 forward (proj = mean, gmean = bias, gscale = scale)
+template <int VEC, int MODE>
+__device__ __forceinline__ void apply_piece(const Args& A, int c, int piece, float sft, float proj,
+                                            float gmean, float gscale) {
+  typedef typename Vec<VEC>::type V;
+  const Shape& sh = A.sh;
+  Cursor cur(sh, piece);
+  while (cur.valid()) {
+    V va[kU], vb[kU];
+    size_t o[kU];
+    bool ok[kU];
+#pragma unroll
+    for (int u = 0; u < kU; ++u) {
+      ok[u] = cur.valid();
+      if (ok[u]) {
+        o[u] = cur.off<VEC>(sh.C, c, sh.HW);
+        vb[u] = ldv<VEC>(A.b + o[u]);
+        if (MODE != FWD_TRAIN) va[u] = ldv<VEC>(A.a + o[u]);
+      }
+      cur.next();
+    }
+#pragma unroll
+    for (int u = 0; u < kU; ++u) {
+      if (ok[u]) {
+        V r;
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+          if (MODE == FWD_TRAIN)
+            setc(r, k, (comp(vb[u], k) - proj) * gscale + gmean);
+          else
+            setc(r, k, (comp(va[u], k) - (comp(vb[u], k) - sft) * proj - gmean) * gscale);
+        }
+        stv<VEC>(A.out + o[u], r);
+      }
+    }
   }
 }
 
-// Re-add the S partial pairs of channel c; every thread gets the totals.
+// Turn the channel totals into the apply coefficients; piece 0 also writes
+// the per-channel outputs.
+template <int MODE>
+__device__ __forceinline__ void coefficients(const Args& A, int c, int piece, float t0, float t1,
+                                             float pivot, float& sft, float& proj, float& gmean,
+                                             float& gscale) {
+  const float w = A.gamma ? A.gamma[c] : 1.f;
+  const bool writer = piece == 0 && threadIdx.x == 0;
+  if (MODE == FWD_TRAIN) {
+    const float dm = t0 * A.inv_m;
+    const float mean = pivot + dm;
+    const float var = fmaxf(t1 * A.inv_m - dm * dm, 0.f);
+    const float istd = 1.f / sqrtf(var + A.eps);
+    if (writer) {
+      A.vec0[c] = mean;
+      A.vec1[c] = istd;
+      if (A.running_mean)
+        A.running_mean[c] = (1.f - A.momentum) * A.running_mean[c] + A.momentum * mean;
+      if (A.running_var)
+        A.running_var[c] = (1.f - A.momentum) * A.running_var[c] + A.momentum * (var * A.unbias);
+    }
+    sft = 0.f;
+    proj = mean;
+    gscale = istd * w;
+    gmean = A.shift ? A.shift[c] : 0.f;
+  } else {
+    sft = A.shift ? A.shift[c] : 0.f;
+    const float istd = A.invstd[c];
+    float dg;
+    if (MODE == BWD_FROM_Y) {
+      const float inv_w = 1.f / w;
+      proj = t1 * A.inv_m * inv_w * inv_w;
+      dg = t1 * inv_w;
+    } else {
+      proj = t1 * A.inv_m * istd * istd;
+      dg = t1 * istd;
+    }
+    gmean = t0 * A.inv_m;
+    gscale = istd * w;
+    if (writer) {
+      if (A.vec0) A.vec0[c] = dg;
+      if (A.vec1) A.vec1[c] = t0;
+    }
+  }
+}
+
+// Re-add the S (<= 64) partial pairs of channel c in a fixed order; every
+// thread gets the totals.  COHERENT: read past the caches of this XCD, for
+// partials written by other workgroups of the same launch.
+template <bool COHERENT>
 __device__ __forceinline__ void channel_totals(const float* partial, int c, int S, float& t0,
                                                float& t1) {
-  // S <= 64: lane l of each wave fetches partial l, then a fixed-order lane tree
   const int lane = threadIdx.x % MN_WAVE;
   float p0 = 0.f, p1 = 0.f;
   if (lane < S) {
-    p0 = partial[2 * ((size_t)c * S + lane)];
-    p1 = partial[2 * ((size_t)c * S + lane) + 1];
+    const float* p = partial + 2 * ((size_t)c * S + lane);
+    if (COHERENT) {
+      p0 = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      p1 = __hip_atomic_load(p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else {
+      p0 = p[0];
+      p1 = p[1];
+    }
   }
   t0 = wave_sum(p0);
   t1 = wave_sum(p1);
 }
 
-// ------------------------------------------------------------ bwd: apply --
-// dx = (dy - (t - shift)*proj - gmean) * gscale, coefficients per channel.
-// FROM_Y: t = y, shift = beta, proj = dot/(M*gamma^2); dgamma = dot/gamma
-// else  : t = x, shift = mean, proj = dot*invstd^2/M;  dgamma = dot*invstd
-template <int VEC, bool FROM_Y>
-__global__ __launch_bounds__(kThreads) void bn_bwd_apply_kernel(
-    const Shape sh, const float* dy, const float* t, const float* gamma, const float* shift,
-    const float* invstd, const float* partial, float* dx, float* dgamma, float* dbeta,
-    float inv_m) {
-  typedef typename Vec<VEC>::type V;
-  const int c = blockIdx.x / sh.S;
-  const int piece = blockIdx.x - c * sh.S;
-  float gsum, dot;
-  channel_totals(partial, c, sh.S, gsum, dot);
-  const float w = gamma ? gamma[c] : 1.f;
-  const float sft = shift ? shift[c] : 0.f;
-  const float istd = invstd[c];
-  float proj, dg;
-  if (FROM_Y) {
-    const float inv_w = 1.f / w;
-    proj = dot * inv_m * inv_w * inv_w;
-    dg = dot * inv_w;
-  } else {
-    proj = dot * inv_m * istd * istd;
-    dg = dot * istd;
-  }
-  const float gmean = gsum * inv_m;
-  const float gscale = istd * w;
-  if (piece == 0 && threadIdx.x == 0) {
-    if (dgamma) dgamma[c] = dg;
-    if (dbeta) dbeta[c] = gsum;
-  }
-  if (!dx) return;
-  Cursor cur(sh, piece);
-  while (cur.valid()) {
-    V vg[kU], vt[kU];
-    size_t o[kU];
-    bool ok[kU];
-#pragma unroll
-    for (int u = 0; u < kU; ++u) {
-      ok[u] = cur.valid();
-      if (ok[u]) {
-        o[u] = cur.off<VEC>(sh.C, c, sh.HW);
-        vg[u] = ldv<VEC>(dy + o[u]);
-        vt[u] = ldv<VEC>(t + o[u]);
-      }
-      cur.next();
-    }
-#pragma unroll
-    for (int u = 0; u < kU; ++u) {
-      if (ok[u]) {
-        V r;
-#pragma unroll
-        for (int k = 0; k < VEC; ++k)
-          setc(r, k, (comp(vg[u], k) - (comp(vt[u], k) - sft) * proj - gmean) * gscale);
-        stv<VEC>(dx + o[u], r);
-      }
-    }
+// ------------------------------------------------- two-launch formulation --
+template <int VEC, int MODE>
+__global__ __launch_bounds__(kThreads) void bn_reduce_kernel(const Args A) {
+  __shared__ float lds[2 * kWaves];
+  const int c = blockIdx.x / A.sh.S;
+  const int piece = blockIdx.x - c * A.sh.S;
+  const float sft = reduce_shift<MODE>(A, c);
+  if (MODE == FWD_TRAIN && piece == 0 && threadIdx.x == 0) A.pivot[c] = sft;
+  float s0, s1;
+  reduce_piece<VEC, MODE>(A, c, piece, sft, s0, s1);
+  block_sum2<kWaves>(s0, s1, lds);
+  if (threadIdx.x == 0) {
+    A.partial[2 * (size_t)blockIdx.x] = s0;
+    A.partial[2 * (size_t)blockIdx.x + 1] = s1;
   }
 }
 
-// ------------------------------------------------------------ fwd: apply --
-// y = (x - mean) * (invstd*gamma) + beta.  FINALIZE: mean / invstd come from
-// the partial sums of bn_reduce_kernel<STATS> and piece 0 also writes
-// save_mean, save_invstd and the running statistics.
-template <int VEC, bool FINALIZE>
-__global__ __launch_bounds__(kThreads) void bn_fwd_apply_kernel(
-    const Shape sh, const float* x, const float* mean_in, const float* invstd_in,
-    const float* gamma, const float* beta, const float* partial, const float* pivot, float* y,
-    float* save_mean, float* save_invstd, float* running_mean, float* running_var, float inv_m,
-    float unbias, float momentum, float eps) {
-  typedef typename Vec<VEC>::type V;
-  const int c = blockIdx.x / sh.S;
-  const int piece = blockIdx.x - c * sh.S;
-  float mean, istd;
-  if (FINALIZE) {
-    float s1, s2;
-    channel_totals(partial, c, sh.S, s1, s2);
-    const float dm = s1 * inv_m;
-    mean = pivot[c] + dm;
-    const float var = fmaxf(s2 * inv_m - dm * dm, 0.f);
-    istd = 1.f / sqrtf(var + eps);
-    if (piece == 0 && threadIdx.x == 0) {
-      save_mean[c] = mean;
-      save_invstd[c] = istd;
-      if (running_mean) running_mean[c] = (1.f - momentum) * running_mean[c] + momentum * mean;
-      if (running_var)
-        running_var[c] = (1.f - momentum) * running_var[c] + momentum * (var * unbias);
+template <int VEC, int MODE>
+__global__ __launch_bounds__(kThreads) void bn_apply_kernel(const Args A) {
+  const int c = blockIdx.x / A.sh.S;
+  const int piece = blockIdx.x - c * A.sh.S;
+  float t0, t1, sft, proj, gmean, gscale;
+  channel_totals<false>(A.partial, c, A.sh.S, t0, t1);
+  coefficients<MODE>(A, c, piece, t0, t1, MODE == FWD_TRAIN ? A.pivot[c] : 0.f, sft, proj, gmean,
+                     gscale);
+  if (!A.out) return;
+  apply_piece<VEC, MODE>(A, c, piece, sft, proj, gmean, gscale);
+}
+
+// Forward from saved statistics (no reduction).
+template <int VEC>
+__global__ __launch_bounds__(kThreads) void bn_fwd_saved_kernel(const Args A, const float* mean,
+                                                                const float* invstd) {
+  const int c = blockIdx.x / A.sh.S;
+  const int piece = blockIdx.x - c * A.sh.S;
+  const float scale = invstd[c] * (A.gamma ? A.gamma[c] : 1.f);
+  const float bias = A.shift ? A.shift[c] : 0.f;
+  apply_piece<VEC, FWD_TRAIN>(A, c, piece, 0.f, mean[c], bias, scale);
+}
+
+// ------------------------------------------------- one-launch formulation --
+// A published partial pair is ONE 64-bit word (low = s0, high = s1) written
+// and read with relaxed device-scope atomics, so the word itself is the
+// "ready" flag and no cache flush / invalidate is ever needed.  Unpublished
+// slots hold kEmptySlot, which publish() never writes.
+constexpr uint64_t kEmptySlot = 0xFFFFFFFFFFFFFFFFull;
+
+__global__ void bn_prepare_kernel(uint64_t* slots, uint32_t nslots, uint32_t* ticket) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < nslots) slots[i] = kEmptySlot;
+  if (i == 0) *ticket = 0u;
+}
+
+__device__ __forceinline__ void publish(uint64_t* slot, float s0, float s1) {
+  uint64_t w = (uint64_t)__float_as_uint(s0) | ((uint64_t)__float_as_uint(s1) << 32);
+  if (w == kEmptySlot) w = 0x7FC000007FC00000ull;  // same meaning (NaN, NaN), different bits
+  __hip_atomic_store(slot, w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+constexpr int kMaxResident = 256;  // most pieces per channel in the resident formulation
+
+// Wave 0 polls the S slots of a channel until all are published, adds them in
+// a fixed order (lane l takes slots l, l+64, ..; then a lane tree) and hands
+// the totals to the workgroup through `lds`.
+__device__ __forceinline__ void gather_totals(const uint64_t* slots, int S, float* lds, float& t0,
+                                              float& t1) {
+  if (threadIdx.x < MN_WAVE) {
+    const int lane = threadIdx.x;
+    float p0 = 0.f, p1 = 0.f;
+    for (int k = lane; k < S; k += MN_WAVE) {  // at most kMaxResident / 64 rounds
+      uint64_t w;
+      uint32_t spins = 0;
+      // The pieces polled here are published or held by running workgroups that publish
+      // before they wait, so this ends; the bound only keeps a broken launch from hanging
+      // the device (the results are then wrong).
+      while ((w = __hip_atomic_load(slots + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) ==
+                 kEmptySlot &&
+             ++spins < (1u << 22))
+        __builtin_amdgcn_s_sleep(1);
+      p0 += __uint_as_float((uint32_t)w);
+      p1 += __uint_as_float((uint32_t)(w >> 32));
     }
-  } else {
-    mean = mean_in[c];
-    istd = invstd_in[c];
+    p0 = wave_sum(p0);
+    p1 = wave_sum(p1);
+    if (lane == 0) {
+      lds[0] = p0;
+      lds[1] = p1;
+    }
   }
-  const float scale = istd * (gamma ? gamma[c] : 1.f);
-  const float bias = beta ? beta[c] : 0.f;
-  Cursor cur(sh, piece);
-  while (cur.valid()) {
-    V vx[kU];
-    size_t o[kU];
-    bool ok[kU];
+  __syncthreads();
+  t0 = lds[0];
+  t1 = lds[1];
+}
+
+// One piece held in registers: thread t owns vectors p*L + t + k*THREADS, k < KEEP
+// (sh.L must be THREADS * KEEP).
+template <int VEC, int KEEP>
+struct Held {
+  typename Vec<VEC>::type a[KEEP], b[KEEP];
+  int c, piece;
+  float sft;
+};
+
+// Load a piece, reduce it and publish its partial pair.  Never waits for
+// another workgroup.
+template <int VEC, int MODE, int KEEP, int THREADS>
+__device__ __forceinline__ void hold_piece(const Args& A, uint32_t item, Held<VEC, KEEP>& h,
+                                           float* lds) {
+  typedef CursorT<THREADS> Cursor;
+  const Shape& sh = A.sh;
+  const int S = sh.S;
+  h.c = item / S;
+  h.piece = item - h.c * S;
+  h.sft = reduce_shift<MODE>(A, h.c);  // forward: the pivot, read before any store to the channel
+  {
+    Cursor cur(sh, h.piece);
 #pragma unroll
-    for (int u = 0; u < kU; ++u) {
-      ok[u] = cur.valid();
-      if (ok[u]) {
-        o[u] = cur.off<VEC>(sh.C, c, sh.HW);
-        vx[u] = ldv<VEC>(x + o[u]);
+    for (int k = 0; k < KEEP; ++k) {
+      if (cur.valid()) {
+        const size_t o = cur.template off<VEC>(sh.C, h.c, sh.HW);
+        h.b[k] = ldv<VEC>(A.b + o);
+        if (MODE != FWD_TRAIN) h.a[k] = ldv<VEC>(A.a + o);
       }
       cur.next();
     }
+  }
+  float s0 = 0.f, s1 = 0.f;
+  {
+    Cursor cur(sh, h.piece);
 #pragma unroll
-    for (int u = 0; u < kU; ++u) {
-      if (ok[u]) {
-        V r;
+    for (int k = 0; k < KEEP; ++k) {
+      if (cur.valid()) {
 #pragma unroll
-        for (int k = 0; k < VEC; ++k) setc(r, k, (comp(vx[u], k) - mean) * scale + bias);
-        stv<VEC>(y + o[u], r);
+        for (int e = 0; e < VEC; ++e) {
+          const float d = comp(h.b[k], e) - h.sft;
+          if (MODE == FWD_TRAIN) {
+            s0 += d;
+            s1 += d * d;
+          } else {
+            const float g = comp(h.a[k], e);
+            s0 += g;
+            s1 += g * d;
+          }
+        }
       }
+      cur.next();
     }
+  }
+  block_sum2<THREADS / MN_WAVE>(s0, s1, lds);
+  if (threadIdx.x == 0)
+    publish(reinterpret_cast<uint64_t*>(A.partial) + (size_t)h.c * S + h.piece, s0, s1);
+}
+
+// Wait for the channel totals of a held piece and write its result.
+template <int VEC, int MODE, int KEEP, int THREADS>
+__device__ __forceinline__ void finish_piece(const Args& A, const Held<VEC, KEEP>& h, float* lds) {
+  typedef typename Vec<VEC>::type V;
+  typedef CursorT<THREADS> Cursor;
+  const Shape& sh = A.sh;
+  float t0, t1;
+  __syncthreads();  // lds is free again
+  gather_totals(reinterpret_cast<uint64_t*>(A.partial) + (size_t)h.c * sh.S, sh.S, lds, t0, t1);
+  float s_, proj, gmean, gscale;
+  coefficients<MODE>(A, h.c, h.piece, t0, t1, h.sft, s_, proj, gmean, gscale);
+  if (!A.out) return;
+  Cursor cur(sh, h.piece);
+#pragma unroll
+  for (int k = 0; k < KEEP; ++k) {
+    if (cur.valid()) {
+      V r;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        if (MODE == FWD_TRAIN)
+          setc(r, e, (comp(h.b[k], e) - proj) * gscale + gmean);
+        else
+          setc(r, e, (comp(h.a[k], e) - (comp(h.b[k], e) - s_) * proj - gmean) * gscale);
+      }
+      stv<VEC>(A.out + cur.template off<VEC>(sh.C, h.c, sh.HW), r);
+    }
+    cur.next();
+  }
+}
+
+// Persistent workgroups: each keeps two pieces in flight, so the wait for the
+// other workgroups of one piece's channel is spent loading the next piece.
+// Every piece is published before its holder waits for anything, and pieces
+// are handed out in ticket order, so the lowest unfinished channel always has
+// all its pieces either published or about to be taken by a running workgroup
+// (at least kMaxResident workgroups run at once).
+template <int VEC, int MODE, int KEEP, int THREADS>
+__global__ __launch_bounds__(THREADS) void bn_resident_kernel(const Args A, uint32_t items) {
+  __shared__ float lds[2 * (THREADS / MN_WAVE)];
+  __shared__ uint32_t s_ticket;
+  Held<VEC, KEEP> h0, h1;
+  auto take = [&]() -> uint32_t {
+    __syncthreads();  // s_ticket of the previous round has been read by everyone
+    if (threadIdx.x == 0)
+      s_ticket = __hip_atomic_fetch_add(A.ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    return s_ticket;
+  };
+  uint32_t i0 = take();
+  if (i0 >= items) return;
+  hold_piece<VEC, MODE, KEEP, THREADS>(A, i0, h0, lds);
+  for (;;) {
+    const uint32_t i1 = take();
+    if (i1 < items) hold_piece<VEC, MODE, KEEP, THREADS>(A, i1, h1, lds);
+    finish_piece<VEC, MODE, KEEP, THREADS>(A, h0, lds);
+    if (i1 >= items) break;
+    i0 = take();
+    if (i0 < items) hold_piece<VEC, MODE, KEEP, THREADS>(A, i0, h0, lds);
+    finish_piece<VEC, MODE, KEEP, THREADS>(A, h1, lds);
+    if (i0 >= items) break;
   }
 }
 
 // ------------------------------------------------------------------ host --
-struct Plan {
-  Shape sh;
-  int vec;
-  unsigned blocks;
+// Launch choices.  `resident`: 1 = one launch keeping the operands in
+// registers (falls back when a channel needs more than kMaxResident pieces),
+// 0 = always reduce launch + apply launch.
+struct Tuning {
+  int target_blocks = 2048;  // two-launch formulation: aim for C*S workgroups
+  int resident = 1;
+  int keep = 8;              // vectors kept per thread, tensor and piece (two pieces in flight)
+  int threads = 256;         // workgroup size of the resident kernel
+  int grid = 768;            // persistent workgroups of the resident kernel (3 per CU)
 };
 
-// `target_blocks`: aim of the split, ~16 workgroups per CU on 256 CUs.
-static bool make_plan(int64_t N, int64_t C, int64_t HW, bool aligned16, int target_blocks,
-                      Plan& p) {
-  if (N <= 0 || C <= 0 || HW <= 0) return false;
-  if (C > (1 << 24) || HW >= (1ll << 31) || N >= (1ll << 31)) return false;
-  p.vec = (HW % 4 == 0 && aligned16) ? 4 : 1;
-  const uint64_t hwv = (uint64_t)HW / p.vec;
-  const uint64_t tot = (uint64_t)N * hwv;
-  int64_t S = (target_blocks + C - 1) / C;
-  const int64_t cap = (int64_t)((tot + kThreads * kU - 1) / (kThreads * kU));  // >= 1 batch each
+static bool shape_limits(int64_t N, int64_t C, int64_t HW) {
+  return N > 0 && C > 0 && HW > 0 && C <= (1 << 22) && HW < (1ll << 31) && N < (1ll << 31);
+}
+static int64_t resident_pieces(int64_t N, int64_t HW, int vec, int keep) {
+  const int64_t tot = N * (HW / vec);
+  return (tot + kThreads * keep - 1) / (kThreads * keep);
+}
+// Vectors per resident piece in product builds: (keep 8 x 256 threads) float4, or
+// (keep 16 x 256 threads) scalars when the shape / alignment rules out float4.
+static int64_t product_pieces(int64_t N, int64_t HW, int vec) {
+  return resident_pieces(N, HW, vec, vec == 4 ? 8 : 16);
+}
+// Workspace: partial pairs [C][P][2] floats, pivot [C] floats, ticket word; P covers both the
+// resident formulation (if the channel qualifies) and the two-launch one.
+static size_t ws_floats(int64_t N, int64_t C, int64_t HW) {
+  int64_t P = kMaxSplit;
+  const int64_t p1 = product_pieces(N, HW, 1);
+  if (p1 <= kMaxResident && p1 > P) P = p1;
+  if (HW % 4 == 0) {
+    const int64_t p4 = product_pieces(N, HW, 4);
+    if (p4 <= kMaxResident && p4 > P) P = p4;
+  }
+  return (size_t)C * (2 * (size_t)P + 1);
+}
+static size_t ws_bytes_for(int64_t N, int64_t C, int64_t HW) {
+  return ws_floats(N, C, HW) * sizeof(float) + 2 * sizeof(uint32_t);
+}
+
+static void fill_shape(int64_t N, int64_t C, int64_t HW, int vec, int64_t S, uint64_t L,
+                       Shape& sh) {
+  sh.C = (int)C;
+  sh.S = (int)S;
+  sh.HWV = (uint32_t)(HW / vec);
+  sh.HW = (uint32_t)HW;
+  sh.tot = (uint64_t)N * sh.HWV;
+  sh.L = L;
+}
+
+template <int MODE>
+static int run(Args& A, int64_t N, int64_t C, int64_t HW, bool aligned16, void* ws,
+               const Tuning& t, hipStream_t s) {
+  const int vec = (HW % 4 == 0 && aligned16) ? 4 : 1;
+  A.partial = static_cast<float*>(ws);
+  uint32_t* counters = reinterpret_cast<uint32_t*>(A.partial + ws_floats(N, C, HW));
+  A.pivot = reinterpret_cast<float*>(counters) - C;  // last C floats of the float area
+  A.ticket = counters;
+  const int keep = t.keep > 0 ? t.keep : 8, threads = t.threads > 0 ? t.threads : kThreads;
+  const int64_t rp = resident_pieces(N, HW, vec, (vec == 4 ? keep * threads : 16 * kThreads) / kThreads);
+  if (t.resident && rp <= kMaxResident) {
+    fill_shape(N, C, HW, vec, rp, vec == 4 ? (uint64_t)threads * keep : (uint64_t)kThreads * 16, A.sh);
+    const unsigned blocks = (unsigned)(C * rp);
+    bn_prepare_kernel<<<(blocks + 255) / 256, 256, 0, s>>>(
+          reinterpret_cast<uint64_t*>(A.partial), blocks, A.ticket);
+    // persistent grid: enough workgroups to fill 256 CUs at this register footprint
+    const unsigned grid = blocks < (unsigned)t.grid ? blocks : (unsigned)t.grid;
+#define MN_BN_RES(V, K, T) bn_resident_kernel<V, MODE, K, T><<<grid, T, 0, s>>>(A, blocks)
+    if (vec == 4) {
+#ifdef MN_TUNING
+      if (keep == 8 && threads == 256) MN_BN_RES(4, 8, 256);
+      else if (keep == 4 && threads == 512) MN_BN_RES(4, 4, 512);
+      else if (keep == 8 && threads == 512) MN_BN_RES(4, 8, 512);
+      else if (keep == 4 && threads == 1024) MN_BN_RES(4, 4, 1024);
+      else if (keep == 16 && threads == 256) MN_BN_RES(4, 16, 256);
+      else if (keep == 12 && threads == 256) MN_BN_RES(4, 12, 256);
+      else
+#endif
+      MN_BN_RES(4, 8, 256);
+    } else {
+      MN_BN_RES(1, 16, 256);
+    }
+#undef MN_BN_RES
+    return mn_launch_status();
+  }
+  const uint64_t tot = (uint64_t)N * (HW / vec);
+  int64_t S = (t.target_blocks + C - 1) / C;
+  const int64_t cap = (int64_t)((tot + kThreads * kU - 1) / (kThreads * kU));
   if (S > cap) S = cap;
   if (S > kMaxSplit) S = kMaxSplit;
   if (S < 1) S = 1;
-  p.sh.C = (int)C;
-  p.sh.S = (int)S;
-  p.sh.HWV = (uint32_t)hwv;
-  p.sh.HW = (uint32_t)HW;
-  p.sh.tot = tot;
-  p.sh.L = (tot + S - 1) / S;
-  p.blocks = (unsigned)(C * S);
-  return true;
+  fill_shape(N, C, HW, vec, S, (tot + S - 1) / S, A.sh);
+  const unsigned blocks = (unsigned)(C * S);
+  if (vec == 4) {
+    bn_reduce_kernel<4, MODE><<<blocks, kThreads, 0, s>>>(A);
+    bn_apply_kernel<4, MODE><<<blocks, kThreads, 0, s>>>(A);
+  } else {
+    bn_reduce_kernel<1, MODE><<<blocks, kThreads, 0, s>>>(A);
+    bn_apply_kernel<1, MODE><<<blocks, kThreads, 0, s>>>(A);
+  }
+  return mn_launch_status();
 }
-
-constexpr int kTargetBlocks = 4096;
-
-static size_t ws_bytes_for(int64_t C) { return (size_t)C * (2 * kMaxSplit + 1) * sizeof(float); }
 
 int bwd_launch(bool from_y, const float* dy, const float* t, const float* gamma, const float* shift,
                const float* invstd, float* dx, float* dgamma, float* dbeta, int64_t N, int64_t C,
-               int64_t HW, void* ws, size_t ws_bytes, hipStream_t s, int target_blocks) {
+               int64_t HW, void* ws, size_t ws_bytes, hipStream_t s, const Tuning& tune) {
+  if (N < 0 || C < 0 || HW < 0) return MN_EINVAL;
   if (N == 0 || C == 0 || HW == 0) return MN_OK;
   if (!dy || !t || !invstd || !ws) return MN_EINVAL;
-  if (ws_bytes < ws_bytes_for(C) || !mn_aligned(ws, 4)) return MN_EINVAL;
-  Plan p;
+  if (!shape_limits(N, C, HW)) return MN_EUNSUPPORTED;
+  if (ws_bytes < ws_bytes_for(N, C, HW) || !mn_aligned(ws, 8)) return MN_EINVAL;
+  Args A = {};
   const bool al = mn_aligned(dy, 16) && mn_aligned(t, 16) && (!dx || mn_aligned(dx, 16));
-  if (!make_plan(N, C, HW, al, target_blocks, p)) return MN_EUNSUPPORTED;
-  float* partial = static_cast<float*>(ws);
-  const float inv_m = 1.f / (float)((double)N * (double)HW);
-  if (p.vec == 4)
-    bn_reduce_kernel<4, false><<<p.blocks, kThreads, 0, s>>>(p.sh, dy, t, shift, partial, nullptr);
-  else
-    bn_reduce_kernel<1, false><<<p.blocks, kThreads, 0, s>>>(p.sh, dy, t, shift, partial, nullptr);
-#define MN_BN_APPLY(V, FY)                                                                      \
-  bn_bwd_apply_kernel<V, FY><<<p.blocks, kThreads, 0, s>>>(p.sh, dy, t, gamma, shift, invstd,   \
-                                                           partial, dx, dgamma, dbeta, inv_m)
-  if (p.vec == 4) {
-    if (from_y) MN_BN_APPLY(4, true); else MN_BN_APPLY(4, false);
-  } else {
-    if (from_y) MN_BN_APPLY(1, true); else MN_BN_APPLY(1, false);
-  }
-#undef MN_BN_APPLY
-  return mn_launch_status();
+  A.a = dy;
+  A.b = t;
+  A.gamma = gamma;
+  A.shift = shift;
+  A.invstd = invstd;
+  A.out = dx;
+  A.vec0 = dgamma;
+  A.vec1 = dbeta;
+  A.inv_m = 1.f / (float)((double)N * (double)HW);
+  return from_y ? run<BWD_FROM_Y>(A, N, C, HW, al, ws, tune, s)
+                : run<BWD_FROM_X>(A, N, C, HW, al, ws, tune, s);
+}
+
+int fwd_train_launch(const float* x, const float* gamma, const float* beta, float* running_mean,
+                     float* running_var, float* y, float* save_mean, float* save_invstd, int64_t N,
+                     int64_t C, int64_t HW, double momentum, double eps, void* ws, size_t ws_bytes,
+                     hipStream_t s, const Tuning& tune) {
+  if (N < 0 || C < 0 || HW < 0) return MN_EINVAL;
+  if (N == 0 || C == 0 || HW == 0) return MN_OK;
+  if (!x || !y || !save_mean || !save_invstd || !ws) return MN_EINVAL;
+  if (!shape_limits(N, C, HW)) return MN_EUNSUPPORTED;
+  if (ws_bytes < ws_bytes_for(N, C, HW) || !mn_aligned(ws, 8)) return MN_EINVAL;
+  Args A = {};
+  const bool al = mn_aligned(x, 16) && mn_aligned(y, 16);
+  const double M = (double)N * (double)HW;
+  A.b = x;
+  A.gamma = gamma;
+  A.shift = beta;
+  A.out = y;
+  A.vec0 = save_mean;
+  A.vec1 = save_invstd;
+  A.running_mean = running_mean;
+  A.running_var = running_var;
+  A.inv_m = (float)(1.0 / M);
+  A.unbias = M > 1.0 ? (float)(M / (M - 1.0)) : 1.f;
+  A.momentum = (float)momentum;
+  A.eps = (float)eps;
+  return run<FWD_TRAIN>(A, N, C, HW, al, ws, tune, s);
 }
 
 }  // namespace mn_bn
@@ -342,43 +660,16 @@ int bwd_launch(bool from_y, const float* dy, const float* t, const float* gamma,
 extern "C" {
 
 size_t mn_bn_ws_bytes(int64_t N, int64_t C, int64_t HW) {
-  (void)N;
-  (void)HW;
-  return C > 0 ? mn_bn::ws_bytes_for(C) : 0;
+  return (N > 0 && C > 0 && HW > 0) ? mn_bn::ws_bytes_for(N, C, HW) : 0;
 }
 
 int mn_bn_fwd_train_f32(const float* x, const float* gamma, const float* beta, float* running_mean,
                         float* running_var, float* y, float* save_mean, float* save_invstd,
                         int64_t N, int64_t C, int64_t HW, double momentum, double eps, void* ws,
                         size_t ws_bytes, mn_stream_t stream) {
-  using namespace mn_bn;
-  if (N < 0 || C < 0 || HW < 0) return MN_EINVAL;
-  if (N == 0 || C == 0 || HW == 0) return MN_OK;
-  if (!x || !y || !save_mean || !save_invstd || !ws) return MN_EINVAL;
-  if (ws_bytes < ws_bytes_for(C) || !mn_aligned(ws, 4)) return MN_EINVAL;
-  Plan p;
-  if (!make_plan(N, C, HW, mn_aligned(x, 16) && mn_aligned(y, 16), kTargetBlocks, p))
-    return MN_EUNSUPPORTED;
-  hipStream_t s = mn_stream(stream);
-  float* partial = static_cast<float*>(ws);
-  float* pivot = partial + 2 * (size_t)C * kMaxSplit;
-  const double M = (double)N * (double)HW;
-  const float inv_m = (float)(1.0 / M);
-  const float unbias = M > 1.0 ? (float)(M / (M - 1.0)) : 1.f;
-  if (p.vec == 4) {
-    bn_reduce_kernel<4, true><<<p.blocks, kThreads, 0, s>>>(p.sh, nullptr, x, nullptr, partial,
-                                                            pivot);
-    bn_fwd_apply_kernel<4, true><<<p.blocks, kThreads, 0, s>>>(
-        p.sh, x, nullptr, nullptr, gamma, beta, partial, pivot, y, save_mean, save_invstd,
-        running_mean, running_var, inv_m, unbias, (float)momentum, (float)eps);
-  } else {
-    bn_reduce_kernel<1, true><<<p.blocks, kThreads, 0, s>>>(p.sh, nullptr, x, nullptr, partial,
-                                                            pivot);
-    bn_fwd_apply_kernel<1, true><<<p.blocks, kThreads, 0, s>>>(
-        p.sh, x, nullptr, nullptr, gamma, beta, partial, pivot, y, save_mean, save_invstd,
-        running_mean, running_var, inv_m, unbias, (float)momentum, (float)eps);
-  }
-  return mn_launch_status();
+  return mn_bn::fwd_train_launch(x, gamma, beta, running_mean, running_var, y, save_mean,
+                                 save_invstd, N, C, HW, momentum, eps, ws, ws_bytes,
+                                 mn_stream(stream), mn_bn::Tuning());
 }
 
 int mn_bn_fwd_apply_f32(const float* x, const float* mean, const float* invstd, const float* gamma,
@@ -388,35 +679,62 @@ int mn_bn_fwd_apply_f32(const float* x, const float* mean, const float* invstd, 
   if (N < 0 || C < 0 || HW < 0) return MN_EINVAL;
   if (N == 0 || C == 0 || HW == 0) return MN_OK;
   if (!x || !y || !mean || !invstd) return MN_EINVAL;
-  Plan p;
-  if (!make_plan(N, C, HW, mn_aligned(x, 16) && mn_aligned(y, 16), kTargetBlocks, p))
-    return MN_EUNSUPPORTED;
+  if (!shape_limits(N, C, HW)) return MN_EUNSUPPORTED;
+  Args A = {};
+  const int vec = (HW % 4 == 0 && mn_aligned(x, 16) && mn_aligned(y, 16)) ? 4 : 1;
+  {
+    const uint64_t tot = (uint64_t)N * (HW / vec);
+    int64_t S = (4096 + C - 1) / C;
+    const int64_t cap = (int64_t)((tot + kThreads * kU - 1) / (kThreads * kU));
+    if (S > cap) S = cap;
+    if (S < 1) S = 1;
+    fill_shape(N, C, HW, vec, S, (tot + S - 1) / S, A.sh);
+  }
+  A.b = x;
+  A.gamma = gamma;
+  A.shift = beta;
+  A.out = y;
+  const unsigned blocks = (unsigned)C * A.sh.S;
   hipStream_t s = mn_stream(stream);
-  if (p.vec == 4)
-    bn_fwd_apply_kernel<4, false><<<p.blocks, kThreads, 0, s>>>(
-        p.sh, x, mean, invstd, gamma, beta, nullptr, nullptr, y, nullptr, nullptr, nullptr, nullptr,
-        0.f, 0.f, 0.f, 0.f);
+  if (vec == 4)
+    bn_fwd_saved_kernel<4><<<blocks, kThreads, 0, s>>>(A, mean, invstd);
   else
-    bn_fwd_apply_kernel<1, false><<<p.blocks, kThreads, 0, s>>>(
-        p.sh, x, mean, invstd, gamma, beta, nullptr, nullptr, y, nullptr, nullptr, nullptr, nullptr,
-        0.f, 0.f, 0.f, 0.f);
+    bn_fwd_saved_kernel<1><<<blocks, kThreads, 0, s>>>(A, mean, invstd);
   return mn_launch_status();
 }
 
 int mn_bn_bwd_from_x_f32(const float* dy, const float* x, const float* gamma, const float* mean,
                          const float* invstd, float* dx, float* dgamma, float* dbeta, int64_t N,
                          int64_t C, int64_t HW, void* ws, size_t ws_bytes, mn_stream_t stream) {
-  if (N < 0 || C < 0 || HW < 0 || !mean) return MN_EINVAL;
+  if (!mean) return MN_EINVAL;
   return mn_bn::bwd_launch(false, dy, x, gamma, mean, invstd, dx, dgamma, dbeta, N, C, HW, ws,
-                           ws_bytes, mn_stream(stream), mn_bn::kTargetBlocks);
+                           ws_bytes, mn_stream(stream), mn_bn::Tuning());
 }
 
 int mn_bn_bwd_from_y_f32(const float* dy, const float* y, const float* gamma, const float* beta,
                          const float* invstd, float* dx, float* dgamma, float* dbeta, int64_t N,
                          int64_t C, int64_t HW, void* ws, size_t ws_bytes, mn_stream_t stream) {
-  if (N < 0 || C < 0 || HW < 0) return MN_EINVAL;
   return mn_bn::bwd_launch(true, dy, y, gamma, beta, invstd, dx, dgamma, dbeta, N, C, HW, ws,
-                           ws_bytes, mn_stream(stream), mn_bn::kTargetBlocks);
+                           ws_bytes, mn_stream(stream), mn_bn::Tuning());
 }
 
 }  // extern "C"
+
+#ifdef MN_TUNING
+// Only in tuning builds: the backward-from-output with explicit launch tunables.
+extern "C" int mn_tune_bn_bwd_from_y(const float* dy, const float* y, const float* gamma,
+                                     const float* beta, const float* invstd, float* dx,
+                                     float* dgamma, float* dbeta, int64_t N, int64_t C, int64_t HW,
+                                     void* ws, size_t ws_bytes, mn_stream_t stream,
+                                     int target_blocks, int resident, int keep, int threads,
+                                     int grid) {
+  mn_bn::Tuning t;
+  t.target_blocks = target_blocks;
+  t.resident = resident;
+  t.keep = keep;
+  t.threads = threads;
+  t.grid = grid;
+  return mn_bn::bwd_launch(true, dy, y, gamma, beta, invstd, dx, dgamma, dbeta, N, C, HW, ws,
+                           ws_bytes, mn_stream(stream), t);
+}
+#endif

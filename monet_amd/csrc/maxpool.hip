@@ -162,6 +162,68 @@ __global__ __launch_bounds__(kThreads) void maxpool_bwd_idx_kernel(
   }
 }
 
+// Backward for kernel 3, stride 2, pad 1, dilation 1 with even H, W % 4 == 0
+// (so PH = H/2, PW = W/2).  One workgroup per (n, c) plane; a thread produces a
+// 2-row x 4-column patch of dx from the 2 x 3 windows that can reach it, so
+// every dy / index element is fetched by at most two threads and every dx
+// element is written once with 16-byte stores.  Window (ph, pw) covers rows
+// 2ph-1..2ph+1 and columns 2pw-1..2pw+1; index k = ch*3 + cw.
+__global__ __launch_bounds__(kThreads) void maxpool_bwd_k3s2p1_kernel(
+    const float* __restrict__ dy, const uint8_t* __restrict__ idx4, float* __restrict__ dx, int H,
+    int W) {
+  const int PH = H >> 1, PW = W >> 1, QW = W >> 2, RH = H >> 1;
+  const size_t plane = blockIdx.x;
+  const float* dyp = dy + plane * (size_t)PH * PW;
+  const uint8_t* ip = idx4 + ((plane * (size_t)PH * PW) >> 1);  // PH*PW is even
+  float* dxp = dx + plane * (size_t)H * W;
+  const int items = RH * QW;
+  const int qstep = kThreads / QW, rstep = kThreads - qstep * QW;
+  int r = threadIdx.x / QW;
+  int q = threadIdx.x - r * QW;
+  for (int it = threadIdx.x; it < items; it += kThreads) {
+    // windows: rows r (A) and r+1 (B); columns 2q, 2q+1, 2q+2
+    const bool rowB = r + 1 < PH;
+    const bool col2 = 2 * q + 2 < PW;
+    const int oA = r * PW + 2 * q;  // even
+    const int oB = oA + PW;
+    const uint32_t a01 = ip[oA >> 1];
+    const uint32_t a2 = col2 ? ip[(oA >> 1) + 1] : 0xFFu;
+    const uint32_t b01 = rowB ? ip[oB >> 1] : 0xFFu;
+    const uint32_t b2 = (rowB && col2) ? ip[(oB >> 1) + 1] : 0xFFu;
+    const float2_t ga = *reinterpret_cast<const float2_t*>(dyp + oA);
+    const float ga2 = col2 ? dyp[oA + 2] : 0.f;
+    float2_t gb = {0.f, 0.f};
+    if (rowB) gb = *reinterpret_cast<const float2_t*>(dyp + oB);
+    const float gb2 = (rowB && col2) ? dyp[oB + 2] : 0.f;
+    const uint32_t iA0 = a01 >> 4, iA1 = a01 & 15u, iA2 = a2 >> 4;
+    const uint32_t iB0 = b01 >> 4, iB1 = b01 & 15u, iB2 = b2 >> 4;  // 0xFF >> 4 = 15: never a k < 9
+#define MN_M(i, k, g) ((i) == (k) ? (g) : 0.f)
+    float4_t top, bot;
+    // row 2r: only window row A, ch = 1
+    top.x = 0.f + MN_M(iA0, 4u, ga.x);
+    top.y = 0.f + MN_M(iA0, 5u, ga.x) + MN_M(iA1, 3u, ga.y);
+    top.z = 0.f + MN_M(iA1, 4u, ga.y);
+    top.w = 0.f + MN_M(iA1, 5u, ga.y) + MN_M(iA2, 3u, ga2);
+    // row 2r+1: window row A with ch = 2, then window row B with ch = 0
+    bot.x = 0.f + MN_M(iA0, 7u, ga.x) + MN_M(iB0, 1u, gb.x);
+    bot.y = 0.f + MN_M(iA0, 8u, ga.x) + MN_M(iA1, 6u, ga.y) + MN_M(iB0, 2u, gb.x) +
+            MN_M(iB1, 0u, gb.y);
+    bot.z = 0.f + MN_M(iA1, 7u, ga.y) + MN_M(iB1, 1u, gb.y);
+    bot.w = 0.f + MN_M(iA1, 8u, ga.y) + MN_M(iA2, 6u, ga2) + MN_M(iB1, 2u, gb.y) +
+            MN_M(iB2, 0u, gb2);
+#undef MN_M
+    float* o = dxp + (size_t)(2 * r) * W + 4 * q;
+    st_stream(reinterpret_cast<float4_t*>(o), top);
+    st_stream(reinterpret_cast<float4_t*>(o + W), bot);
+    r += qstep;
+    q += rstep;
+    if (q >= QW) {
+      q -= QW;
+      ++r;
+    }
+  }
+}
+
 int check_geo(const mn_pool2d* g) {
   if (!g) return MN_EINVAL;
   if (g->N < 0 || g->C < 0 || g->H <= 0 || g->W <= 0 || g->PH <= 0 || g->PW <= 0) return MN_EINVAL;
@@ -250,7 +312,10 @@ int mn_maxpool_bwd_idx_f32(const mn_pool2d* g, const float* dy, const uint8_t* i
   if ((size_t)g->N * g->C == 0) return MN_OK;
   if (!dy || !dx || !idx4) return MN_EINVAL;
   hipStream_t s = mn_stream(stream);
-  if (is_ct(g, 3, 2, 1))
+  if (is_ct(g, 3, 2, 1) && g->H % 2 == 0 && g->W % 4 == 0 && mn_aligned(dx, 16) &&
+      mn_aligned(dy, 8) && g->W / 4 <= kThreads)
+    maxpool_bwd_k3s2p1_kernel<<<(unsigned)g->N * g->C, kThreads, 0, s>>>(dy, idx4, dx, g->H, g->W);
+  else if (is_ct(g, 3, 2, 1))
     launch_bwd(CtGeo<3, 2, 1>{}, g, dy, idx4, dx, s);
   else if (is_ct(g, 2, 2, 0))
     launch_bwd(CtGeo<2, 2, 0>{}, g, dy, idx4, dx, s);

@@ -300,6 +300,22 @@ def test_bn_from_output_with_large_mean_and_small_gamma(cuda):
     assert_rel(host(dg), odg, 5e-4, "dgamma")
 
 
+def test_bn_channel_too_large_to_keep_on_chip(cuda):
+    # 4.3M elements per channel: more than 256 register-resident pieces, so the
+    # two-launch (reduce, apply) formulation runs
+    shape = (1, 2, 2100, 2048)
+    x, gamma, beta, dy = bn_problem(shape, 5)
+    oy, omean, oinv, _, _ = O.bn_fwd_train(x, gamma, beta, None, None, 0.1, 1e-5)
+    odx, odg, odb = O.bn_bwd_from_x(dy, x, gamma, omean, oinv)
+    tw, tb = dev(gamma, cuda), dev(beta, cuda)
+    y, mean, invstd = bn_ops.bn_forward_train(dev(x, cuda), tw, tb, None, None, 0.1, 1e-5)
+    assert_rel(host(y), oy, 1e-5, "y")
+    dx, dg, db = bn_ops.bn_backward_from_output(dev(dy, cuda), y, tw, tb, invstd)
+    assert_rel(host(dx), odx, 2e-5, "dx from y")
+    assert_rel(host(dg), odg, 1e-4, "dgamma")
+    assert_rel(host(db), odb, 1e-4, "dbeta")
+
+
 def test_bn_non_affine_and_inplace_output(cuda):
     shape = (4, 3, 8, 8)
     x, _, _, dy = bn_problem(shape, 3)
