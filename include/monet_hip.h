@@ -157,6 +157,51 @@ int mn_softmax_bwd_f32(const float* dy, const float* y, float* dx, int64_t outer
 int mn_xent_bwd_f32(const float* logits, const int64_t* labels, float* dlogits, int64_t outer,
                     int64_t dim, int64_t inner, float scale, mn_stream_t stream);
 
+/* ----------------------------------------------------------- convolution --
+ * 2-D convolution over NCHW tensors, weights [K, C, R, S], groups == 1.
+ * P/Q are the output sizes: floor((H + 2*pH - dH*(R-1) - 1) / sH) + 1. */
+typedef struct mn_conv2d {
+  int32_t N, C, H, W;
+  int32_t K, R, S;
+  int32_t sH, sW, pH, pW, dH, dW;
+  int32_t P, Q;
+  int32_t groups;
+} mn_conv2d;
+
+#define MN_CONV_FWD 0
+#define MN_CONV_BWD_DATA 1
+#define MN_CONV_BWD_WEIGHT 2
+#define MN_F32 0 /* fp32 tensors, fp32 matrix-core arithmetic */
+
+/* Number of kernel variants ("algorithms") per direction; variant 0 always
+ * runs and needs no workspace.  Takes the role of n_fwd_algos / n_bwd_ip_algos
+ * / n_bwd_wt_algos (monet/lm_ops/conv.cpp:728-730); the variants are this
+ * library's own memory / speed tiers, not cuDNN's algorithm list
+ * (conv.cpp:21-46):
+ *   forward          0 implicit GEMM, no workspace
+ *   backward-data    0 implicit GEMM reading the weights through strides
+ *                    1 same with a transposed weight copy in the workspace
+ *   backward-weight  0 split reduction combined with atomics into a cleared dw
+ *                    1 split reduction through per-split partials in the
+ *                      workspace, then a fixed-order sum (reproducible) */
+int mn_conv_n_variants(int direction);
+/* Workspace bytes a (direction, variant, dtype) needs for this geometry
+ * (role of the cudnnGet*WorkspaceSize queries at conv.cpp:314-324). */
+int mn_conv_ws_bytes(const mn_conv2d* g, int direction, int variant, int dtype, size_t* bytes);
+/* y = conv(x, w) (+ bias[k] if bias != NULL).  Replaces cudnn_convolution
+ * (monet/lm_ops/conv.cpp:389-400, raw call :299-340) plus the bias add of
+ * conv.py:284-285.  MN_EUNSUPPORTED for a variant that cannot run the shape. */
+int mn_conv_fwd(const mn_conv2d* g, const void* x, const void* w, const void* bias, void* y,
+                void* ws, size_t ws_bytes, int variant, int dtype, mn_stream_t stream);
+/* dx = gradient w.r.t. the input; writes every element of dx.  Replaces
+ * cudnn_convolution_backward_input (conv.cpp:503-515, raw call :409-449). */
+int mn_conv_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void* dx, void* ws,
+                     size_t ws_bytes, int variant, int dtype, mn_stream_t stream);
+/* dw = gradient w.r.t. the weights; writes every element of dw.  Replaces
+ * cudnn_convolution_backward_weight (conv.cpp:676-688, raw call :550-591). */
+int mn_conv_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, void* dw, void* ws,
+                       size_t ws_bytes, int variant, int dtype, mn_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -24,6 +24,17 @@ class MonetHipError(RuntimeError):
         self.status = status
 
 
+class Conv2d(Structure):
+    """Mirror of `struct mn_conv2d`."""
+    _fields_ = [(k, c_int32) for k in
+                ("N", "C", "H", "W", "K", "R", "S", "sH", "sW", "pH", "pW", "dH", "dW", "P", "Q",
+                 "groups")]
+
+
+CONV_FWD, CONV_BWD_DATA, CONV_BWD_WEIGHT = 0, 1, 2
+F32 = 0
+
+
 class Pool2d(Structure):
     """Mirror of `struct mn_pool2d`."""
     _fields_ = [(k, c_int32) for k in
@@ -57,9 +68,14 @@ _SIGNATURES = {
     "mn_softmax_fwd_f32": (c_int, [_P, _P, c_int64, c_int64, c_int64, _P]),
     "mn_softmax_bwd_f32": (c_int, [_P, _P, _P, c_int64, c_int64, c_int64, _P]),
     "mn_xent_bwd_f32": (c_int, [_P, _P, _P, c_int64, c_int64, c_int64, c_float, _P]),
+    "mn_conv_n_variants": (c_int, [c_int]),
+    "mn_conv_ws_bytes": (c_int, [POINTER(Conv2d), c_int, c_int, c_int, POINTER(c_size_t)]),
+    "mn_conv_fwd": (c_int, [POINTER(Conv2d), _P, _P, _P, _P, _P, c_size_t, c_int, c_int, _P]),
+    "mn_conv_bwd_data": (c_int, [POINTER(Conv2d), _P, _P, _P, _P, c_size_t, c_int, c_int, _P]),
+    "mn_conv_bwd_weight": (c_int, [POINTER(Conv2d), _P, _P, _P, _P, c_size_t, c_int, c_int, _P]),
 }
 # entry points whose int return value is NOT a status code
-_UNCHECKED = {"mn_abi_version"}
+_UNCHECKED = {"mn_abi_version", "mn_conv_n_variants"}
 
 _lib = None
 

@@ -1,0 +1,301 @@
+"""Convolution operator implementations (reference: monet/lm_ops/conv.py).
+
+  GreedyAlgoConvolution    times every kernel variant on first use and keeps
+                           the fastest that fits the memory budget (conv.py:105-258)
+  SpecificAlgoConvolution  runs the variant the schedule solver chose
+                           (conv.py:260-341)
+
+`algorithm` follows the reference's encoding: forward uses it as the variant
+index; backward uses `algorithm // 10` as what to compute (0: weight gradient
+(+ bias gradient), 1: input gradient, 2: both) and `algorithm % 10` as the
+variant index.  A variant that cannot run (index out of range, unsupported
+shape) raises; the op then retries with variant 0, which always runs, and
+rewrites `algorithm` the way the reference falls back to its default
+algorithm (conv.py:279-283, 308-312, 321-325).
+
+The variants are the kernels' own memory / speed tiers (see
+include/monet_hip.h), and their workspaces are torch tensors, so the caching
+allocator - and with it the solver's memory profile - sees them.
+"""
+import ctypes
+from time import time
+
+import torch
+
+from .. import _lib, config
+from .base import OP, InputStorage, implements
+
+DEFAULT_VARIANT = 0
+
+
+def _pair(v):
+    v = list(v) if isinstance(v, (list, tuple, torch.Size)) else [v]
+    if len(v) == 1:
+        v = v * 2
+    return int(v[0]), int(v[1])
+
+
+def conv_geometry(input_shape, weight_shape, stride, padding, dilation, groups):
+    N, C, H, W = [int(d) for d in input_shape]
+    K, Cg, R, S = [int(d) for d in weight_shape]
+    sH, sW = _pair(stride)
+    pH, pW = _pair(padding)
+    dH, dW = _pair(dilation)
+    if Cg * groups != C:
+        raise RuntimeError("weight does not match the input channels")
+    P = (H + 2 * pH - dH * (R - 1) - 1) // sH + 1
+    Q = (W + 2 * pW - dW * (S - 1) - 1) // sW + 1
+    if P <= 0 or Q <= 0:
+        raise RuntimeError("convolution output would be empty")
+    return _lib.Conv2d(N, C, H, W, K, R, S, sH, sW, pH, pW, dH, dW, P, Q, int(groups))
+
+
+def n_fwd_algos():
+    return _lib.load().mn_conv_n_variants(_lib.CONV_FWD)
+
+
+def n_bwd_ip_algos():
+    return _lib.load().mn_conv_n_variants(_lib.CONV_BWD_DATA)
+
+
+def n_bwd_wt_algos():
+    return _lib.load().mn_conv_n_variants(_lib.CONV_BWD_WEIGHT)
+
+
+def _workspace(geo, direction, variant, device):
+    n = ctypes.c_size_t(0)
+    _lib.call("mn_conv_ws_bytes", geo, direction, variant, _lib.F32, ctypes.byref(n))
+    if n.value == 0:
+        return None, 0
+    return torch.empty(n.value, dtype=torch.uint8, device=device), n.value
+
+
+def _prep(t, name):
+    _lib.require_gpu_tensor(t, name, torch.float32)
+    t = t.detach()
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def conv_forward(input_, weight, bias, padding, stride, dilation, groups, variant):
+    """y = conv2d(input, weight) (+ bias) with kernel variant `variant`."""
+    x, w = _prep(input_, "input"), _prep(weight, "weight")
+    b = None if bias is None else _prep(bias, "bias")
+    geo = conv_geometry(x.shape, w.shape, stride, padding, dilation, groups)
+    ws, nbytes = _workspace(geo, _lib.CONV_FWD, variant, x.device)
+    y = torch.empty((geo.N, geo.K, geo.P, geo.Q), dtype=torch.float32, device=x.device)
+    _lib.call("mn_conv_fwd", geo, _lib.ptr(x), _lib.ptr(w), _lib.ptr(b), _lib.ptr(y), _lib.ptr(ws),
+              nbytes, variant, _lib.F32, _lib.stream_ptr(x.device))
+    return y
+
+
+def conv_backward_input(input_shape, grad_output, weight, padding, stride, dilation, groups,
+                        variant):
+    g, w = _prep(grad_output, "grad_output"), _prep(weight, "weight")
+    geo = conv_geometry(input_shape, w.shape, stride, padding, dilation, groups)
+    if tuple(g.shape) != (geo.N, geo.K, geo.P, geo.Q):
+        raise RuntimeError("grad_output does not match the convolution geometry")
+    ws, nbytes = _workspace(geo, _lib.CONV_BWD_DATA, variant, g.device)
+    dx = torch.empty([int(d) for d in input_shape], dtype=torch.float32, device=g.device)
+    _lib.call("mn_conv_bwd_data", geo, _lib.ptr(g), _lib.ptr(w), _lib.ptr(dx), _lib.ptr(ws), nbytes,
+              variant, _lib.F32, _lib.stream_ptr(g.device))
+    return dx
+
+
+def conv_backward_weight(weight_shape, grad_output, input_, padding, stride, dilation, groups,
+                         variant):
+    g, x = _prep(grad_output, "grad_output"), _prep(input_, "input")
+    geo = conv_geometry(x.shape, weight_shape, stride, padding, dilation, groups)
+    if tuple(g.shape) != (geo.N, geo.K, geo.P, geo.Q):
+        raise RuntimeError("grad_output does not match the convolution geometry")
+    ws, nbytes = _workspace(geo, _lib.CONV_BWD_WEIGHT, variant, g.device)
+    dw = torch.empty([int(d) for d in weight_shape], dtype=torch.float32, device=g.device)
+    _lib.call("mn_conv_bwd_weight", geo, _lib.ptr(g), _lib.ptr(x), _lib.ptr(dw), _lib.ptr(ws),
+              nbytes, variant, _lib.F32, _lib.stream_ptr(g.device))
+    return dw
+
+
+def _depthwise_forward(input_, weight, bias, stride, padding, dilation, groups):
+    return torch.ops.aten.convolution(input_, weight, bias, list(stride), list(padding),
+                                      list(dilation), False, [0, 0], groups)
+
+
+def _depthwise_backward(grad, input_, weight, stride, padding, dilation, groups, mask):
+    di, dw, _ = torch.ops.aten.convolution_backward(
+        grad, input_, weight, None, list(stride), list(padding), list(dilation), False, [0, 0],
+        groups, [bool(mask[0]), bool(mask[1]), False])
+    return di, dw
+
+
+class _ConvBase(OP):
+    backward_storage = InputStorage(0, 1)
+    params = None
+    algorithm = -1
+    is_depthwise = False
+
+    n_fwd_algos = staticmethod(n_fwd_algos)
+    n_bwd_ip_algos = staticmethod(n_bwd_ip_algos)
+    n_bwd_wt_algos = staticmethod(n_bwd_wt_algos)
+
+    def _record(self, input_, weight, bias, stride, padding, dilation, groups):
+        self.params = (stride, padding, dilation, groups, input_.shape, weight.shape,
+                       [input_.requires_grad, weight.requires_grad,
+                        bias is not None and bias.requires_grad])
+
+    # hooks the two subclasses differ in
+    def _fwd_variant(self, *a):
+        raise NotImplementedError
+
+    def _bwd_wt_variant(self, *a):
+        raise NotImplementedError
+
+    def _bwd_ip_variant(self, *a):
+        raise NotImplementedError
+
+    def forward(self, input_, weight, bias, stride, padding, dilation, transposed, output_padding,
+                groups, *args, **kwargs):
+        with torch.no_grad():
+            assert not transposed
+            self._record(input_, weight, bias, stride, padding, dilation, groups)
+            if self.is_depthwise or groups != 1:
+                return _depthwise_forward(input_, weight, bias, stride, padding, dilation, groups)
+            return self._fwd_variant(input_, weight, bias, padding, stride, dilation, groups)
+
+    def backward(self, grad_output, stored, nodel=False):
+        with torch.no_grad():
+            input_, weight = stored
+            stride, padding, dilation, groups, input_shape, weight_shape, do_grad = self.params
+            kind = self.algorithm // 10
+            if not nodel:
+                del stored[1]
+                del stored[0]
+            di = dw = db = None
+            if self.is_depthwise or groups != 1:
+                di, dw = _depthwise_backward(grad_output, input_, weight, stride, padding, dilation,
+                                             groups, do_grad[:2])
+            else:
+                if kind in (0, 2) and input_ is not None:
+                    if do_grad[1]:
+                        dw = self._bwd_wt_variant(weight_shape, grad_output, input_, padding, stride,
+                                                  dilation, groups)
+                    if do_grad[2]:
+                        db = grad_output.sum([0, 2, 3])
+                del input_
+                if kind in (1, 2) and weight is not None and do_grad[0]:
+                    di = self._bwd_ip_variant(input_shape, grad_output, weight, padding, stride,
+                                              dilation, groups)
+            if do_grad[2]:
+                return di, dw, db
+            return di, dw
+
+
+@implements(['aten::_convolution'], ['conv_multiway_newnode', 'conv_normal'])
+class SpecificAlgoConvolution(_ConvBase):
+    """Runs exactly the variant in `self.algorithm`; falls back to variant 0."""
+
+    def _fwd_variant(self, input_, weight, bias, padding, stride, dilation, groups):
+        try:
+            return conv_forward(input_, weight, bias, padding, stride, dilation, groups,
+                                self.algorithm)
+        except Exception:
+            out = conv_forward(input_, weight, bias, padding, stride, dilation, groups,
+                               DEFAULT_VARIANT)
+            self.algorithm = DEFAULT_VARIANT
+            return out
+
+    def _bwd_wt_variant(self, weight_shape, grad, input_, padding, stride, dilation, groups):
+        kind, algo = self.algorithm // 10, self.algorithm % 10
+        try:
+            return conv_backward_weight(weight_shape, grad, input_, padding, stride, dilation,
+                                        groups, algo)
+        except Exception:
+            out = conv_backward_weight(weight_shape, grad, input_, padding, stride, dilation,
+                                       groups, DEFAULT_VARIANT)
+            self.algorithm = kind * 10 + DEFAULT_VARIANT
+            return out
+
+    def _bwd_ip_variant(self, input_shape, grad, weight, padding, stride, dilation, groups):
+        kind, algo = self.algorithm // 10, self.algorithm % 10
+        try:
+            return conv_backward_input(input_shape, grad, weight, padding, stride, dilation, groups,
+                                       algo)
+        except Exception:
+            out = conv_backward_input(input_shape, grad, weight, padding, stride, dilation, groups,
+                                      DEFAULT_VARIANT)
+            self.algorithm = kind * 10 + DEFAULT_VARIANT
+            return out
+
+
+def _autotune(n_variants, run):
+    """Index of the fastest variant (10 runs each) whose peak allocation stays
+    under config.budget * 1.01 GB (no limit when the budget is 0)."""
+    best, best_t = -1, None
+    torch.cuda.empty_cache()
+    for alg in range(n_variants):
+        try:
+            torch.cuda.reset_peak_memory_stats()
+            torch.cuda.synchronize()
+            t1 = time()
+            for _ in range(10):
+                out = run(alg)
+                del out
+            torch.cuda.synchronize()
+            t = time() - t1
+            peak_gb = torch.cuda.max_memory_allocated() / 1024 / 1024 / 1024
+            fits = config.budget <= 0 or peak_gb < config.budget * 1.01
+            if fits and (best_t is None or t < best_t):
+                best, best_t = alg, t
+        except Exception:
+            pass
+        torch.cuda.empty_cache()
+        torch.cuda.reset_peak_memory_stats()
+    if best == -1:
+        best = DEFAULT_VARIANT
+    return best
+
+
+@implements(['aten::_convolution'], ['normal', 'multiway_newnode', 'multiway', 'newnode'])
+class GreedyAlgoConvolution(_ConvBase):
+    """Picks each direction's variant by timing on first use, then keeps it."""
+    fwd_algo = -1
+    bwd_ip_algo = -1
+    bwd_wt_algo = -1
+
+    def _fwd_variant(self, input_, weight, bias, padding, stride, dilation, groups):
+        if self.fwd_algo == -1:
+            self.fwd_algo = _autotune(n_fwd_algos(), lambda alg: conv_forward(
+                input_, weight, bias, padding, stride, dilation, groups, alg))
+        try:
+            return conv_forward(input_, weight, bias, padding, stride, dilation, groups,
+                                self.fwd_algo)
+        except Exception:
+            self.fwd_algo = DEFAULT_VARIANT
+            return conv_forward(input_, weight, bias, padding, stride, dilation, groups,
+                                DEFAULT_VARIANT)
+
+    def _bwd_wt_variant(self, weight_shape, grad, input_, padding, stride, dilation, groups):
+        if self.bwd_wt_algo == -1:
+            self.bwd_wt_algo = _autotune(n_bwd_wt_algos(), lambda alg: conv_backward_weight(
+                weight_shape, grad, input_, padding, stride, dilation, groups, alg))
+        try:
+            return conv_backward_weight(weight_shape, grad, input_, padding, stride, dilation,
+                                        groups, self.bwd_wt_algo)
+        except Exception:
+            self.bwd_wt_algo = DEFAULT_VARIANT
+            return conv_backward_weight(weight_shape, grad, input_, padding, stride, dilation,
+                                        groups, DEFAULT_VARIANT)
+
+    def _bwd_ip_variant(self, input_shape, grad, weight, padding, stride, dilation, groups):
+        if self.bwd_ip_algo == -1:
+            self.bwd_ip_algo = _autotune(n_bwd_ip_algos(), lambda alg: conv_backward_input(
+                input_shape, grad, weight, padding, stride, dilation, groups, alg))
+        try:
+            return conv_backward_input(input_shape, grad, weight, padding, stride, dilation, groups,
+                                       self.bwd_ip_algo)
+        except Exception:
+            self.bwd_ip_algo = DEFAULT_VARIANT
+            return conv_backward_input(input_shape, grad, weight, padding, stride, dilation, groups,
+                                       DEFAULT_VARIANT)
+
+    def backward(self, grad_output, stored, nodel=False):
+        # the greedy op ignores the variant digit of `algorithm` (it uses its own choice)
+        return super().backward(grad_output, stored, nodel)

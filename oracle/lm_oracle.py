@@ -349,3 +349,76 @@ def xent_bwd(logits, labels, scale=None, dtype=np.float64):
     o, i = np.meshgrid(np.arange(p.shape[0]), np.arange(p.shape[2]), indexing="ij")
     p[o, lab, i] -= 1.0
     return (p * scale).reshape(np.shape(logits))
+
+
+# -------------------------------------------------------------- convolution
+
+
+def _conv_geo(x_shape, w_shape, stride, padding, dilation):
+    N, C, H, W = x_shape
+    K, C2, R, S = w_shape
+    assert C == C2, "groups == 1 only"
+    sH, sW = _pair(stride)
+    pH, pW = _pair(padding)
+    dH, dW = _pair(dilation)
+    P = (H + 2 * pH - dH * (R - 1) - 1) // sH + 1
+    Q = (W + 2 * pW - dW * (S - 1) - 1) // sW + 1
+    return (N, C, H, W, K, R, S, sH, sW, pH, pW, dH, dW, P, Q)
+
+
+def conv_fwd(x, w, bias=None, stride=1, padding=0, dilation=1, dtype=np.float64):
+    """y[n,k,p,q] = sum_{c,r,s} w[k,c,r,s] * x[n,c,p*sH+r*dH-pH,q*sW+s*dW-pW] (+ bias[k]).
+
+    What cudnnConvolutionForward computes for cudnn_convolution
+    (monet/lm_ops/conv.cpp:299-340) with CUDNN_CROSS_CORRELATION, plus the bias
+    add of conv.py:284-285.  Pinned by: F.conv2d on CPU in float64.
+    """
+    x = np.asarray(x, dtype=dtype)
+    w = np.asarray(w, dtype=dtype)
+    N, C, H, W, K, R, S, sH, sW, pH, pW, dH, dW, P, Q = _conv_geo(x.shape, w.shape, stride,
+                                                                  padding, dilation)
+    xp = np.zeros((N, C, H + 2 * pH, W + 2 * pW), dtype=dtype)
+    xp[:, :, pH:pH + H, pW:pW + W] = x
+    y = np.zeros((N, K, P, Q), dtype=dtype)
+    for r in range(R):
+        for s in range(S):
+            patch = xp[:, :, r * dH:r * dH + (P - 1) * sH + 1:sH, s * dW:s * dW + (Q - 1) * sW + 1:sW]
+            y += np.einsum("ncpq,kc->nkpq", patch, w[:, :, r, s], optimize=True)
+    if bias is not None:
+        y += np.asarray(bias, dtype=dtype)[None, :, None, None]
+    return y
+
+
+def conv_bwd_data(dy, w, x_shape, stride=1, padding=0, dilation=1, dtype=np.float64):
+    """dx: every output gradient is spread back over the taps that produced it
+    (cudnnConvolutionBackwardData, conv.cpp:409-449).
+    Pinned by: aten.convolution_backward on CPU in float64."""
+    dy = np.asarray(dy, dtype=dtype)
+    w = np.asarray(w, dtype=dtype)
+    N, C, H, W, K, R, S, sH, sW, pH, pW, dH, dW, P, Q = _conv_geo(x_shape, w.shape, stride,
+                                                                  padding, dilation)
+    dxp = np.zeros((N, C, H + 2 * pH, W + 2 * pW), dtype=dtype)
+    for r in range(R):
+        for s in range(S):
+            dxp[:, :, r * dH:r * dH + (P - 1) * sH + 1:sH,
+                s * dW:s * dW + (Q - 1) * sW + 1:sW] += np.einsum("nkpq,kc->ncpq", dy,
+                                                                 w[:, :, r, s], optimize=True)
+    return dxp[:, :, pH:pH + H, pW:pW + W]
+
+
+def conv_bwd_weight(dy, x, w_shape, stride=1, padding=0, dilation=1, dtype=np.float64):
+    """dw[k,c,r,s] = sum_{n,p,q} dy[n,k,p,q] * x[n,c,p*sH+r*dH-pH,q*sW+s*dW-pW]
+    (cudnnConvolutionBackwardFilter, conv.cpp:550-591).
+    Pinned by: aten.convolution_backward on CPU in float64."""
+    dy = np.asarray(dy, dtype=dtype)
+    x = np.asarray(x, dtype=dtype)
+    N, C, H, W, K, R, S, sH, sW, pH, pW, dH, dW, P, Q = _conv_geo(x.shape, w_shape, stride,
+                                                                  padding, dilation)
+    xp = np.zeros((N, C, H + 2 * pH, W + 2 * pW), dtype=dtype)
+    xp[:, :, pH:pH + H, pW:pW + W] = x
+    dw = np.zeros((K, C, R, S), dtype=dtype)
+    for r in range(R):
+        for s in range(S):
+            patch = xp[:, :, r * dH:r * dH + (P - 1) * sH + 1:sH, s * dW:s * dW + (Q - 1) * sW + 1:sW]
+            dw[:, :, r, s] = np.einsum("nkpq,ncpq->kc", dy, patch, optimize=True)
+    return dw

@@ -1,0 +1,169 @@
+"""GPU parity of the convolution kernels (all directions, all variants) against
+the float64 CPU oracle, through the operator classes and the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+import monet_amd.lm_ops as lm_ops
+from monet_amd.lm_ops import conv as conv_ops
+from oracle import lm_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+# fp32 matrix-core accumulation against a float64 oracle: error relative to the largest
+# magnitude of the expected tensor
+TOL = 1e-5
+
+CASES = [
+    # (x shape, w shape, stride, padding, dilation)
+    ((2, 3, 9, 9), (4, 3, 3, 3), 1, 1, 1),
+    ((1, 5, 12, 10), (7, 5, 3, 3), 2, 1, 1),
+    ((2, 4, 8, 8), (6, 4, 1, 1), 1, 0, 1),
+    ((2, 4, 9, 9), (6, 4, 1, 1), 2, 0, 1),
+    ((1, 3, 15, 15), (8, 3, 7, 7), 2, 3, 1),
+    ((1, 2, 11, 11), (3, 2, 3, 3), 1, 2, 2),
+    ((2, 3, 7, 9), (2, 3, 2, 3), (2, 1), (1, 0), 1),
+    ((3, 130, 14, 14), (140, 130, 3, 3), 1, 1, 1),     # tiles with ragged edges in every dimension
+    ((4, 256, 14, 14), (256, 256, 3, 3), 1, 1, 1),     # ResNet-50 layer3 shape at a small batch
+    ((2, 64, 56, 56), (256, 64, 1, 1), 1, 0, 1),       # 1x1 expansion
+    ((2, 128, 28, 28), (128, 128, 3, 3), 2, 1, 1),     # strided 3x3
+    ((2, 256, 28, 28), (512, 256, 1, 1), 2, 0, 1),     # strided 1x1 (downsample)
+    ((2, 3, 64, 64), (64, 3, 7, 7), 2, 3, 1),          # stem
+    ((1, 16, 33, 47), (24, 16, 3, 3), 1, 1, 1),        # odd spatial sizes
+]
+
+
+def dev(a, cuda):
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(cuda)
+
+
+def host(t):
+    return t.detach().cpu().numpy()
+
+
+def assert_rel(got, exp, tol, what):
+    exp = np.asarray(exp, np.float64)
+    err = np.abs(np.asarray(got, np.float64) - exp).max()
+    scale = max(np.abs(exp).max(), 1e-30)
+    assert err <= tol * scale, f"{what}: max err {err:.3e} vs scale {scale:.3e} ({err / scale:.2e})"
+
+
+def problem(xs, ws, seed=0):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal(xs).astype(np.float32)
+    fan_out = ws[0] * ws[2] * ws[3]
+    w = (rng.standard_normal(ws) * np.sqrt(2.0 / fan_out)).astype(np.float32)
+    b = rng.standard_normal(ws[0]).astype(np.float32)
+    return x, w, b
+
+
+@pytest.mark.parametrize("xs,ws,st,pad,dil", CASES)
+def test_conv_forward(cuda, xs, ws, st, pad, dil):
+    x, w, b = problem(xs, ws)
+    exp = O.conv_fwd(x, w, b, st, pad, dil)
+    exp_nobias = O.conv_fwd(x, w, None, st, pad, dil)
+    for v in range(conv_ops.n_fwd_algos()):
+        y = conv_ops.conv_forward(dev(x, cuda), dev(w, cuda), dev(b, cuda), pad, st, dil, 1, v)
+        assert list(y.shape) == list(exp.shape)
+        assert_rel(host(y), exp, TOL, f"forward variant {v}")
+        y = conv_ops.conv_forward(dev(x, cuda), dev(w, cuda), None, pad, st, dil, 1, v)
+        assert_rel(host(y), exp_nobias, TOL, f"forward variant {v} (no bias)")
+
+
+@pytest.mark.parametrize("xs,ws,st,pad,dil", CASES)
+def test_conv_backward_data(cuda, xs, ws, st, pad, dil):
+    x, w, _ = problem(xs, ws, 1)
+    yshape = O.conv_fwd(x, w, None, st, pad, dil).shape
+    dy = np.random.default_rng(2).standard_normal(yshape).astype(np.float32)
+    exp = O.conv_bwd_data(dy, w, xs, st, pad, dil)
+    for v in range(conv_ops.n_bwd_ip_algos()):
+        # poison the output: the kernel must write every element
+        dx = conv_ops.conv_backward_input(xs, dev(dy, cuda), dev(w, cuda), pad, st, dil, 1, v)
+        assert_rel(host(dx), exp, TOL, f"backward-data variant {v}")
+
+
+@pytest.mark.parametrize("xs,ws,st,pad,dil", CASES)
+def test_conv_backward_weight(cuda, xs, ws, st, pad, dil):
+    x, w, _ = problem(xs, ws, 3)
+    yshape = O.conv_fwd(x, w, None, st, pad, dil).shape
+    dy = np.random.default_rng(4).standard_normal(yshape).astype(np.float32)
+    exp = O.conv_bwd_weight(dy, x, ws, st, pad, dil)
+    outs = []
+    for v in range(conv_ops.n_bwd_wt_algos()):
+        dw = conv_ops.conv_backward_weight(ws, dev(dy, cuda), dev(x, cuda), pad, st, dil, 1, v)
+        assert_rel(host(dw), exp, TOL, f"backward-weight variant {v}")
+        outs.append(dw)
+    # the workspace variant sums its partials in a fixed order: bit-identical run to run
+    again = conv_ops.conv_backward_weight(ws, dev(dy, cuda), dev(x, cuda), pad, st, dil, 1, 1)
+    assert torch.equal(again, outs[1])
+
+
+def test_conv_op_classes_follow_the_algorithm_encoding(cuda):
+    xs, ws = (2, 8, 10, 10), (12, 8, 3, 3)
+    x, w, b = problem(xs, ws, 5)
+    tx = dev(x, cuda).requires_grad_(True)
+    tw = dev(w, cuda).requires_grad_(True)
+    tb = dev(b, cuda).requires_grad_(True)
+    args = (tx, tw, tb, [1, 1], [1, 1], [1, 1], False, [0, 0], 1, False, False, True, True)
+    exp_y = O.conv_fwd(x, w, b, 1, 1, 1)
+    dy = np.random.default_rng(6).standard_normal(exp_y.shape).astype(np.float32)
+    exp_dx = O.conv_bwd_data(dy, w, xs, 1, 1, 1)
+    exp_dw = O.conv_bwd_weight(dy, x, ws, 1, 1, 1)
+    for cls in (lm_ops.conv.SpecificAlgoConvolution, lm_ops.conv.GreedyAlgoConvolution):
+        op = cls()
+        op.algorithm = 0
+        y = op.forward(*args)
+        assert_rel(host(y), exp_y, TOL, "op forward")
+        # timestep t-1: parameter gradients (kind 0); both stored tensors present
+        op.algorithm = 0 * 10 + 1
+        stored = [tx.detach(), tw.detach()]
+        di, dw, db = op.backward(dev(dy, cuda), stored)
+        assert stored == [] and di is None
+        assert_rel(host(dw), exp_dw, TOL, "op dw")
+        assert_rel(host(db), dy.sum(axis=(0, 2, 3)), TOL, "op db")
+        # timestep t: input gradient (kind 1); only the weight is guaranteed
+        op.algorithm = 1 * 10 + 1
+        di, dw, db = op.backward(dev(dy, cuda), [None, tw.detach()], nodel=True)
+        assert dw is None
+        assert_rel(host(di), exp_dx, TOL, "op dx")
+        # kind 2: everything at once, no bias -> 2-tuple
+        op2 = cls()
+        op2.algorithm = 0
+        op2.forward(tx, tw, None, [1, 1], [1, 1], [1, 1], False, [0, 0], 1)
+        op2.algorithm = 20
+        out = op2.backward(dev(dy, cuda), [tx.detach(), tw.detach()])
+        assert len(out) == 2
+        assert_rel(host(out[0]), exp_dx, TOL, "op2 dx")
+        assert_rel(host(out[1]), exp_dw, TOL, "op2 dw")
+
+
+def test_conv_unsupported_variant_falls_back(cuda):
+    xs, ws = (1, 4, 6, 6), (4, 4, 3, 3)
+    x, w, _ = problem(xs, ws, 7)
+    with pytest.raises(RuntimeError, match="unsupported"):
+        conv_ops.conv_forward(dev(x, cuda), dev(w, cuda), None, 1, 1, 1, 1, 7)
+    op = lm_ops.conv.SpecificAlgoConvolution()
+    op.algorithm = 7
+    y = op.forward(dev(x, cuda).requires_grad_(True), dev(w, cuda), None, [1, 1], [1, 1], [1, 1],
+                   False, [0, 0], 1)
+    assert op.algorithm == 0
+    assert_rel(host(y), O.conv_fwd(x, w, None, 1, 1, 1), TOL, "fallback forward")
+    op.algorithm = 19
+    di, dw = op.backward(torch.ones_like(y), [None, dev(w, cuda)], nodel=True)
+    assert op.algorithm == 10 and di is not None
+
+
+def test_depthwise_passthrough(cuda):
+    x = torch.randn(2, 6, 9, 9, device=cuda, requires_grad=True)
+    w = torch.randn(6, 1, 3, 3, device=cuda, requires_grad=True)
+    op = lm_ops.conv.SpecificAlgoConvolution()
+    op.is_depthwise = True
+    y = op.forward(x, w, None, [1, 1], [1, 1], [1, 1], False, [0, 0], 6)
+    ref = torch.nn.functional.conv2d(x, w, None, 1, 1, 1, 6)
+    torch.testing.assert_close(y, ref)
+    g = torch.randn_like(y)
+    ref.backward(g)
+    op.algorithm = 20
+    di, dw = op.backward(g, [x.detach(), w.detach()])
+    torch.testing.assert_close(di, x.grad)
+    torch.testing.assert_close(dw, w.grad)

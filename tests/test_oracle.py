@@ -266,3 +266,54 @@ def test_xent_bwd_matches_autograd(shape):
     tx = torch.from_numpy(x).requires_grad_(True)
     F.cross_entropy(tx, torch.from_numpy(labels)).backward()
     np.testing.assert_allclose(O.xent_bwd(x, labels), tx.grad.numpy(), rtol=1e-10, atol=1e-13)
+
+
+# --------------------------------------------------------------- convolution
+CONV_CASES = [
+    # (x shape, w shape, stride, padding, dilation)
+    ((2, 3, 9, 9), (4, 3, 3, 3), 1, 1, 1),
+    ((1, 5, 12, 10), (7, 5, 3, 3), 2, 1, 1),
+    ((2, 4, 8, 8), (6, 4, 1, 1), 1, 0, 1),
+    ((2, 4, 9, 9), (6, 4, 1, 1), 2, 0, 1),
+    ((1, 3, 15, 15), (8, 3, 7, 7), 2, 3, 1),
+    ((1, 2, 11, 11), (3, 2, 3, 3), 1, 2, 2),
+    ((2, 3, 7, 9), (2, 3, 2, 3), (2, 1), (1, 0), 1),
+]
+
+
+@pytest.mark.parametrize("xs,ws,st,pad,dil", CONV_CASES)
+def test_conv_oracle_matches_torch(xs, ws, st, pad, dil):
+    rng = np.random.default_rng(7)
+    x, w = rng.standard_normal(xs), rng.standard_normal(ws)
+    b = rng.standard_normal(ws[0])
+    tx = torch.from_numpy(x).requires_grad_(True)
+    tw = torch.from_numpy(w).requires_grad_(True)
+    ty = F.conv2d(tx, tw, torch.from_numpy(b), st, pad, dil)
+    y = O.conv_fwd(x, w, b, st, pad, dil)
+    np.testing.assert_allclose(y, ty.detach().numpy(), rtol=1e-11, atol=1e-11)
+    dy = rng.standard_normal(y.shape)
+    ty.backward(torch.from_numpy(dy))
+    np.testing.assert_allclose(O.conv_bwd_data(dy, w, xs, st, pad, dil), tx.grad.numpy(),
+                               rtol=1e-11, atol=1e-11)
+    np.testing.assert_allclose(O.conv_bwd_weight(dy, x, ws, st, pad, dil), tw.grad.numpy(),
+                               rtol=1e-11, atol=1e-11)
+
+
+def test_conv_oracle_brute_force():
+    rng = np.random.default_rng(8)
+    x, w = rng.standard_normal((1, 2, 5, 6)), rng.standard_normal((3, 2, 3, 2))
+    st, pad, dil = (2, 1), (1, 1), (1, 2)
+    y = O.conv_fwd(x, w, None, st, pad, dil)
+    N, C, H, W = x.shape
+    K, _, R, S = w.shape
+    for k in range(K):
+        for p in range(y.shape[2]):
+            for q in range(y.shape[3]):
+                acc = 0.0
+                for c in range(C):
+                    for r in range(R):
+                        for s in range(S):
+                            h, ww = p * st[0] + r * dil[0] - pad[0], q * st[1] + s * dil[1] - pad[1]
+                            if 0 <= h < H and 0 <= ww < W:
+                                acc += w[k, c, r, s] * x[0, c, h, ww]
+                assert abs(acc - y[0, k, p, q]) < 1e-12
