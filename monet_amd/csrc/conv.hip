@@ -89,6 +89,14 @@ __device__ __forceinline__ int acc_row(int v, int lane) {
   return 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
 }
 
+// FAST: the source has a multiple of BK channels and every tensor is < 4 GB.
+// Then the reduction index runs tap-major (kk = tap*Cs + ch): a k-tile lies
+// inside one tap, so the window test and the spatial offset are computed once
+// per tile and thread, every address is a 32-bit byte offset = per-thread
+// constant + per-tile scalar, and almost no vector ALU work competes with the
+// matrix cores.  Otherwise (e.g. 3 input channels) kk = ch*T + tap and every
+// element is decomposed on its own.
+template <bool FAST>
 __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
                                                                const float* __restrict__ a,
                                                                const float* __restrict__ src,
@@ -107,27 +115,66 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
   __syncthreads();
 
   // B loader: this thread always fetches column bcol, rows brow0 + 2*i
+  constexpr int kBRows = BN * BK / kThreads, kARows = BM * BK / kThreads;
   const int bcol = tid & (BN - 1), brow0 = tid / BN;
   const uint32_t col = n0 + bcol;
   const bool col_ok = col < g.ncols;
   int ohs = 0, ows = 0;
-  size_t srcbase = 0;
+  uint32_t img = 0;
   {
     const uint32_t c = col_ok ? col : 0;
-    const uint32_t n = c / ((uint32_t)g.OH * g.OW);
-    const uint32_t rem = c - n * (uint32_t)g.OH * g.OW;
+    img = c / ((uint32_t)g.OH * g.OW);
+    const uint32_t rem = c - img * (uint32_t)g.OH * g.OW;
     const uint32_t oh = rem / g.OW, ow = rem - oh * g.OW;
     ohs = oh * g.ish;
     ows = ow * g.isw;
-    srcbase = (size_t)n * g.Cs * g.Hs * g.Ws;
   }
+  const size_t srcbase = (size_t)img * g.Cs * g.Hs * g.Ws;
   // A loader: this thread always fetches k-column ak, rows arow0 + 16*i
   const int ak = tid & (BK - 1), arow0 = tid / BK;
 
-  float ra[BM * BK / kThreads], rb[BN * BK / kThreads];
+  // FAST: per-thread constant byte offsets
+  const uint32_t plane_b = (uint32_t)g.Hs * g.Ws * 4u;
+  const uint32_t pix_b = ((img * (uint32_t)g.Cs * g.Hs + ohs) * (uint32_t)g.Ws + ows) * 4u +
+                         brow0 * plane_b;
+  uint32_t am_b[kARows];
+  uint32_t am_ok = 0;
+  if (FAST) {
+#pragma unroll
+    for (int i = 0; i < kARows; ++i) {
+      const int m = m0 + arow0 + (kThreads / BK) * i;
+      const bool ok = m < g.M;
+      am_b[i] = ok ? (uint32_t)(((long long)m * g.lda + (long long)ak * g.cha) * 4) : 0u;
+      am_ok |= (ok ? 1u : 0u) << i;
+    }
+  }
+
+  float ra[kARows], rb[kBRows];
+  bool b_ok = true;  // FAST: whether rb holds window elements or must be staged as zeros
+  // FAST fetch of the k-tile at (tap t, first channel c0); t and c0 are uniform.
+  // Only issues the loads: masking happens in stage(), after the multiply of the
+  // current tile, so the loads stay in flight behind the matrix instructions.
+  auto fetch_fast = [&](int t, int c0) {
+    const int dh = lds.tdh[t], dw = lds.tdw[t];
+    const int hh = ohs + dh, ww = ows + dw;
+    b_ok = col_ok && (unsigned)hh < (unsigned)g.Hs && (unsigned)ww < (unsigned)g.Ws;
+    const uint32_t sb = (uint32_t)((((long long)c0 * g.Hs + dh) * g.Ws + dw) * 4);
+    const uint32_t base = b_ok ? pix_b + sb : brow0 * plane_b;
+    const char* sp = reinterpret_cast<const char*>(src);
+#pragma unroll
+    for (int i = 0; i < kBRows; ++i)
+      rb[i] = *reinterpret_cast<const float*>(sp + (base + (kThreads / BN) * i * plane_b));
+    const uint32_t sa = (uint32_t)(((long long)c0 * g.cha + lds.taoff[t]) * 4);
+    const char* ap = reinterpret_cast<const char*>(a);
+#pragma unroll
+    for (int i = 0; i < kARows; ++i) {
+      const bool mok = (am_ok >> i) & 1u;
+      ra[i] = *reinterpret_cast<const float*>(ap + (am_b[i] + (mok ? sa : 0u)));
+    }
+  };
   auto fetch = [&](int k0) {
 #pragma unroll
-    for (int i = 0; i < BN * BK / kThreads; ++i) {
+    for (int i = 0; i < kBRows; ++i) {
       const uint32_t kk = k0 + brow0 + (kThreads / BN) * i;
       float v = 0.f;
       if (col_ok && kk < (uint32_t)g.Kd) {
@@ -148,18 +195,19 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
     }
     const long long koff = k_ok ? (long long)ch * g.cha + lds.taoff[t] : 0;
 #pragma unroll
-    for (int i = 0; i < BM * BK / kThreads; ++i) {
+    for (int i = 0; i < kARows; ++i) {
       const int m = m0 + arow0 + (kThreads / BK) * i;
       ra[i] = (k_ok && m < g.M) ? a[(long long)m * g.lda + koff] : 0.f;
     }
   };
   auto stage = [&](int buf) {
 #pragma unroll
-    for (int i = 0; i < BN * BK / kThreads; ++i)
-      lds.b[buf][brow0 + (kThreads / BN) * i][bcol] = rb[i];
+    for (int i = 0; i < kBRows; ++i)
+      lds.b[buf][brow0 + (kThreads / BN) * i][bcol] = (!FAST || b_ok) ? rb[i] : 0.f;
 #pragma unroll
-    for (int i = 0; i < BM * BK / kThreads; ++i)
-      lds.a[buf][ak][arow0 + (kThreads / BK) * i] = ra[i];
+    for (int i = 0; i < kARows; ++i)
+      lds.a[buf][ak][arow0 + (kThreads / BK) * i] =
+          (!FAST || ((am_ok >> i) & 1u)) ? ra[i] : 0.f;
   };
 
   float16_t acc[2][2];
@@ -172,12 +220,25 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
 
   const int ktiles = (g.Kd + BK - 1) / BK;
   if (ktiles > 0) {
-    fetch(0);
+    int t = 0, c0 = 0;  // FAST: position of the tile being fetched
+    auto fetch_next = [&](int kt) {
+      if (FAST) {
+        fetch_fast(t, c0);
+        c0 += BK;
+        if (c0 == g.Cs) {
+          c0 = 0;
+          ++t;
+        }
+      } else {
+        fetch(kt * BK);
+      }
+    };
+    fetch_next(0);
     stage(0);
     __syncthreads();
     for (int kt = 0; kt < ktiles; ++kt) {
       const int buf = kt & 1;
-      if (kt + 1 < ktiles) fetch((kt + 1) * BK);
+      if (kt + 1 < ktiles) fetch_next(kt + 1);
       mma_tile(lds.a[buf], lds.b[buf], wm, wn, lane, acc);
       if (kt + 1 < ktiles) stage(buf ^ 1);
       __syncthreads();
@@ -416,10 +477,16 @@ static int check(const mn_conv2d* g) {
 }
 
 static void launch_gather(const Gather& g, const float* a, const float* src, const float* bias,
-                          float* dst, hipStream_t s) {
+                          float* dst, unsigned long long src_bytes, unsigned long long a_bytes,
+                          hipStream_t s) {
   if (g.ncols == 0 || g.M == 0) return;
   dim3 grid((g.ncols + BN - 1) / BN, (g.M + BM - 1) / BM);
-  gather_gemm_kernel<<<grid, kThreads, 0, s>>>(g, a, src, bias, dst);
+  const unsigned long long limit = 1ull << 32;
+  const bool fast = g.T > 0 && g.Cs % BK == 0 && src_bytes < limit && a_bytes < limit;
+  if (fast)
+    gather_gemm_kernel<true><<<grid, kThreads, 0, s>>>(g, a, src, bias, dst);
+  else
+    gather_gemm_kernel<false><<<grid, kThreads, 0, s>>>(g, a, src, bias, dst);
 }
 
 // Split of the (n, p, q) reduction: enough workgroups for ~2 per CU.
@@ -512,6 +579,7 @@ int mn_conv_fwd(const mn_conv2d* g, const void* x, const void* w, const void* bi
       q.aoff[t] = t;
     }
   launch_gather(q, (const float*)w, (const float*)x, (const float*)bias, (float*)y,
+                4ull * g->N * g->C * g->H * g->W, 4ull * g->K * g->C * g->R * g->S,
                 mn_stream(stream));
   return mn_launch_status();
 }
@@ -573,7 +641,8 @@ int mn_conv_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void* dx
       q.osw = g->sW;
       q.lda = lda;
       q.cha = cha;
-      launch_gather(q, a, (const float*)dy, nullptr, (float*)dx, s);
+      launch_gather(q, a, (const float*)dy, nullptr, (float*)dx, 4ull * g->N * g->K * g->P * g->Q,
+                    4ull * g->K * g->C * g->R * g->S, s);
     }
   }
   return mn_launch_status();
