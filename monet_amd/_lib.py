@@ -4,13 +4,16 @@ The library is the only compute path: if it is missing or a call fails the
 caller gets an exception, never a fallback.
 """
 import ctypes
+import os
 from ctypes import (POINTER, Structure, c_char_p, c_double, c_float, c_int, c_int32, c_int64,
                     c_size_t, c_void_p)
 from pathlib import Path
 
 import torch
 
-LIB_PATH = Path(__file__).resolve().parent / "libmonet_hip.so"
+# MONET_HIP_LIBRARY overrides the in-tree build (e.g. to load an instrumented build).
+LIB_PATH = Path(os.environ.get("MONET_HIP_LIBRARY",
+                               Path(__file__).resolve().parent / "libmonet_hip.so"))
 ABI_VERSION = 1
 
 MN_OK, MN_EINVAL, MN_EUNSUPPORTED, MN_ELAUNCH = 0, 1, 2, 3

@@ -19,15 +19,33 @@
 // Operand tiles (BK = 16 deep) are staged through LDS k-major, double buffered:
 // the global loads of tile t+1 are in flight while tile t is multiplied.
 #include "common.h"
+#ifdef MN_TUNING
+#include <cstdlib>
+#endif
 
 namespace mn_conv {
 
 typedef float float16_t __attribute__((ext_vector_type(16)));
 
-constexpr int kThreads = 256;
-constexpr int BM = 128, BN = 128, BK = 16;
-constexpr int kPad = 1;  // LDS row padding (floats)
+constexpr int kThreads = 256;  // 4 wavefronts
+constexpr int BK = 16;         // depth of a staged tile, gather GEMM
+constexpr int WBK = 32;        // depth of a staged tile, backward-weight
+constexpr int kPad = 1;        // LDS row padding (floats)
 constexpr int kMaxTaps = 49;
+
+// Workgroup tile BM x BN computed by WM x WN wavefronts; each wavefront owns
+// TM x TN MFMA tiles of 32 x 32.
+template <int BM_, int BN_, int WM_, int WN_>
+struct Tile {
+  static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_;
+  static constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+  static_assert(WM * WN * 64 == kThreads && TM >= 1 && TN >= 1, "bad tile");
+};
+typedef Tile<128, 128, 2, 2> T128x128;
+typedef Tile<64, 256, 1, 4> T64x256;
+typedef Tile<64, 128, 1, 4> T64x128;
+typedef Tile<128, 64, 4, 1> T128x64;
+typedef Tile<64, 64, 2, 2> T64x64;
 
 // n / d for n < 2^20, d < 4096 (mul = floor(2^32 / d) + 1).
 struct FastDiv {
@@ -41,6 +59,35 @@ static FastDiv make_fastdiv(uint32_t d) {
   f.d = d ? d : 1;
   f.mul = (uint32_t)((1ull << 32) / f.d + 1);
   return f;
+}
+
+// Multiply one staged k-tile (DEPTH deep, k-major in LDS) into the accumulators.
+template <class TL, int DEPTH>
+__device__ __forceinline__ void mma_tile(const float (*As)[TL::BM + kPad],
+                                         const float (*Bs)[TL::BN + kPad], int wm, int wn,
+                                         int lane, float16_t (&acc)[TL::TM][TL::TN]) {
+  const int r = lane & 31, half = lane >> 5;
+  const int arow = wm * (TL::TM * 32) + r, bcol = wn * (TL::TN * 32) + r;
+#pragma unroll
+  for (int ks = 0; ks < DEPTH; ks += 2) {
+    const int k = ks + half;
+    float af[TL::TM], bf[TL::TN];
+#pragma unroll
+    for (int i = 0; i < TL::TM; ++i) af[i] = As[k][arow + 32 * i];
+#pragma unroll
+    for (int j = 0; j < TL::TN; ++j) bf[j] = Bs[k][bcol + 32 * j];
+#pragma unroll
+    for (int i = 0; i < TL::TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TL::TN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bf[j], acc[i][j], 0, 0, 0);
+  }
+}
+
+// Row of accumulator register v within a 32x32 MFMA tile, for this lane
+// (the column is lane % 32).
+__device__ __forceinline__ int acc_row(int v, int lane) {
+  return 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
 }
 
 // One launch of the gather GEMM (forward, or one parity class of backward-data).
@@ -59,64 +106,38 @@ struct Gather {
   int32_t aoff[kMaxTaps];
 };
 
-struct Lds {
-  float a[2][BK][BM + kPad];
-  float b[2][BK][BN + kPad];
-  int tdh[kMaxTaps], tdw[kMaxTaps], taoff[kMaxTaps];
-};
-
-// Wavefront-level multiply of one staged k-tile: wave (wm, wn) owns rows
-// wm*64.. and columns wn*64.. of the workgroup tile.
-__device__ __forceinline__ void mma_tile(const float (*As)[BM + kPad], const float (*Bs)[BN + kPad],
-                                         int wm, int wn, int lane, float16_t (&acc)[2][2]) {
-  const int r = lane & 31, half = lane >> 5;
-#pragma unroll
-  for (int ks = 0; ks < BK; ks += 2) {
-    const int k = ks + half;
-    const float a0 = As[k][wm * 64 + r];
-    const float a1 = As[k][wm * 64 + 32 + r];
-    const float b0 = Bs[k][wn * 64 + r];
-    const float b1 = Bs[k][wn * 64 + 32 + r];
-    acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
-    acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
-    acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
-    acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
-  }
-}
-
-// Row of accumulator register v within a 32x32 MFMA tile, for this lane.
-__device__ __forceinline__ int acc_row(int v, int lane) {
-  return 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-}
-
-// FAST: the source has a multiple of BK channels and every tensor is < 4 GB.
-// Then the reduction index runs tap-major (kk = tap*Cs + ch): a k-tile lies
-// inside one tap, so the window test and the spatial offset are computed once
-// per tile and thread, every address is a 32-bit byte offset = per-thread
-// constant + per-tile scalar, and almost no vector ALU work competes with the
-// matrix cores.  Otherwise (e.g. 3 input channels) kk = ch*T + tap and every
-// element is decomposed on its own.
-template <bool FAST>
+// FAST: the source has a multiple of BK channels.  Then the reduction index
+// runs tap-major (kk = tap*Cs + ch): a k-tile lies inside one tap, so the
+// window test and the spatial offset are computed once per tile and thread,
+// every address is a 32-bit byte offset = per-thread constant + per-tile
+// scalar, and little vector ALU work competes with the matrix cores.
+// Otherwise (e.g. 3 input channels) kk = ch*T + tap and every element is
+// decomposed on its own.  All tensors are < 4 GB (checked by the host).
+template <class TL, bool FAST>
 __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
                                                                const float* __restrict__ a,
                                                                const float* __restrict__ src,
                                                                const float* __restrict__ bias,
                                                                float* __restrict__ dst) {
-  __shared__ Lds lds;
+  constexpr int BM = TL::BM, BN = TL::BN;
+  __shared__ float lds_a[2][BK][BM + kPad];
+  __shared__ float lds_b[2][BK][BN + kPad];
+  __shared__ int tdh[kMaxTaps], tdw[kMaxTaps], taoff[kMaxTaps];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / TL::WN, wn = wave % TL::WN;
   const int m0 = blockIdx.y * BM;
   const uint32_t n0 = blockIdx.x * BN;
   if (tid < g.T) {
-    lds.tdh[tid] = g.dh[tid];
-    lds.tdw[tid] = g.dw[tid];
-    lds.taoff[tid] = g.aoff[tid];
+    tdh[tid] = g.dh[tid];
+    tdw[tid] = g.dw[tid];
+    taoff[tid] = g.aoff[tid];
   }
   __syncthreads();
 
-  // B loader: this thread always fetches column bcol, rows brow0 + 2*i
-  constexpr int kBRows = BN * BK / kThreads, kARows = BM * BK / kThreads;
-  const int bcol = tid & (BN - 1), brow0 = tid / BN;
+  // B loader: this thread always fetches column bcol, rows brow0 + kBStep*i
+  constexpr int kBStep = kThreads / BN, kBRows = BK / kBStep;
+  constexpr int kAStep = kThreads / BK, kARows = BM / kAStep;
+  const int bcol = tid % BN, brow0 = tid / BN;
   const uint32_t col = n0 + bcol;
   const bool col_ok = col < g.ncols;
   int ohs = 0, ows = 0;
@@ -129,92 +150,91 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
     ohs = oh * g.ish;
     ows = ow * g.isw;
   }
-  const size_t srcbase = (size_t)img * g.Cs * g.Hs * g.Ws;
-  // A loader: this thread always fetches k-column ak, rows arow0 + 16*i
-  const int ak = tid & (BK - 1), arow0 = tid / BK;
+  // A loader: this thread always fetches k-column ak, rows arow0 + kAStep*i
+  const int ak = tid % BK, arow0 = tid / BK;
 
-  // FAST: per-thread constant byte offsets
+  // per-thread constant byte offsets
   const uint32_t plane_b = (uint32_t)g.Hs * g.Ws * 4u;
-  const uint32_t pix_b = ((img * (uint32_t)g.Cs * g.Hs + ohs) * (uint32_t)g.Ws + ows) * 4u +
-                         brow0 * plane_b;
+  const uint32_t img_b = img * (uint32_t)g.Cs * plane_b;
+  const uint32_t pix_b = img_b + (uint32_t)(ohs * g.Ws + ows) * 4u + brow0 * plane_b;
   uint32_t am_b[kARows];
   uint32_t am_ok = 0;
-  if (FAST) {
 #pragma unroll
-    for (int i = 0; i < kARows; ++i) {
-      const int m = m0 + arow0 + (kThreads / BK) * i;
-      const bool ok = m < g.M;
-      am_b[i] = ok ? (uint32_t)(((long long)m * g.lda + (long long)ak * g.cha) * 4) : 0u;
-      am_ok |= (ok ? 1u : 0u) << i;
-    }
+  for (int i = 0; i < kARows; ++i) {
+    const int m = m0 + arow0 + kAStep * i;
+    const bool ok = m < g.M;
+    am_b[i] = ok ? (uint32_t)(((long long)m * g.lda + (FAST ? (long long)ak * g.cha : 0)) * 4) : 0u;
+    am_ok |= (ok ? 1u : 0u) << i;
   }
 
+  const char* sp = reinterpret_cast<const char*>(src);
+  const char* ap = reinterpret_cast<const char*>(a);
   float ra[kARows], rb[kBRows];
-  bool b_ok = true;  // FAST: whether rb holds window elements or must be staged as zeros
-  // FAST fetch of the k-tile at (tap t, first channel c0); t and c0 are uniform.
-  // Only issues the loads: masking happens in stage(), after the multiply of the
-  // current tile, so the loads stay in flight behind the matrix instructions.
-  auto fetch_fast = [&](int t, int c0) {
-    const int dh = lds.tdh[t], dw = lds.tdw[t];
+  uint32_t b_ok = 0;  // bit i: rb[i] holds a window element (else it is staged as zero)
+  bool a_ok = true;
+  // Only issues loads: masking happens in stage(), after the multiply of the current
+  // tile, so the loads stay in flight behind the matrix instructions.
+  auto fetch_fast = [&](int t, int c0) {  // t, c0 uniform
+    const int dh = tdh[t], dw = tdw[t];
     const int hh = ohs + dh, ww = ows + dw;
-    b_ok = col_ok && (unsigned)hh < (unsigned)g.Hs && (unsigned)ww < (unsigned)g.Ws;
+    const bool ok = col_ok && (unsigned)hh < (unsigned)g.Hs && (unsigned)ww < (unsigned)g.Ws;
+    b_ok = ok ? 0xFFFFFFFFu : 0u;
     const uint32_t sb = (uint32_t)((((long long)c0 * g.Hs + dh) * g.Ws + dw) * 4);
-    const uint32_t base = b_ok ? pix_b + sb : brow0 * plane_b;
-    const char* sp = reinterpret_cast<const char*>(src);
+    const uint32_t base = ok ? pix_b + sb : brow0 * plane_b;
 #pragma unroll
     for (int i = 0; i < kBRows; ++i)
-      rb[i] = *reinterpret_cast<const float*>(sp + (base + (kThreads / BN) * i * plane_b));
-    const uint32_t sa = (uint32_t)(((long long)c0 * g.cha + lds.taoff[t]) * 4);
-    const char* ap = reinterpret_cast<const char*>(a);
+      rb[i] = *reinterpret_cast<const float*>(sp + (base + kBStep * i * plane_b));
+    const uint32_t sa = (uint32_t)(((long long)c0 * g.cha + taoff[t]) * 4);
 #pragma unroll
     for (int i = 0; i < kARows; ++i) {
       const bool mok = (am_ok >> i) & 1u;
       ra[i] = *reinterpret_cast<const float*>(ap + (am_b[i] + (mok ? sa : 0u)));
     }
   };
-  auto fetch = [&](int k0) {
+  auto fetch_any = [&](int k0) {
+    b_ok = 0;
 #pragma unroll
     for (int i = 0; i < kBRows; ++i) {
-      const uint32_t kk = k0 + brow0 + (kThreads / BN) * i;
-      float v = 0.f;
+      const uint32_t kk = k0 + brow0 + kBStep * i;
+      uint32_t off = 0;
       if (col_ok && kk < (uint32_t)g.Kd) {
         const uint32_t ch = g.divT.div(kk);
         const uint32_t t = kk - ch * g.T;
-        const int hh = ohs + lds.tdh[t], ww = ows + lds.tdw[t];
-        if ((unsigned)hh < (unsigned)g.Hs && (unsigned)ww < (unsigned)g.Ws)
-          v = src[srcbase + ((size_t)ch * g.Hs + hh) * g.Ws + ww];
+        const int hh = ohs + tdh[t], ww = ows + tdw[t];
+        if ((unsigned)hh < (unsigned)g.Hs && (unsigned)ww < (unsigned)g.Ws) {
+          off = img_b + ch * plane_b + (uint32_t)(hh * g.Ws + ww) * 4u;
+          b_ok |= 1u << i;
+        }
       }
-      rb[i] = v;
+      rb[i] = *reinterpret_cast<const float*>(sp + off);
     }
     const uint32_t kk = k0 + ak;
-    uint32_t ch = 0, t = 0;
-    const bool k_ok = kk < (uint32_t)g.Kd;
-    if (k_ok) {
-      ch = g.divT.div(kk);
-      t = kk - ch * g.T;
+    a_ok = kk < (uint32_t)g.Kd;
+    uint32_t koff = 0;
+    if (a_ok) {
+      const uint32_t ch = g.divT.div(kk);
+      koff = (uint32_t)(((long long)ch * g.cha + taoff[kk - ch * g.T]) * 4);
     }
-    const long long koff = k_ok ? (long long)ch * g.cha + lds.taoff[t] : 0;
 #pragma unroll
     for (int i = 0; i < kARows; ++i) {
-      const int m = m0 + arow0 + (kThreads / BK) * i;
-      ra[i] = (k_ok && m < g.M) ? a[(long long)m * g.lda + koff] : 0.f;
+      const bool mok = a_ok && ((am_ok >> i) & 1u);
+      ra[i] = *reinterpret_cast<const float*>(ap + (mok ? am_b[i] + koff : 0u));
     }
   };
   auto stage = [&](int buf) {
 #pragma unroll
     for (int i = 0; i < kBRows; ++i)
-      lds.b[buf][brow0 + (kThreads / BN) * i][bcol] = (!FAST || b_ok) ? rb[i] : 0.f;
+      lds_b[buf][brow0 + kBStep * i][bcol] = ((b_ok >> i) & 1u) ? rb[i] : 0.f;
 #pragma unroll
     for (int i = 0; i < kARows; ++i)
-      lds.a[buf][ak][arow0 + (kThreads / BK) * i] =
-          (!FAST || ((am_ok >> i) & 1u)) ? ra[i] : 0.f;
+      lds_a[buf][ak][arow0 + kAStep * i] = (a_ok && ((am_ok >> i) & 1u)) ? ra[i] : 0.f;
   };
 
-  float16_t acc[2][2];
+  float16_t acc[TL::TM][TL::TN];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < TL::TM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < TL::TN; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
@@ -230,7 +250,7 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
           ++t;
         }
       } else {
-        fetch(kt * BK);
+        fetch_any(kt * BK);
       }
     };
     fetch_next(0);
@@ -239,16 +259,16 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
     for (int kt = 0; kt < ktiles; ++kt) {
       const int buf = kt & 1;
       if (kt + 1 < ktiles) fetch_next(kt + 1);
-      mma_tile(lds.a[buf], lds.b[buf], wm, wn, lane, acc);
+      mma_tile<TL, BK>(lds_a[buf], lds_b[buf], wm, wn, lane, acc);
       if (kt + 1 < ktiles) stage(buf ^ 1);
       __syncthreads();
     }
   }
 
-  // epilogue: lane owns columns (ni*32 + lane%32) and 16 rows per MFMA tile
+  // epilogue: lane owns columns (nj*32 + lane%32) and 16 rows per MFMA tile
 #pragma unroll
-  for (int ni = 0; ni < 2; ++ni) {
-    const uint32_t c = n0 + wn * 64 + ni * 32 + (lane & 31);
+  for (int nj = 0; nj < TL::TN; ++nj) {
+    const uint32_t c = n0 + wn * (TL::TN * 32) + nj * 32 + (lane & 31);
     if (c >= g.ncols) continue;
     const uint32_t n = c / ((uint32_t)g.OH * g.OW);
     const uint32_t rem = c - n * (uint32_t)g.OH * g.OW;
@@ -257,12 +277,12 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
     float* out = dst + (size_t)n * g.M * plane + (size_t)(oh * g.osh + g.oh0) * g.DW +
                  (ow * g.osw + g.ow0);
 #pragma unroll
-    for (int mi = 0; mi < 2; ++mi) {
+    for (int mi = 0; mi < TL::TM; ++mi) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const int m = m0 + wm * 64 + mi * 32 + acc_row(v, lane);
+        const int m = m0 + wm * (TL::TM * 32) + mi * 32 + acc_row(v, lane);
         if (m < g.M) {
-          float r = acc[mi][ni][v];
+          float r = acc[mi][nj][v];
           if (bias) r += bias[m];
           out[(size_t)m * plane] = r;
         }
@@ -273,7 +293,7 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
 
 // ------------------------------------------------------- backward weight --
 // dw[k][c][r][s] = sum over (n, p, q) dy[n,k,p,q] * x[n,c,p*sH + r*dH - pH, q*sW + s*dW - pW]
-// GEMM: rows = k (M = K), columns = (c, r, s) (Ncol = C*R*S), depth = (n, p, q).
+// GEMM: rows = k (M = K), columns = (c, r, s) (ncols = C*R*S), depth = (n, p, q).
 struct WGrad {
   int K, C, R, S, H, W, P, Q, N;
   int sH, sW, pH, pW, dH, dW;
@@ -284,67 +304,59 @@ struct WGrad {
   int mode;             // 0: store, 1: atomicAdd into dw, 2: store partial [z][K][ncols]
 };
 
-constexpr int WBK = 32;  // depth of a staged tile for backward-weight
-
-struct WLds {
-  float a[2][WBK][BM + kPad];
-  float b[2][WBK][BN + kPad];
-};
-
-__device__ __forceinline__ void mma_tile_w(const float (*As)[BM + kPad],
-                                           const float (*Bs)[BN + kPad], int wm, int wn, int lane,
-                                           float16_t (&acc)[2][2]) {
-  const int r = lane & 31, half = lane >> 5;
-#pragma unroll
-  for (int ks = 0; ks < WBK; ks += 2) {
-    const int k = ks + half;
-    const float a0 = As[k][wm * 64 + r];
-    const float a1 = As[k][wm * 64 + 32 + r];
-    const float b0 = Bs[k][wn * 64 + r];
-    const float b1 = Bs[k][wn * 64 + 32 + r];
-    acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
-    acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
-    acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
-    acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
-  }
-}
-
+template <class TL>
 __global__ __launch_bounds__(kThreads) void wgrad_kernel(const WGrad g,
                                                          const float* __restrict__ dy,
                                                          const float* __restrict__ x,
                                                          float* __restrict__ out) {
-  __shared__ WLds lds;
+  constexpr int BM = TL::BM, BN = TL::BN;
+  __shared__ float lds_a[2][WBK][BM + kPad];
+  __shared__ float lds_b[2][WBK][BN + kPad];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / TL::WN, wn = wave % TL::WN;
   const int m0 = blockIdx.y * BM;
   const uint32_t n0 = blockIdx.x * BN;
   const uint32_t PQ = (uint32_t)g.P * g.Q;
 
-  // this thread always fetches depth lane kd = tid % 32 and rows row0 + 8*i of both tiles
-  const int kdl = tid & (WBK - 1), row0 = tid / WBK;
-  constexpr int kRows = BM * WBK / kThreads;  // 16
+  // this thread always fetches depth lane kdl and rows row0 + kStep*i of both tiles
+  constexpr int kStep = kThreads / WBK, kRowsA = BM / kStep, kRowsB = BN / kStep;
+  const int kdl = tid % WBK, row0 = tid / WBK;
 
-  // the (c, r, s) of this thread's 16 B rows never change: keep offset and window shift
-  int bo_h[kRows], bo_w[kRows];
-  uint32_t bo_c[kRows];
+  // A rows: dy offset of row m (bytes), relative to the (n, p, q) of the tile
+  uint32_t am_b[kRowsA];
+  uint32_t am_ok = 0;
 #pragma unroll
-  for (int i = 0; i < kRows; ++i) {
-    const uint32_t cc = n0 + row0 + (kThreads / WBK) * i;
+  for (int i = 0; i < kRowsA; ++i) {
+    const int m = m0 + row0 + kStep * i;
+    const bool ok = m < g.K;
+    am_b[i] = ok ? (uint32_t)m * PQ * 4u : 0u;
+    am_ok |= (ok ? 1u : 0u) << i;
+  }
+  // B rows: the (c, r, s) of a row never changes: byte offset inside an image and window shift
+  uint32_t bo_b[kRowsB];
+  int16_t bo_h[kRowsB], bo_w[kRowsB];
+  uint32_t bo_ok = 0;
+#pragma unroll
+  for (int i = 0; i < kRowsB; ++i) {
+    const uint32_t cc = n0 + row0 + kStep * i;
+    bo_b[i] = 0;
+    bo_h[i] = 0;
+    bo_w[i] = 0;
     if (cc < g.ncols) {
       const uint32_t c = g.divRS.div(cc);
       const uint32_t rs = cc - c * (uint32_t)(g.R * g.S);
       const uint32_t r = g.divS.div(rs), s = rs - r * g.S;
-      bo_c[i] = c;
-      bo_h[i] = (int)r * g.dH - g.pH;
-      bo_w[i] = (int)s * g.dW - g.pW;
-    } else {
-      bo_c[i] = 0xFFFFFFFFu;
-      bo_h[i] = 0;
-      bo_w[i] = 0;
+      bo_h[i] = (int16_t)((int)r * g.dH - g.pH);
+      bo_w[i] = (int16_t)((int)s * g.dW - g.pW);
+      bo_b[i] = (uint32_t)(((int)(c * g.H) + bo_h[i]) * g.W + bo_w[i]) * 4u;
+      bo_ok |= 1u << i;
     }
   }
 
-  float ra[kRows], rb[kRows];
+  const char* dyp = reinterpret_cast<const char*>(dy);
+  const char* xp = reinterpret_cast<const char*>(x);
+  float ra[kRowsA], rb[kRowsB];
+  uint32_t a_mask = 0, b_mask = 0;
   auto fetch = [&](uint32_t d0) {
     const uint32_t d = d0 + kdl;
     const bool d_ok = d < g.depth;
@@ -355,35 +367,37 @@ __global__ __launch_bounds__(kThreads) void wgrad_kernel(const WGrad g,
       p = pq / g.Q;
       q = pq - p * g.Q;
     }
-    const float* dyp = dy + (size_t)n * g.K * PQ + (size_t)p * g.Q + q;
-    const float* xp = x + (size_t)n * g.C * g.H * g.W;
-    const int h0 = (int)p * g.sH, w0 = (int)q * g.sW;
+    const uint32_t abase = ((n * (uint32_t)g.K) * PQ + p * g.Q + q) * 4u;
+    a_mask = d_ok ? am_ok : 0u;
 #pragma unroll
-    for (int i = 0; i < kRows; ++i) {
-      const int m = m0 + row0 + (kThreads / WBK) * i;
-      ra[i] = (d_ok && m < g.K) ? dyp[(size_t)m * PQ] : 0.f;
-      float v = 0.f;
-      if (d_ok && bo_c[i] != 0xFFFFFFFFu) {
-        const int hh = h0 + bo_h[i], ww = w0 + bo_w[i];
-        if ((unsigned)hh < (unsigned)g.H && (unsigned)ww < (unsigned)g.W)
-          v = xp[((size_t)bo_c[i] * g.H + hh) * g.W + ww];
-      }
-      rb[i] = v;
+    for (int i = 0; i < kRowsA; ++i)
+      ra[i] = *reinterpret_cast<const float*>(dyp + (((a_mask >> i) & 1u) ? abase + am_b[i] : 0u));
+    const int h0 = (int)p * g.sH, w0 = (int)q * g.sW;
+    const uint32_t bbase = ((n * (uint32_t)g.C * g.H + h0) * (uint32_t)g.W + w0) * 4u;
+    b_mask = 0;
+#pragma unroll
+    for (int i = 0; i < kRowsB; ++i) {
+      const int hh = h0 + bo_h[i], ww = w0 + bo_w[i];
+      const bool ok = d_ok && ((bo_ok >> i) & 1u) && (unsigned)hh < (unsigned)g.H &&
+                      (unsigned)ww < (unsigned)g.W;
+      b_mask |= (ok ? 1u : 0u) << i;
+      rb[i] = *reinterpret_cast<const float*>(xp + (ok ? bbase + bo_b[i] : 0u));
     }
   };
   auto stage = [&](int buf) {
 #pragma unroll
-    for (int i = 0; i < kRows; ++i) {
-      lds.a[buf][kdl][row0 + (kThreads / WBK) * i] = ra[i];
-      lds.b[buf][kdl][row0 + (kThreads / WBK) * i] = rb[i];
-    }
+    for (int i = 0; i < kRowsA; ++i)
+      lds_a[buf][kdl][row0 + kStep * i] = ((a_mask >> i) & 1u) ? ra[i] : 0.f;
+#pragma unroll
+    for (int i = 0; i < kRowsB; ++i)
+      lds_b[buf][kdl][row0 + kStep * i] = ((b_mask >> i) & 1u) ? rb[i] : 0.f;
   };
 
-  float16_t acc[2][2];
+  float16_t acc[TL::TM][TL::TN];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < TL::TM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < TL::TN; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
@@ -397,7 +411,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_kernel(const WGrad g,
     for (uint32_t kt = t_begin; kt < t_end; ++kt) {
       const int buf = (kt - t_begin) & 1;
       if (kt + 1 < t_end) fetch((kt + 1) * WBK);
-      mma_tile_w(lds.a[buf], lds.b[buf], wm, wn, lane, acc);
+      mma_tile<TL, WBK>(lds_a[buf], lds_b[buf], wm, wn, lane, acc);
       if (kt + 1 < t_end) stage(buf ^ 1);
       __syncthreads();
     }
@@ -406,20 +420,20 @@ __global__ __launch_bounds__(kThreads) void wgrad_kernel(const WGrad g,
   float* base = out;
   if (g.mode == 2) base += (size_t)blockIdx.z * g.K * g.ncols;
 #pragma unroll
-  for (int ni = 0; ni < 2; ++ni) {
-    const uint32_t c = n0 + wn * 64 + ni * 32 + (lane & 31);
+  for (int nj = 0; nj < TL::TN; ++nj) {
+    const uint32_t c = n0 + wn * (TL::TN * 32) + nj * 32 + (lane & 31);
     if (c >= g.ncols) continue;
 #pragma unroll
-    for (int mi = 0; mi < 2; ++mi) {
+    for (int mi = 0; mi < TL::TM; ++mi) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const int m = m0 + wm * 64 + mi * 32 + acc_row(v, lane);
+        const int m = m0 + wm * (TL::TM * 32) + mi * 32 + acc_row(v, lane);
         if (m < g.K) {
           float* o = base + (size_t)m * g.ncols + c;
           if (g.mode == 1)
-            atomicAdd(o, acc[mi][ni][v]);
+            atomicAdd(o, acc[mi][nj][v]);
           else
-            *o = acc[mi][ni][v];
+            *o = acc[mi][nj][v];
         }
       }
     }
@@ -437,9 +451,16 @@ __global__ __launch_bounds__(kThreads) void wgrad_reduce_kernel(const float* __r
   dw[i] = s;
 }
 
+// Clears n floats; float4 stores where the pointer allows.
 __global__ __launch_bounds__(kThreads) void fill_zero_kernel(float* p, size_t n) {
   const size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x;
-  if (i < n) p[i] = 0.f;
+  const size_t n4 = (reinterpret_cast<uintptr_t>(p) & 15) == 0 ? n / 4 : 0;
+  if (i < n4) {
+    const float4_t z = {0.f, 0.f, 0.f, 0.f};
+    reinterpret_cast<float4_t*>(p)[i] = z;
+  }
+  // tail (or everything, if unaligned): grid covers at least n/4 + 1 threads
+  for (size_t j = n4 * 4 + i; j < n; j += (size_t)gridDim.x * kThreads) p[j] = 0.f;
 }
 
 // wt[c][k][r][s] = w[k][c][r][s]
@@ -473,29 +494,80 @@ static int check(const mn_conv2d* g) {
     return MN_EUNSUPPORTED;
   if ((long long)g->N * g->H * g->W >= (1ll << 31) || (long long)g->N * g->P * g->Q >= (1ll << 31))
     return MN_EUNSUPPORTED;
+  // the kernels address every tensor with 32-bit byte offsets
+  const long long lim = 1ll << 30;  // elements
+  if ((long long)g->N * g->C * g->H * g->W >= lim || (long long)g->N * g->K * g->P * g->Q >= lim ||
+      (long long)g->K * g->C * g->R * g->S >= lim)
+    return MN_EUNSUPPORTED;
   return MN_OK;
 }
 
-static void launch_gather(const Gather& g, const float* a, const float* src, const float* bias,
-                          float* dst, unsigned long long src_bytes, unsigned long long a_bytes,
-                          hipStream_t s) {
-  if (g.ncols == 0 || g.M == 0) return;
-  dim3 grid((g.ncols + BN - 1) / BN, (g.M + BM - 1) / BM);
-  const unsigned long long limit = 1ull << 32;
-  const bool fast = g.T > 0 && g.Cs % BK == 0 && src_bytes < limit && a_bytes < limit;
-  if (fast)
-    gather_gemm_kernel<true><<<grid, kThreads, 0, s>>>(g, a, src, bias, dst);
+// Tile choice, from sweeps over the ResNet-50 shapes at batch 184 on MI355X:
+// 64 x 128 is within a few percent of the best tile everywhere (its 6 waves per
+// SIMD hide the staging latency better than the larger tiles' 3), and GEMMs with
+// at most 64 rows want all four wavefronts side by side on the columns.  The
+// element-wise path (channels not a multiple of 16) always takes 64 x 128: the
+// wider tiles spill there.
+static int pick_tile(long long M, long long ncols, bool fast) {
+  (void)ncols;
+  if (!fast) return 2;
+  return M <= 64 ? 1 : 2;
+}
+
+template <class TL>
+static void launch_gather_t(const Gather& g, const float* a, const float* src, const float* bias,
+                            float* dst, hipStream_t s) {
+  dim3 grid((g.ncols + TL::BN - 1) / TL::BN, (g.M + TL::BM - 1) / TL::BM);
+  if (g.T > 0 && g.Cs % BK == 0)
+    gather_gemm_kernel<TL, true><<<grid, kThreads, 0, s>>>(g, a, src, bias, dst);
   else
-    gather_gemm_kernel<false><<<grid, kThreads, 0, s>>>(g, a, src, bias, dst);
+    gather_gemm_kernel<TL, false><<<grid, kThreads, 0, s>>>(g, a, src, bias, dst);
+}
+
+static void launch_gather(const Gather& g, const float* a, const float* src, const float* bias,
+                          float* dst, hipStream_t s, int tile = -1) {
+  if (g.ncols == 0 || g.M == 0) return;
+#ifdef MN_TUNING
+  if (const char* e = getenv("MN_CONV_TILE")) tile = atoi(e);
+#endif
+  if (tile < 0) tile = pick_tile(g.M, g.ncols, g.T > 0 && g.Cs % BK == 0);
+  switch (tile) {
+    case 1: launch_gather_t<T64x256>(g, a, src, bias, dst, s); break;
+    case 2: launch_gather_t<T64x128>(g, a, src, bias, dst, s); break;
+    case 3: launch_gather_t<T128x64>(g, a, src, bias, dst, s); break;
+    case 4: launch_gather_t<T64x64>(g, a, src, bias, dst, s); break;
+    default: launch_gather_t<T128x128>(g, a, src, bias, dst, s); break;
+  }
 }
 
 // Split of the (n, p, q) reduction: enough workgroups for ~2 per CU.
+static int wgrad_tile(const mn_conv2d* g) {
+#ifdef MN_TUNING
+  if (const char* e = getenv("MN_WGRAD_TILE")) return atoi(e);
+#endif
+  // from the same sweeps: 128 x 128 for windows, 128 x 64 for 1x1 filters, 64 rows for K <= 64
+  const long long ncols = (long long)g->C * g->R * g->S;
+  if (g->K <= 64) return ncols <= 64 ? 4 : 2;
+  return (g->R * g->S == 1 || ncols <= 64) ? 3 : 0;
+}
+static void tile_dims(int tile, int* bm, int* bn) {
+  switch (tile) {
+    case 1: *bm = 64; *bn = 256; break;
+    case 2: *bm = 64; *bn = 128; break;
+    case 3: *bm = 128; *bn = 64; break;
+    case 4: *bm = 64; *bn = 64; break;
+    default: *bm = 128; *bn = 128; break;
+  }
+}
+// Split of the (n, p, q) reduction: enough workgroups for ~3 per CU.
 static void wgrad_split(const mn_conv2d* g, int* splits, int* tiles_per_split) {
+  int bm, bn;
+  tile_dims(wgrad_tile(g), &bm, &bn);
   const long long depth = (long long)g->N * g->P * g->Q;
   const long long total_tiles = (depth + WBK - 1) / WBK;
   const long long out_tiles =
-      (((long long)g->C * g->R * g->S + BN - 1) / BN) * (((long long)g->K + BM - 1) / BM);
-  long long want = (512 + out_tiles - 1) / out_tiles;
+      (((long long)g->C * g->R * g->S + bn - 1) / bn) * (((long long)g->K + bm - 1) / bm);
+  long long want = (768 + out_tiles - 1) / out_tiles;
   if (want > total_tiles) want = total_tiles;
   if (want > 256) want = 256;
   if (want < 1) want = 1;
@@ -504,7 +576,6 @@ static void wgrad_split(const mn_conv2d* g, int* splits, int* tiles_per_split) {
   *splits = (int)((total_tiles + *tiles_per_split - 1) / (*tiles_per_split));
   if (*splits < 1) *splits = 1;
 }
-
 
 }  // namespace mn_conv
 
@@ -579,7 +650,6 @@ int mn_conv_fwd(const mn_conv2d* g, const void* x, const void* w, const void* bi
       q.aoff[t] = t;
     }
   launch_gather(q, (const float*)w, (const float*)x, (const float*)bias, (float*)y,
-                4ull * g->N * g->C * g->H * g->W, 4ull * g->K * g->C * g->R * g->S,
                 mn_stream(stream));
   return mn_launch_status();
 }
@@ -606,6 +676,23 @@ int mn_conv_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void* dx
     lda = (long long)g->K * RS;
     cha = RS;
   }
+  // Classes no tap can reach (e.g. 1x1 filters with stride 2) are plain zeros: clear dx once
+  // with full-width stores instead of scattering zeros class by class.
+  bool empty_class = false;
+  for (int ca = 0; ca < g->sH && !empty_class; ++ca) {
+    bool any = false;
+    for (int r = 0; r < g->R; ++r) any |= (r * g->dH) % g->sH == ca;
+    empty_class |= !any;
+  }
+  for (int cb = 0; cb < g->sW && !empty_class; ++cb) {
+    bool any = false;
+    for (int sx = 0; sx < g->S; ++sx) any |= (sx * g->dW) % g->sW == cb;
+    empty_class |= !any;
+  }
+  if (empty_class) {
+    const size_t n = (size_t)g->N * g->C * g->H * g->W;
+    fill_zero_kernel<<<(unsigned)((n / 4 + kThreads) / kThreads), kThreads, 0, s>>>((float*)dx, n);
+  }
   // one dense gather per parity class (a, b) of (h + pH, w + pW) modulo the stride
   for (int ca = 0; ca < g->sH; ++ca) {
     for (int cb = 0; cb < g->sW; ++cb) {
@@ -626,6 +713,7 @@ int mn_conv_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void* dx
           ++T;
         }
       }
+      if (T == 0) continue;  // already cleared above
       q.T = T;
       q.Kd = g->K * T;
       q.divT = make_fastdiv(T);
@@ -641,8 +729,7 @@ int mn_conv_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void* dx
       q.osw = g->sW;
       q.lda = lda;
       q.cha = cha;
-      launch_gather(q, a, (const float*)dy, nullptr, (float*)dx, 4ull * g->N * g->K * g->P * g->Q,
-                    4ull * g->K * g->C * g->R * g->S, s);
+      launch_gather(q, a, (const float*)dy, nullptr, (float*)dx, s);
     }
   }
   return mn_launch_status();
@@ -659,7 +746,7 @@ int mn_conv_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, void* 
   hipStream_t s = mn_stream(stream);
   const size_t nw = (size_t)g->K * g->C * g->R * g->S;
   if (g->N == 0) {
-    fill_zero_kernel<<<(unsigned)((nw + kThreads - 1) / kThreads), kThreads, 0, s>>>((float*)dw, nw);
+    fill_zero_kernel<<<(unsigned)((nw / 4 + kThreads) / kThreads), kThreads, 0, s>>>((float*)dw, nw);
     return mn_launch_status();
   }
   if (!dy || !x) return MN_EINVAL;
@@ -691,14 +778,22 @@ int mn_conv_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, void* 
     q.mode = 0;
   } else if (variant == 0) {
     q.mode = 1;
-    fill_zero_kernel<<<(unsigned)((nw + kThreads - 1) / kThreads), kThreads, 0, s>>>((float*)dw, nw);
+    fill_zero_kernel<<<(unsigned)((nw / 4 + kThreads) / kThreads), kThreads, 0, s>>>((float*)dw, nw);
   } else {
     q.mode = 2;
     if (!ws || ws_bytes < nw * sizeof(float) * splits || !mn_aligned(ws, 4)) return MN_EINVAL;
     out = (float*)ws;
   }
-  dim3 grid((q.ncols + BN - 1) / BN, (g->K + BM - 1) / BM, splits);
-  wgrad_kernel<<<grid, kThreads, 0, s>>>(q, (const float*)dy, (const float*)x, out);
+  const int tile = wgrad_tile(g);
+  int bm, bn;
+  tile_dims(tile, &bm, &bn);
+  dim3 grid((q.ncols + bn - 1) / bn, (g->K + bm - 1) / bm, splits);
+  switch (tile) {
+    case 2: wgrad_kernel<T64x128><<<grid, kThreads, 0, s>>>(q, (const float*)dy, (const float*)x, out); break;
+    case 3: wgrad_kernel<T128x64><<<grid, kThreads, 0, s>>>(q, (const float*)dy, (const float*)x, out); break;
+    case 4: wgrad_kernel<T64x64><<<grid, kThreads, 0, s>>>(q, (const float*)dy, (const float*)x, out); break;
+    default: wgrad_kernel<T128x128><<<grid, kThreads, 0, s>>>(q, (const float*)dy, (const float*)x, out); break;
+  }
   if (q.mode == 2)
     wgrad_reduce_kernel<<<(unsigned)((nw + kThreads - 1) / kThreads), kThreads, 0, s>>>(
         (const float*)ws, (float*)dw, nw, splits);
