@@ -1,0 +1,383 @@
+"""The schedule ILP (reference: monet/cvxpy_solver.py:54-334, restated from the
+clearer monet/gurobi_solver.py:84-271) on scipy's HiGHS MILP solver, because
+neither cvxpy nor CBC / Gurobi are available where this runs.
+
+Binary variables, for timestep t (0 = forward pass, t > 0 = backward node
+V+t-1) and forward solver node i:
+  R[t,i]   i is (re)computed at t            P[t,i]  its output is kept after computing
+  S[t,i]   i is in memory entering t         M[t,p]  backward implementation p runs at t
+  SM[p][t,i] = S[t+1,i] * M[t,p]             IP[t,i] i runs in place
+  RF[c][t,k] convolution k uses kernel variant c at t
+The constraints and the three memory bounds per (t, i) are the reference's.
+Two exact reductions keep the model small enough for HiGHS:
+  * forward nodes that no backward step at or after t can use are never
+    computed or kept at t (R = S = 0 beyond a per-timestep frontier);
+  * SM is only a variable where the backward node has more than one
+    implementation; with a single one it is S itself.
+"""
+import math
+import pickle
+from time import time
+
+import numpy as np
+from scipy import sparse
+from scipy.optimize import Bounds, LinearConstraint, milp
+
+from .solver_info import BwdNode, IntNode, SolverInfo
+
+CPU_GCD_MULTIPLIER = 100
+MEM_GCD_MULTIPLIER = 1
+GB_TO_KB = 1024 * 1024
+Y = 3  # implementation slots per operator
+
+
+class Solution:
+    def __init__(self, r, s, m, rf, ip, p, solve_time, fwd_init, bwd_init, runtime_expected):
+        self.r = r
+        self.s = s
+        self.m = m
+        self.rf = rf
+        self.ip = ip
+        self.p = p
+        self.solve_time = solve_time
+        self.fwd_init = fwd_init
+        self.bwd_init = bwd_init
+        self.runtime_expected = runtime_expected
+
+
+class _Builder:
+    """Accumulates variables, linear rows lo <= a.x <= hi and the objective."""
+
+    def __init__(self):
+        self.nvars = 0
+        self.rows, self.cols, self.vals = [], [], []
+        self.lo, self.hi = [], []
+        self.cost = {}
+
+    def var(self):
+        self.nvars += 1
+        return self.nvars - 1
+
+    def add(self, terms, lo=-np.inf, hi=np.inf, const=0.0):
+        """Row sum(coef * x[var]) + const within [lo, hi]; terms = [(var, coef)];
+        var None is a constant 1."""
+        acc = {}
+        for v, c in terms:
+            if c == 0:
+                continue
+            if v is None:
+                const += c
+            else:
+                acc[v] = acc.get(v, 0.0) + c
+        if not acc:
+            if not (lo - 1e-9 <= const <= hi + 1e-9):
+                raise ValueError("Infeasible: a constraint without variables is violated "
+                                 "(%g not in [%g, %g])" % (const, lo, hi))
+            return
+        r = len(self.lo)
+        for v, c in acc.items():
+            self.rows.append(r)
+            self.cols.append(v)
+            self.vals.append(c)
+        self.lo.append(lo - const)
+        self.hi.append(hi - const)
+
+    def minimise(self, terms):
+        for v, c in terms:
+            if v is not None and c != 0:
+                self.cost[v] = self.cost.get(v, 0.0) + c
+
+
+class Model:
+    def __init__(self, si: SolverInfo, budget, time_limit=86400, solver="HIGHS", ablation=False,
+                 mip_rel_gap=0.01, verbose=False):
+        self.si = si
+        self.budget = budget
+        self.time_limit = time_limit
+        self.solver = solver
+        self.ablation = ablation
+        self.mip_rel_gap = mip_rel_gap
+        self.verbose = verbose
+        n = si.nodes
+        self.ram = np.array([math.ceil(n[i].mem * MEM_GCD_MULTIPLIER / 1024) for i in n])  # KB
+        scale = lambda vals: [math.ceil(v * CPU_GCD_MULTIPLIER) for v in vals]
+        self.cpu = {i: scale(n[i].workspace_compute) for i in n}
+        self.cpu_recompute = {i: scale(n[i].recompute_workspace_compute) for i in n}
+        self.cpu_inplace = {i: scale(n[i].inplace_workspace_compute) for i in n}
+
+    def cmem(self, j, recompute=False, inplace=False):
+        node = self.si.nodes[j]
+        vals = node.inplace_workspace_mem if inplace else (
+            node.recompute_workspace_mem if recompute else node.workspace_mem)
+        return [math.ceil(v * MEM_GCD_MULTIPLIER * 1024) for v in vals]  # MB -> KB
+
+    def local_memory(self, j):
+        return math.ceil(self.si.nodes[j].local_memory * MEM_GCD_MULTIPLIER / 1024)
+
+    def fixed_ram(self, j):
+        return math.ceil(self.si.nodes[j].fixed_mem * MEM_GCD_MULTIPLIER / 1024)
+
+    # ------------------------------------------------------------------ build
+    def _frontier(self, V, T):
+        """lim[t]: largest forward node any backward step at or after t can use."""
+        si = self.si
+        lim = [V - 1] * T
+        for t in range(1, T):
+            b = si.nodes[V + t - 1]
+            f = si.bwd_to_fwd[V + t - 1]
+            top = f + len(si.nodes[f].intermediates)
+            for deps in b.dep_list_fwd:
+                top = max([top] + [d for d in deps if d < V])
+            lim[t] = top
+        for t in range(T - 2, 0, -1):
+            lim[t] = max(lim[t], lim[t + 1])
+        return lim
+
+    def solve(self, out_file=None):
+        si = self.si
+        ram = self.ram
+        budget = self.budget * MEM_GCD_MULTIPLIER * GB_TO_KB
+        V = si.loss + 1
+        T = len(si.nodes) - si.loss
+        lim = self._frontier(V, T)
+        B = _Builder()
+        ONE = None  # the constant-1 pseudo variable
+
+        paths = [1] + [len(si.nodes[V + t - 1].args) for t in range(1, T)]
+        R = [[B.var() if i <= lim[t] else -1 for i in range(V)] for t in range(T)]
+        # S[t][i], t = 0..T; S[0] = 0; S[t+1][i] exists for i <= lim[t]
+        S = [[-1] * V] + [[B.var() if i <= lim[t] else -1 for i in range(V)] for t in range(T)]
+        if si.do_inplace:
+            P = [[B.var() if i <= lim[t] else -1 for i in range(V)] for t in range(T)]
+            IP = [[B.var() if (i in si.inplace_list and i <= lim[t]) else -1 for i in range(V)]
+                  for t in range(T)]
+        else:
+            P = R
+            IP = [[-1] * V for _ in range(T)]
+        M = [[-2] + [-1] * (Y - 1)] + [[B.var() if p < paths[t] else -1 for p in range(Y)]
+                                      for t in range(1, T)]  # -2: the constant 1 (M[0,0])
+        SM = [[[-1] * V for _ in range(T)] for _ in range(Y)]
+        for t in range(T):
+            for p in range(paths[t]):
+                for i in range(V):
+                    if S[t + 1][i] == -1:
+                        continue
+                    SM[p][t][i] = S[t + 1][i] if paths[t] == 1 else B.var()
+        RF = {}
+        n_algos = si.num_conv_algos if si.select_conv_algo else 0
+        for i, k in (si.conv_list.items() if si.select_conv_algo else []):
+            for c in range(n_algos):
+                ok = c < len(self.cpu[i]) and self.cpu[i][c] >= 0
+                for t in range(T):
+                    if not ok:
+                        continue
+                    if i < si.loss:
+                        if R[t][i] != -1:
+                            RF[c, t, k] = B.var()
+                    elif t == i + 1 - V:
+                        RF[c, t, k] = B.var()
+
+        def term(v, coef=1.0):
+            """(var, coef) with -1 = absent (0) and -2 = constant 1."""
+            if v == -1:
+                return (ONE, 0.0)
+            if v == -2:
+                return (ONE, coef)
+            return (v, coef)
+
+        # ---- structural constraints
+        for t in range(T):
+            for i in range(V):
+                if si.do_inplace and R[t][i] != -1:
+                    B.add([term(P[t][i]), term(R[t][i], -1)], hi=0)
+                    if IP[t][i] != -1:
+                        B.add([term(IP[t][i]), term(R[t][i], -1)], hi=0)
+                if S[t + 1][i] != -1:  # stored next only if stored or produced now
+                    B.add([term(S[t + 1][i]), term(S[t][i], -1), term(P[t][i], -1)], hi=0)
+        if si.do_inplace:
+            for v, u in si.inplace_list.items():
+                if isinstance(si.nodes[v], IntNode):
+                    continue
+                for t in range(T):
+                    if IP[t][v] == -1:
+                        continue
+                    B.add([term(P[t][u]), term(R[t][u], -1), term(IP[t][v], 2)], lo=0)
+                    B.add([term(P[t][u]), term(IP[t][v], 2)], hi=2)
+                    B.add([term(S[t + 1][u]), term(IP[t][v], 2)], hi=2)
+        for i in range(V):  # the forward pass computes everything but optional intermediates
+            if not isinstance(si.nodes[i], IntNode):
+                B.add([term(R[0][i])], lo=1, hi=1)
+        for t in range(1, T):
+            B.add([term(M[t][p]) for p in range(Y)], lo=1)
+        for p in range(Y):
+            for t in range(T):
+                if paths[t] == 1:
+                    continue
+                for i in range(V):
+                    sm = SM[p][t][i]
+                    if sm == -1:
+                        continue
+                    B.add([term(sm), term(M[t][p], -1), term(S[t + 1][i], -1)], lo=-1)
+                    B.add([term(sm), term(M[t][p], -1)], hi=0)
+                    B.add([term(sm), term(S[t + 1][i], -1)], hi=0)
+        if self.ablation:
+            for t in range(1, T):
+                for i in range(V):
+                    if R[t][i] != -1:
+                        B.add([term(R[t][i])], hi=0)
+            if si.do_inplace:
+                for v in si.inplace_list:
+                    for t in range(T):
+                        if IP[t][v] != -1:
+                            B.add([term(IP[t][v]), term(R[t][v], -1)], lo=0, hi=0)
+        for (u, v, p) in si.edge_list:
+            if u < V and v < V:
+                for t in range(T):
+                    if R[t][v] != -1:
+                        B.add([term(R[t][v]), term(R[t][u], -1), term(S[t][u], -1)], hi=0)
+            elif u < V <= v:
+                t = v + 1 - V
+                B.add([term(M[t][p]), term(P[t][u], -1), term(S[t + 1][u], -1)], hi=0)
+        for i in range(V):
+            for (_, intid) in si.nodes[i].intermediates:
+                for t in range(T):
+                    if R[t][intid] == -1:
+                        continue
+                    B.add([term(R[t][intid]), term(R[t][i], -1)], hi=0)
+                    if si.do_inplace and i in si.inplace_list:
+                        B.add([term(IP[t][intid]), term(IP[t][i], -1), term(R[t][intid], -1)], lo=-1)
+                        B.add([term(IP[t][intid]), term(IP[t][i], -1)], hi=0)
+        if si.select_conv_algo:
+            for i, k in si.conv_list.items():
+                if i < si.loss:
+                    for t in range(T):
+                        if R[t][i] != -1:
+                            B.add([term(RF.get((c, t, k), -1)) for c in range(n_algos)] +
+                                  [term(R[t][i], -1)], lo=0)
+                else:
+                    t = i + 1 - V
+                    B.add([term(RF.get((c, t, k), -1)) for c in range(n_algos)], lo=1)
+
+        # ---- memory constraints
+        gradm = [(self.local_memory(V + t - 1) if t else 0) + self.fixed_ram(V + t - 2)
+                 for t in range(T)]
+        keep = [[[] for _ in range(T)] for _ in range(Y)]  # keep[p][t] = [i < j in args_p(t)]
+        args_at = [[set(a for a in path if a < V) for path in si.nodes[V + t - 1].args]
+                   for t in range(T)]
+        for j in range(V):
+            local_j = self.local_memory(j)
+            ws_first = self.cmem(j)
+            ws_again = self.cmem(j, recompute=True)
+            ws_inpl = self.cmem(j, inplace=True)
+            sm2_zero = si.nodes[j].local_tensors
+            for t in range(T):
+                jmax = (lim[t - 1] if t else V - 1) + 1  # rows beyond repeat the row at jmax
+                if j > jmax:
+                    continue
+                common = [(ONE, gradm[t])]
+                for p in range(paths[t]):
+                    kp = keep[p][t]
+                    if kp:
+                        common.append(term(M[t][p], float(sum(ram[i] for i in kp))))
+                        common.extend(term(SM[p][t][i], -float(ram[i])) for i in kp)
+                m1 = list(common)
+                m1.extend(term(S[t][i], float(ram[i])) for i in range(j, V))
+                m1.extend(term(S[t + 1][i], float(ram[i])) for i in range(j))
+                B.add(m1, hi=budget)
+                if R[t][j] == -1:
+                    continue
+                m2 = list(common)
+                ws = ws_first if t == 0 else ws_again
+                if si.select_conv_algo and j in si.conv_list:
+                    k = si.conv_list[j]
+                    m2.extend(term(RF.get((c, t, k), -1), float(ws[c])) for c in range(len(ws)))
+                elif si.do_inplace and j in si.inplace_list:
+                    m2.append(term(IP[t][j], float(ws_inpl[0] - ws[0])))
+                    m2.append(term(R[t][j], float(ws[0])))
+                else:
+                    m2.append(term(R[t][j], float(ws[0])))
+                m2.append(term(R[t][j], float(ram[j] + local_j)))
+                m2.extend(term(S[t][i], float(ram[i])) for i in range(j + 1, V)
+                          if i not in sm2_zero)
+                m2.extend(term(S[t + 1][i], float(ram[i])) for i in range(j) if i not in sm2_zero)
+                B.add(m2, hi=budget)
+            for t in range(T):
+                for p in range(paths[t]):
+                    if j in args_at[t][p]:
+                        keep[p][t].append(j)
+        for t in range(1, T):
+            b = V + t - 1
+            node = si.nodes[b]
+            row = [(ONE, self.local_memory(b) + self.fixed_ram(b) + float(ram[b]))]
+            wmem = self.cmem(b)
+            if si.select_conv_algo and b in si.conv_list:
+                k = si.conv_list[b]
+                row.extend(term(RF.get((c, t, k), -1), float(wmem[c])) for c in range(len(wmem)))
+            else:
+                row.extend(term(M[t][p], float(wmem[p])) for p in range(paths[t]))
+            for p in range(paths[t]):
+                row.append(term(M[t][p], float(sum(ram[i] for i in keep[p][t]))))
+                skip = set(node.dep_list_fwd[p])
+                row.extend(term(SM[p][t][i], float(ram[i])) for i in range(V) if i not in skip)
+            B.add(row, hi=budget)
+
+        # ---- objective
+        obj = []
+        conv = si.conv_list if si.select_conv_algo else {}
+        for i in range(V):
+            if i in conv:
+                continue
+            obj.append(term(R[0][i], self.cpu[i][0]))
+            obj.extend(term(R[t][i], self.cpu_recompute[i][0]) for t in range(1, T))
+        conv_node = {k: i for i, k in conv.items()}
+        for (c, t, k), v in RF.items():
+            obj.append((v, self.cpu[conv_node[k]][c]))
+        if si.do_inplace:
+            for i in si.inplace_list:
+                obj.extend(term(IP[t][i], self.cpu_inplace[i][0] - self.cpu[i][0])
+                           for t in range(T))
+        for t in range(T):
+            b = V + t - 1
+            if b in conv:
+                continue
+            obj.extend(term(M[t][p], self.cpu[b][p]) for p in range(Y)
+                       if p < len(self.cpu[b]) and M[t][p] != -1)
+        const_cost = sum(c for v, c in obj if v is None)
+        B.minimise(obj)
+
+        # ---- solve
+        n = B.nvars
+        A = sparse.csr_matrix((B.vals, (B.rows, B.cols)), shape=(len(B.lo), n))
+        cvec = np.zeros(n)
+        for v, c in B.cost.items():
+            cvec[v] = c
+        if self.verbose:
+            print(f"[solver] {n} binaries, {A.shape[0]} rows, {A.nnz} non-zeros")
+        t0 = time()
+        res = milp(cvec, constraints=LinearConstraint(A, np.array(B.lo), np.array(B.hi)),
+                   integrality=np.ones(n), bounds=Bounds(0, 1),
+                   options={"time_limit": float(self.time_limit), "mip_rel_gap": self.mip_rel_gap,
+                            "disp": bool(self.verbose)})
+        solve_time = time() - t0
+        if res.x is None:
+            raise ValueError("Model infeasible" if res.status == 2 else
+                             f"no schedule found: {res.message}")
+        x = np.around(res.x)
+
+        def val(v):
+            return 0.0 if v == -1 else (1.0 if v == -2 else x[v])
+
+        r = np.array([[val(R[t][i]) for i in range(V)] for t in range(T)])
+        pp = np.array([[val(P[t][i]) for i in range(V)] for t in range(T)])
+        s = np.array([[val(S[t][i]) for i in range(V)] for t in range(T + 1)])
+        m = np.array([[val(M[t][p]) for p in range(Y)] for t in range(T)])
+        ip = np.array([[val(IP[t][i]) for i in range(V)] for t in range(T)])
+        rf = np.zeros((T, len(conv), max(n_algos, 1)))
+        for (c, t, k), v in RF.items():
+            rf[t, k, c] = x[v]
+        solution = Solution(r, s, m, rf, ip, pp, solve_time, float("nan"), float("nan"),
+                            float(res.fun + const_cost))
+        if out_file is not None:
+            with open(out_file, 'wb') as f:
+                pickle.dump([si, solution], f)
+        return solution

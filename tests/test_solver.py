@@ -1,0 +1,155 @@
+"""Solver-side host logic on the CPU: graph tracing, solver-graph construction and the
+schedule ILP, with synthetic operator costs instead of GPU measurements."""
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+from monet_amd.graph import ComputeNode, Graph, Input, Param
+from monet_amd.solver import Model
+from monet_amd.solver_info import BwdNode, FwdNode, IntNode, SolverInfo
+
+
+class SmallNet(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.c1 = nn.Conv2d(3, 8, 3, padding=1, bias=False)
+        self.b1 = nn.BatchNorm2d(8)
+        self.r = nn.ReLU(inplace=True)
+        self.mp = nn.MaxPool2d(3, 2, 1)
+        self.c2 = nn.Conv2d(8, 8, 3, padding=1, bias=True)
+        self.b2 = nn.BatchNorm2d(8)
+        self.ap = nn.AdaptiveAvgPool2d((1, 1))
+        self.fc = nn.Linear(8, 5)
+
+    def forward(self, x):
+        x = self.mp(self.r(self.b1(self.c1(x))))
+        y = self.b2(self.c2(x))
+        y += x
+        y = self.r(y)
+        return self.fc(torch.flatten(self.ap(y), 1))
+
+
+def synthetic_cost(si):
+    """Costs proportional to output size: ms = MB, workspace 0; one entry per variant."""
+    def fn(n, op, bwd_op):
+        mb = abs(np.prod(n.shape)) * 4 * si.bs / 1e6
+        conv = si.select_conv_algo and n.op == "aten::_convolution"
+        if conv:
+            nf = op.n_fwd_algos()
+            nb = op.n_bwd_ip_algos() if bwd_op == "ip_grad" else op.n_bwd_wt_algos()
+            return ([0.0] * nf, [0.1 * c for c in range(nb)], []), \
+                   ([mb] * nf, [mb * (1.0 - 0.1 * c) for c in range(nb)], [])
+        if si.do_inplace and hasattr(op, 'inplace'):
+            return ([0.0, 0.0], [0.0], []), ([0.1 * mb, 0.1 * mb], [0.1 * mb], [])
+        if n.op == "aten::batch_norm":
+            return ([0.0], [0.0], [0.0]), ([0.2 * mb], [0.3 * mb], [0.1 * mb])
+        # implementations that keep an intermediate are a bit slower
+        extra = 0.02 * mb if "Binary" in type(op).__name__ or "Indices" in type(op).__name__ else 0
+        return ([0.0], [0.0], []), ([0.1 * mb + extra], [0.1 * mb + extra], [])
+    return fn
+
+
+def build(mode, bs=16):
+    torch.manual_seed(0)
+    g = Graph.create(SmallNet(), (3, 16, 16))
+    si = SolverInfo(bs, "small", mode)
+    si.extract(g, cost_fn=synthetic_cost(si))
+    return g, si
+
+
+def test_graph_trace():
+    g = Graph.create(SmallNet(), (3, 16, 16))
+    kinds = [n.op for n in g.nodes if isinstance(n, ComputeNode)]
+    assert kinds == ["aten::_convolution", "aten::batch_norm", "aten::relu_", "aten::max_pool2d",
+                     "aten::_convolution", "aten::batch_norm", "aten::add_", "aten::relu_",
+                     "aten::adaptive_avg_pool2d", "aten::flatten", "aten::linear"]
+    assert isinstance(g.nodes[0], Input) and g.nodes[0].shape == [-1, 3, 16, 16]
+    conv1 = next(n for n in g.nodes if isinstance(n, ComputeNode))
+    assert conv1.shape == [-1, 8, 16, 16] and conv1.has_backward
+    # the data input carries no gradient, the weight does
+    assert conv1.dependencies[0][1] is False and conv1.dependencies[1][1] is True
+    assert len(conv1.args) == 13 and conv1.args[3].value == [1, 1]
+    assert g._outputs == [len(g.nodes) - 1]
+
+
+def test_solver_graph_structure():
+    g, si = build("inplace_conv_multiway_newnode")
+    fwd = [n for n in si.nodes.values() if isinstance(n, FwdNode) and not isinstance(n, IntNode)]
+    ints = [n for n in si.nodes.values() if isinstance(n, IntNode)]
+    bwd = [n for n in si.nodes.values() if isinstance(n, BwdNode)]
+    assert len(fwd) == 11 + 1          # operators + loss
+    assert len(ints) == 3              # two ReLU masks, one pool index tensor
+    assert len(bwd) == 11 + 2 + 1      # + param_grad nodes of 2 convs and the linear layer
+    assert si.select_conv_algo and si.do_inplace and si.compute_newnode
+    assert si.mode == "conv_multiway_newnode"
+    # intermediate sizes: packed bits / nibbles, per sample, times batch
+    relu_int = si.nodes[si.nodes[2].intermediates[0][1]]
+    assert relu_int.mem == 16 * (8 * 16 * 16) // 8
+    pool_int = si.nodes[si.nodes[si.graph_to_solver[19]].intermediates[0][1]]
+    assert pool_int.mem == 16 * (8 * 8 * 8) // 2
+    # ReLU backward: three implementations with input / output / intermediate dependencies
+    rb = si.nodes[si.fwd_to_bwd[2]]
+    assert [d[0] for d in rb.dep_list_fwd] == [1, 2, si.nodes[2].intermediates[0][1]]
+    # conv: the parameter-gradient node needs the layer input, the input-gradient node does not
+    cb = si.fwd_to_bwd[si.graph_to_solver[20]]
+    assert si.nodes[cb].bwd_op == "ip_grad" and si.nodes[cb - 1].bwd_op == "param_grad"
+    assert si.nodes[cb - 1].dep_list_fwd[0] == [si.graph_to_solver[19]]
+    assert si.nodes[cb].dep_list_fwd[0] == []
+    # in-place candidates: the ReLUs and the residual add (and the ReLU intermediates)
+    ops = sorted(si.nodes[v].op for v in si.inplace_list)
+    assert ops.count("aten::relu_") == 2 and "aten::add_" in ops
+
+
+def peak_of(si, sol):
+    """Memory (KB) of the forward pass under a solution: stored + live tensors, coarse check."""
+    V = si.loss + 1
+    return sum(sol.s[1][i] * si.nodes[i].mem for i in range(V)) / 1024
+
+
+@pytest.mark.parametrize("mode", ["normal", "multiway_newnode", "inplace_conv_multiway_newnode"])
+def test_ilp_unconstrained_stores_and_never_recomputes(mode):
+    g, si = build(mode)
+    sol = Model(si, budget=1.0, time_limit=120, mip_rel_gap=0.0).solve()
+    V, T = si.loss + 1, len(si.nodes) - si.loss
+    assert sol.r.shape == (T, V) and sol.s.shape == (T + 1, V) and sol.m.shape == (T, 3)
+    non_int = [i for i in range(V) if not isinstance(si.nodes[i], IntNode)]
+    assert all(sol.r[0][i] == 1 for i in non_int)
+    # memory is free, so nothing that costs time is recomputed
+    cost = np.array([max(si.nodes[i].workspace_compute, default=0) for i in range(V)])
+    assert (sol.r[1:] * cost).sum() == 0
+    assert (sol.m.sum(axis=1) >= 1).all()
+    if "conv" in mode:
+        # every backward conv step picked exactly one variant, the cheapest one
+        for i, k in si.conv_list.items():
+            if i > si.loss:
+                t = i + 1 - V
+                assert sol.rf[t, k].sum() == 1 and sol.rf[t, k, -1] == 1
+
+
+def test_ilp_budget_forces_cheaper_storage_or_recomputation():
+    g, si = build("inplace_conv_multiway_newnode", bs=64)
+    free = Model(si, budget=1.0, time_limit=120, mip_rel_gap=0.0).solve()
+    # find the smallest budget that is still feasible by bisection on a coarse grid (MB)
+    lo_mb, hi_mb = 0.5, 64.0
+    feasible = None
+    for mb in [48, 32, 24, 16, 12, 8, 6, 4, 3, 2]:
+        try:
+            sol = Model(si, budget=mb / 1024.0, time_limit=120, mip_rel_gap=0.0).solve()
+            feasible = (mb, sol)
+        except ValueError:
+            break
+    assert feasible is not None
+    mb, tight = feasible
+    assert tight.runtime_expected >= free.runtime_expected
+    # a tight budget recomputes something or keeps compact intermediates instead of activations
+    V = si.loss + 1
+    ints = [i for i in range(V) if isinstance(si.nodes[i], IntNode)]
+    assert tight.r[1:].sum() > 0 or tight.s[:, ints].sum() > 0 or tight.ip.sum() > 0
+    assert tight.s[1:].sum() <= free.s[1:].sum() or tight.runtime_expected > free.runtime_expected
+
+
+def test_ilp_infeasible_budget_raises():
+    g, si = build("normal")
+    with pytest.raises(ValueError):
+        Model(si, budget=1e-6, time_limit=60).solve()
