@@ -139,7 +139,7 @@ class _ConvBase(OP):
     def _record(self, input_, weight, bias, stride, padding, dilation, groups):
         self.params = (stride, padding, dilation, groups, input_.shape, weight.shape,
                        [input_.requires_grad, weight.requires_grad,
-                        bias is not None and bias.requires_grad])
+                        bias is not None and bias.requires_grad, bias is not None])
 
     # hooks the two subclasses differ in
     def _fwd_variant(self, *a):
@@ -183,7 +183,7 @@ class _ConvBase(OP):
                 if kind in (1, 2) and weight is not None and do_grad[0]:
                     di = self._bwd_ip_variant(input_shape, grad_output, weight, padding, stride,
                                               dilation, groups)
-            if do_grad[2]:
+            if do_grad[3]:  # bias present: one gradient per tensor argument of the forward
                 return di, dw, db
             return di, dw
 

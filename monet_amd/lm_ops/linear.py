@@ -58,7 +58,7 @@ class LowMemLinear(OP):
 
     def forward(self, input_, weight, bias=None):
         self.params = [input_.requires_grad, weight.requires_grad,
-                       bias is not None and bias.requires_grad]
+                       bias is not None and bias.requires_grad, bias is not None]
         with torch.no_grad():
             return torch.nn.functional.linear(input_, weight, bias)
 
@@ -70,6 +70,6 @@ class LowMemLinear(OP):
                 del stores[0]
             di, dw, db = _linear_backward(self.algorithm // 10, output_grad, input_, weight,
                                           self.params)
-            if self.params[2]:
+            if self.params[3]:  # bias present: one gradient per tensor argument of the forward
                 return di, dw, db
             return di, dw

@@ -53,9 +53,12 @@ class _Builder:
         self.rows, self.cols, self.vals = [], [], []
         self.lo, self.hi = [], []
         self.cost = {}
+        self.continuous = []  # non-negative real variables (the rest are binary)
 
-    def var(self):
+    def var(self, continuous=False):
         self.nvars += 1
+        if continuous:
+            self.continuous.append(self.nvars - 1)
         return self.nvars - 1
 
     def add(self, terms, lo=-np.inf, hi=np.inf, const=0.0):
@@ -90,7 +93,7 @@ class _Builder:
 
 class Model:
     def __init__(self, si: SolverInfo, budget, time_limit=86400, solver="HIGHS", ablation=False,
-                 mip_rel_gap=0.01, verbose=False):
+                 mip_rel_gap=0.01, verbose=False, presolve=True):
         self.si = si
         self.budget = budget
         self.time_limit = time_limit
@@ -98,6 +101,7 @@ class Model:
         self.ablation = ablation
         self.mip_rel_gap = mip_rel_gap
         self.verbose = verbose
+        self.presolve = presolve
         n = si.nodes
         self.ram = np.array([math.ceil(n[i].mem * MEM_GCD_MULTIPLIER / 1024) for i in n])  # KB
         scale = lambda vals: [math.ceil(v * CPU_GCD_MULTIPLIER) for v in vals]
@@ -136,12 +140,19 @@ class Model:
     def solve(self, out_file=None):
         si = self.si
         ram = self.ram
-        budget = self.budget * MEM_GCD_MULTIPLIER * GB_TO_KB
+        # budget None: minimise the peak memory itself (in GB, through a real variable) and
+        # break ties by run time; useful to find out how far a model can be squeezed
+        # With a budget the same variable is simply bounded by it: HiGHS' presolve wrongly
+        # declares the model infeasible when the budget sits in the rows' right-hand sides.
+        find_floor = self.budget is None
         V = si.loss + 1
         T = len(si.nodes) - si.loss
         lim = self._frontier(V, T)
         B = _Builder()
         ONE = None  # the constant-1 pseudo variable
+        peak = [(B.var(continuous=True), -float(GB_TO_KB * MEM_GCD_MULTIPLIER))]
+        peak_limit = np.inf if find_floor else float(self.budget)
+        budget = 0.0
 
         paths = [1] + [len(si.nodes[V + t - 1].args) for t in range(1, T)]
         R = [[B.var() if i <= lim[t] else -1 for i in range(V)] for t in range(T)]
@@ -264,6 +275,9 @@ class Model:
         keep = [[[] for _ in range(T)] for _ in range(Y)]  # keep[p][t] = [i < j in args_p(t)]
         args_at = [[set(a for a in path if a < V) for path in si.nodes[V + t - 1].args]
                    for t in range(T)]
+        # W[t] = sum_{i>=j} S[t,i] ram_i + sum_{i<j} S[t+1,i] ram_i, carried from j to j+1 as a
+        # real variable so that every memory row stays short
+        W = [None] * T
         for j in range(V):
             local_j = self.local_memory(j)
             ws_first = self.cmem(j)
@@ -274,16 +288,21 @@ class Model:
                 jmax = (lim[t - 1] if t else V - 1) + 1  # rows beyond repeat the row at jmax
                 if j > jmax:
                     continue
-                common = [(ONE, gradm[t])]
+                w = B.var(continuous=True)
+                if j == 0:
+                    B.add([(w, -1.0)] + [term(S[t][i], float(ram[i])) for i in range(V)],
+                          lo=0, hi=0)
+                else:
+                    B.add([(w, -1.0), (W[t], 1.0), term(S[t][j - 1], -float(ram[j - 1])),
+                           term(S[t + 1][j - 1], float(ram[j - 1]))], lo=0, hi=0)
+                W[t] = w
+                common = [(ONE, gradm[t]), (w, 1.0)]
                 for p in range(paths[t]):
                     kp = keep[p][t]
                     if kp:
                         common.append(term(M[t][p], float(sum(ram[i] for i in kp))))
                         common.extend(term(SM[p][t][i], -float(ram[i])) for i in kp)
-                m1 = list(common)
-                m1.extend(term(S[t][i], float(ram[i])) for i in range(j, V))
-                m1.extend(term(S[t + 1][i], float(ram[i])) for i in range(j))
-                B.add(m1, hi=budget)
+                B.add(common + peak, hi=budget)
                 if R[t][j] == -1:
                     continue
                 m2 = list(common)
@@ -297,10 +316,10 @@ class Model:
                 else:
                     m2.append(term(R[t][j], float(ws[0])))
                 m2.append(term(R[t][j], float(ram[j] + local_j)))
-                m2.extend(term(S[t][i], float(ram[i])) for i in range(j + 1, V)
-                          if i not in sm2_zero)
-                m2.extend(term(S[t + 1][i], float(ram[i])) for i in range(j) if i not in sm2_zero)
-                B.add(m2, hi=budget)
+                m2.append(term(S[t][j], -float(ram[j])))
+                m2.extend(term(S[t][i] if i > j else S[t + 1][i], -float(ram[i]))
+                          for i in sm2_zero if i != j and i < V)
+                B.add(m2 + peak, hi=budget)
             for t in range(T):
                 for p in range(paths[t]):
                     if j in args_at[t][p]:
@@ -319,7 +338,7 @@ class Model:
                 row.append(term(M[t][p], float(sum(ram[i] for i in keep[p][t]))))
                 skip = set(node.dep_list_fwd[p])
                 row.extend(term(SM[p][t][i], float(ram[i])) for i in range(V) if i not in skip)
-            B.add(row, hi=budget)
+            B.add(row + peak, hi=budget)
 
         # ---- objective
         obj = []
@@ -343,6 +362,10 @@ class Model:
             obj.extend(term(M[t][p], self.cpu[b][p]) for p in range(Y)
                        if p < len(self.cpu[b]) and M[t][p] != -1)
         const_cost = sum(c for v, c in obj if v is None)
+        if find_floor:
+            total = sum(abs(c) for v, c in obj) + 1.0
+            obj = [(v, c / total * 1e-3) for v, c in obj] + [(peak[0][0], 1.0)]
+            const_cost = 0.0
         B.minimise(obj)
 
         # ---- solve
@@ -352,13 +375,18 @@ class Model:
         for v, c in B.cost.items():
             cvec[v] = c
         if self.verbose:
-            print(f"[solver] {n} binaries, {A.shape[0]} rows, {A.nnz} non-zeros")
+            print(f"[solver] {n - len(B.continuous)} binaries, {len(B.continuous)} reals, {A.shape[0]} rows, {A.nnz} non-zeros")
         t0 = time()
+        integrality, upper = np.ones(n), np.ones(n)
+        integrality[B.continuous] = 0
+        upper[B.continuous] = np.inf
+        upper[peak[0][0]] = peak_limit
         res = milp(cvec, constraints=LinearConstraint(A, np.array(B.lo), np.array(B.hi)),
-                   integrality=np.ones(n), bounds=Bounds(0, 1),
+                   integrality=integrality, bounds=Bounds(0, upper),
                    options={"time_limit": float(self.time_limit), "mip_rel_gap": self.mip_rel_gap,
-                            "disp": bool(self.verbose)})
+                            "disp": bool(self.verbose), "presolve": bool(self.presolve)})
         solve_time = time() - t0
+        self.last_problem = (A, np.array(B.lo), np.array(B.hi), res.x)
         if res.x is None:
             raise ValueError("Model infeasible" if res.status == 2 else
                              f"no schedule found: {res.message}")

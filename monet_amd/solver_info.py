@@ -318,6 +318,10 @@ class SolverInfo:
                     self.conv_list[i] = len(self.conv_list)
 
     def get_inplace_info(self):
+        """inplace_list[v] = u: operator v may overwrite its input u, because v is u's last
+        reader in the forward pass.  u is always v's FIRST tensor argument, the one the
+        in-place kernels write (the reference takes the last argument whose last reader is v,
+        solver_info.py:444-456, which for `a += b` can name b while a is overwritten)."""
         self.inplace_list = {}
         if not self.do_inplace:
             return
@@ -325,12 +329,16 @@ class SolverInfo:
             node = self.nodes[v]
             if isinstance(node, IntNode):
                 continue
-            if hasattr(self._impls(node.op)[0], 'inplace'):
-                for u in node.args[0]:
-                    if self.nodes[u].last_used == v:
-                        self.inplace_list[v] = u
-                        for _, intmd in node.intermediates:
-                            self.inplace_list[intmd] = u
+            if not hasattr(self._impls(node.op)[0], 'inplace'):
+                continue
+            first = node.gnode.args[0]
+            if not isinstance(first, ComputeNode.D) or first.index not in self.graph_to_solver:
+                continue
+            u = self.graph_to_solver[first.index]
+            if self.nodes[u].last_used == v:
+                self.inplace_list[v] = u
+                for _, intmd in node.intermediates:
+                    self.inplace_list[intmd] = u
 
     # ---------------------------------------------------------------- profile
     def _cost_file(self):

@@ -1,0 +1,135 @@
+"""Executor parity on the GPU: a model run through a solved schedule must give the
+output and parameter gradients stock autograd gives, at a generous budget (nothing
+recomputed) and at tight ones (recomputation, compact intermediates, in-place)."""
+import copy
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+pytestmark = pytest.mark.gpu
+
+
+class SmallNet(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.c1 = nn.Conv2d(3, 16, 3, padding=1, bias=False)
+        self.b1 = nn.BatchNorm2d(16)
+        self.r = nn.ReLU(inplace=True)
+        self.mp = nn.MaxPool2d(3, 2, 1)
+        self.c2 = nn.Conv2d(16, 16, 3, padding=1, bias=True)
+        self.b2 = nn.BatchNorm2d(16)
+        self.c3 = nn.Conv2d(16, 16, 1, bias=False)
+        self.b3 = nn.BatchNorm2d(16)
+        self.ap = nn.AdaptiveAvgPool2d((1, 1))
+        self.fc = nn.Linear(16, 5)
+
+    def forward(self, x):
+        x = self.mp(self.r(self.b1(self.c1(x))))
+        y = self.r(self.b2(self.c2(x)))
+        y = self.b3(self.c3(y))
+        y += x
+        y = self.r(y)
+        return self.fc(torch.flatten(self.ap(y), 1))
+
+
+def _solve(model, shape, bs, mode, budget_gb, cuda):
+    from monet_amd.graph import Graph
+    from monet_amd.solver import Model
+    from monet_amd.solver_info import SolverInfo
+    graph = Graph.create(copy.deepcopy(model).cpu(), shape)
+    x = torch.randn((bs,) + shape, device=cuda)
+    si = SolverInfo(bs, "test", mode)
+    si.extract(graph, x, *list(model.state_dict(keep_vars=True).values()))
+    sol = Model(si, budget_gb, time_limit=120, mip_rel_gap=0.0).solve()
+    return graph, si, sol
+
+
+def _reference_grads(model, x, gout):
+    ref = copy.deepcopy(model)
+    y = ref(x)
+    y.backward(gout)
+    return y.detach(), {n: p.grad.clone() for n, p in ref.named_parameters()}, ref
+
+
+def _rel(a, b, floor=1e-30):
+    return float((a - b).abs().max() / b.abs().max().clamp_min(floor))
+
+
+@pytest.mark.parametrize("mode", ["normal", "multiway_newnode", "conv_multiway_newnode",
+                                  "inplace_conv_multiway_newnode"])
+def test_schedule_matches_autograd(cuda, mode):
+    from monet_amd.schedule import Schedule
+    torch.manual_seed(0)
+    bs, shape = 32, (3, 32, 32)
+    model = SmallNet().to(cuda).train()
+    graph, si, free = _solve(model, shape, bs, mode, 1.0, cuda)
+    # budgets from generous down to the tightest feasible one
+    peak_mb = None
+    solutions = [("free", free)]
+    from monet_amd.solver import Model
+    for frac in (0.8, 0.65, 0.55, 0.5, 0.45):
+        total = sum(n.mem for i, n in si.nodes.items() if i < si.loss) + si.nodes[si.loss].fixed_mem
+        try:
+            solutions.append(("%.2f" % frac,
+                              Model(si, frac * total / 2**30, time_limit=120, mip_rel_gap=0.0).solve()))
+        except ValueError:
+            break
+    assert len(solutions) >= 2
+    x = torch.randn((bs,) + shape, device=cuda)
+    gout = torch.randn(bs, 5, device=cuda)
+    for name, sol in solutions:
+        print("case", mode, name, "recomputations", int(sol.r[1:].sum()), flush=True)
+        m = copy.deepcopy(model)
+        y_ref, g_ref, ref = _reference_grads(m, x, gout)
+        sched = Schedule(graph, si)
+        sched.init_schedule(sol, si.mode)
+        # a bias in front of a BatchNorm has an exactly zero gradient: both sides then hold
+        # rounding noise only, which a floor tied to the largest gradient lets through
+        floor = 1e-2 * max(float(g.abs().max()) for g in g_ref.values())
+        for step in range(2):  # a second step must not see state of the first
+            for p in m.parameters():
+                p.grad = None
+            if step == 1:
+                m.load_state_dict(model.state_dict())
+            y = sched.forward(x, *list(m.state_dict(keep_vars=True).values()))
+            assert _rel(y, y_ref) < 1e-5
+            sched.backward(gout.clone())
+            for n, p in m.named_parameters():
+                assert p.grad is not None, n
+                assert _rel(p.grad, g_ref[n], floor) < 2e-4, (mode, name, n)
+        # running statistics advanced exactly once per step, like the stock model's
+        assert _rel(m.b1.running_mean, ref.b1.running_mean) < 1e-5
+        assert _rel(m.b3.running_var, ref.b3.running_var) < 1e-5
+
+
+def test_wrapper_trains_like_the_plain_model(cuda, tmp_path):
+    import pickle
+    from monet_amd.monet_wrapper import MONeTWrapper
+    torch.manual_seed(1)
+    bs, shape = 16, (3, 32, 32)
+    model = SmallNet().to(cuda).train()
+    graph, si, sol = _solve(model, shape, bs, "inplace_conv_multiway_newnode", 1.0, cuda)
+    total = sum(n.mem for i, n in si.nodes.items() if i < si.loss) + si.nodes[si.loss].fixed_mem
+    from monet_amd.solver import Model
+    sol = Model(si, 0.6 * total / 2**30, time_limit=120, mip_rel_gap=0.0).solve()
+    path = tmp_path / "solution.pkl"
+    with open(path, "wb") as f:
+        pickle.dump([si, sol], f)
+    plain = copy.deepcopy(model)
+    wrapped = MONeTWrapper(copy.deepcopy(model), str(path), shape).to(cuda)
+    wrapped.train()
+    opt_a = torch.optim.SGD(plain.parameters(), lr=0.05, momentum=0.9)
+    opt_b = torch.optim.SGD(wrapped.parameters(), lr=0.05, momentum=0.9)
+    crit = nn.CrossEntropyLoss()
+    for step in range(3):
+        x = torch.randn((bs,) + shape, device=cuda)
+        t = torch.randint(0, 5, (bs,), device=cuda)
+        la = crit(plain(x), t)
+        opt_a.zero_grad(); la.backward(); opt_a.step()
+        lb = crit(wrapped(x), t)
+        opt_b.zero_grad(); lb.backward(); opt_b.step()
+        assert abs(float(la) - float(lb)) < 1e-4 * max(1.0, abs(float(la)))
+    for (n, pa), pb in zip(plain.named_parameters(), wrapped.model.parameters()):
+        assert _rel(pb, pa, 1e-2) < 1e-3, n
