@@ -29,6 +29,8 @@ CPU_GCD_MULTIPLIER = 100
 MEM_GCD_MULTIPLIER = 1
 GB_TO_KB = 1024 * 1024
 Y = 3  # implementation slots per operator
+EXCESS_PRICE = 1000.0        # objective for exceeding the budget by 100%, in total run times
+EXCESS_TOLERANCE = 1e-6      # accepted excess, as a fraction of the budget
 
 
 class Solution:
@@ -93,7 +95,7 @@ class _Builder:
 
 class Model:
     def __init__(self, si: SolverInfo, budget, time_limit=86400, solver="HIGHS", ablation=False,
-                 mip_rel_gap=0.01, verbose=False, presolve=True):
+                 mip_rel_gap=0.01, verbose=False, presolve=True, recompute_window=None):
         self.si = si
         self.budget = budget
         self.time_limit = time_limit
@@ -102,6 +104,7 @@ class Model:
         self.mip_rel_gap = mip_rel_gap
         self.verbose = verbose
         self.presolve = presolve
+        self.recompute_window = recompute_window
         n = si.nodes
         self.ram = np.array([math.ceil(n[i].mem * MEM_GCD_MULTIPLIER / 1024) for i in n])  # KB
         scale = lambda vals: [math.ceil(v * CPU_GCD_MULTIPLIER) for v in vals]
@@ -142,8 +145,10 @@ class Model:
         ram = self.ram
         # budget None: minimise the peak memory itself (in GB, through a real variable) and
         # break ties by run time; useful to find out how far a model can be squeezed
-        # With a budget the same variable is simply bounded by it: HiGHS' presolve wrongly
-        # declares the model infeasible when the budget sits in the rows' right-hand sides.
+        # With a budget, what the peak exceeds it by is a second real variable that the
+        # objective prices above any possible gain in run time, and a solution that still
+        # exceeds the budget is reported as infeasible.  (A hard bound would be the obvious
+        # statement, but HiGHS 1.8 presolve then declares feasible models infeasible.)
         find_floor = self.budget is None
         V = si.loss + 1
         T = len(si.nodes) - si.loss
@@ -151,29 +156,48 @@ class Model:
         B = _Builder()
         ONE = None  # the constant-1 pseudo variable
         peak = [(B.var(continuous=True), -float(GB_TO_KB * MEM_GCD_MULTIPLIER))]
-        peak_limit = np.inf if find_floor else float(self.budget)
         budget = 0.0
+        excess = None
+        if not find_floor:
+            excess = B.var(continuous=True)
+            B.add([(peak[0][0], 1.0), (excess, -1.0)], hi=float(self.budget))
 
         paths = [1] + [len(si.nodes[V + t - 1].args) for t in range(1, T)]
-        R = [[B.var() if i <= lim[t] else -1 for i in range(V)] for t in range(T)]
+        # Optional restriction: a backward step may only recompute forward nodes at most
+        # `recompute_window` positions before its own operator.  A tensor below the window
+        # cannot be produced, so it is either kept until the window reaches it or dropped right
+        # after the forward pass (dropping later never helps): its S is one variable until then.
+        lo_at = [0] * T
+        if self.recompute_window is not None:
+            lo_at = [0] + [max(0, si.bwd_to_fwd[V + t - 1] - self.recompute_window)
+                           for t in range(1, T)]
+
+        def active(t, i):
+            return lo_at[t] <= i <= lim[t]
+
+        R = [[B.var() if active(t, i) else -1 for i in range(V)] for t in range(T)]
         # S[t][i], t = 0..T; S[0] = 0; S[t+1][i] exists for i <= lim[t]
-        S = [[-1] * V] + [[B.var() if i <= lim[t] else -1 for i in range(V)] for t in range(T)]
+        S = [[-1] * V]
+        for t in range(T):
+            S.append([(B.var() if active(t, i) else S[t][i]) if i <= lim[t] else -1
+                      for i in range(V)])
         if si.do_inplace:
-            P = [[B.var() if i <= lim[t] else -1 for i in range(V)] for t in range(T)]
-            IP = [[B.var() if (i in si.inplace_list and i <= lim[t]) else -1 for i in range(V)]
+            P = [[B.var() if active(t, i) else -1 for i in range(V)] for t in range(T)]
+            IP = [[B.var() if (i in si.inplace_list and active(t, i)) else -1 for i in range(V)]
                   for t in range(T)]
         else:
             P = R
             IP = [[-1] * V for _ in range(T)]
         M = [[-2] + [-1] * (Y - 1)] + [[B.var() if p < paths[t] else -1 for p in range(Y)]
                                       for t in range(1, T)]  # -2: the constant 1 (M[0,0])
+        # the product S[t+1,i] * M[t,p] is only ever needed for the forward tensors i that
+        # implementation p of the backward step reads (see the memory rows below)
         SM = [[[-1] * V for _ in range(T)] for _ in range(Y)]
         for t in range(T):
             for p in range(paths[t]):
-                for i in range(V):
-                    if S[t + 1][i] == -1:
-                        continue
-                    SM[p][t][i] = S[t + 1][i] if paths[t] == 1 else B.var()
+                for i in (a for a in si.nodes[V + t - 1].args[p] if a < V):
+                    if S[t + 1][i] != -1:
+                        SM[p][t][i] = S[t + 1][i] if paths[t] == 1 else B.var()
         RF = {}
         n_algos = si.num_conv_algos if si.select_conv_algo else 0
         for i, k in (si.conv_list.items() if si.select_conv_algo else []):
@@ -219,7 +243,7 @@ class Model:
             if not isinstance(si.nodes[i], IntNode):
                 B.add([term(R[0][i])], lo=1, hi=1)
         for t in range(1, T):
-            B.add([term(M[t][p]) for p in range(Y)], lo=1)
+            B.add([term(M[t][p]) for p in range(Y)], lo=1, hi=1)  # exactly one implementation
         for p in range(Y):
             for t in range(T):
                 if paths[t] == 1:
@@ -288,21 +312,24 @@ class Model:
                 jmax = (lim[t - 1] if t else V - 1) + 1  # rows beyond repeat the row at jmax
                 if j > jmax:
                     continue
-                w = B.var(continuous=True)
-                if j == 0:
-                    B.add([(w, -1.0)] + [term(S[t][i], float(ram[i])) for i in range(V)],
-                          lo=0, hi=0)
-                else:
-                    B.add([(w, -1.0), (W[t], 1.0), term(S[t][j - 1], -float(ram[j - 1])),
-                           term(S[t + 1][j - 1], float(ram[j - 1]))], lo=0, hi=0)
-                W[t] = w
-                common = [(ONE, gradm[t]), (w, 1.0)]
+                same = j > 0 and S[t][j - 1] == S[t + 1][j - 1]
+                if not same:
+                    w = B.var(continuous=True)
+                    if j == 0:
+                        B.add([(w, -1.0)] + [term(S[t][i], float(ram[i])) for i in range(V)],
+                              lo=0, hi=0)
+                    else:
+                        B.add([(w, -1.0), (W[t], 1.0), term(S[t][j - 1], -float(ram[j - 1])),
+                               term(S[t + 1][j - 1], float(ram[j - 1]))], lo=0, hi=0)
+                    W[t] = w
+                common = [(ONE, gradm[t]), (W[t], 1.0)]
                 for p in range(paths[t]):
                     kp = keep[p][t]
                     if kp:
                         common.append(term(M[t][p], float(sum(ram[i] for i in kp))))
                         common.extend(term(SM[p][t][i], -float(ram[i])) for i in kp)
-                B.add(common + peak, hi=budget)
+                if not (same and all(j - 1 not in a for a in args_at[t])):
+                    B.add(common + peak, hi=budget)  # else: the row written for j - 1
                 if R[t][j] == -1:
                     continue
                 m2 = list(common)
@@ -336,8 +363,9 @@ class Model:
                 row.extend(term(M[t][p], float(wmem[p])) for p in range(paths[t]))
             for p in range(paths[t]):
                 row.append(term(M[t][p], float(sum(ram[i] for i in keep[p][t]))))
-                skip = set(node.dep_list_fwd[p])
-                row.extend(term(SM[p][t][i], float(ram[i])) for i in range(V) if i not in skip)
+                # sum over i not read by p of S[t+1,i] * M[t,p], using sum_p M[t,p] = 1
+                row.extend(term(SM[p][t][i], -float(ram[i])) for i in node.dep_list_fwd[p] if i < V)
+            row.extend(term(S[t + 1][i], float(ram[i])) for i in range(V))
             B.add(row + peak, hi=budget)
 
         # ---- objective
@@ -364,8 +392,13 @@ class Model:
         const_cost = sum(c for v, c in obj if v is None)
         if find_floor:
             total = sum(abs(c) for v, c in obj) + 1.0
-            obj = [(v, c / total * 1e-3) for v, c in obj] + [(peak[0][0], 1.0)]
+            # run time only breaks ties: all of it weighs 1e-4 of the activations' size
+            tie = 1e-4 * float(sum(ram[:V])) / (GB_TO_KB * MEM_GCD_MULTIPLIER)
+            obj = [(v, c / total * tie) for v, c in obj] + [(peak[0][0], 1.0)]
             const_cost = 0.0
+        else:
+            total = sum(abs(c) for v, c in obj) + 1.0
+            obj = obj + [(excess, EXCESS_PRICE * total / float(self.budget))]
         B.minimise(obj)
 
         # ---- solve
@@ -380,7 +413,6 @@ class Model:
         integrality, upper = np.ones(n), np.ones(n)
         integrality[B.continuous] = 0
         upper[B.continuous] = np.inf
-        upper[peak[0][0]] = peak_limit
         res = milp(cvec, constraints=LinearConstraint(A, np.array(B.lo), np.array(B.hi)),
                    integrality=integrality, bounds=Bounds(0, upper),
                    options={"time_limit": float(self.time_limit), "mip_rel_gap": self.mip_rel_gap,
@@ -390,6 +422,9 @@ class Model:
         if res.x is None:
             raise ValueError("Model infeasible" if res.status == 2 else
                              f"no schedule found: {res.message}")
+        if excess is not None and res.x[excess] > EXCESS_TOLERANCE * self.budget:
+            raise ValueError("Model infeasible: the cheapest schedule found needs %.3f GB, budget "
+                             "%.3f GB" % (self.budget + res.x[excess], self.budget))
         x = np.around(res.x)
 
         def val(v):

@@ -176,3 +176,29 @@ def test_compiled_plan_is_consistent_and_within_budget(mode):
         assert peak <= mb * 2**20 * 1.001, (mode, mb, peak / 2**20)
         seen += 1
     assert seen >= 5
+
+
+def test_recompute_window_is_a_restriction_of_the_exact_model():
+    """The windowed model must stay feasible where the exact one is and can only cost more."""
+    g, si = build("multiway_newnode", bs=64)
+    for mb in (2.4, 2.0, 1.7):
+        exact = Model(si, budget=mb / 1024.0, time_limit=120, mip_rel_gap=0.0).solve()
+        windowed = Model(si, budget=mb / 1024.0, time_limit=120, mip_rel_gap=0.0,
+                         recompute_window=4).solve()
+        assert windowed.runtime_expected >= exact.runtime_expected
+        sched = Schedule(g, si)
+        sched.init_schedule(windowed, si.mode)
+        peak, _ = replay(sched, 64)
+        assert peak <= mb * 2**20 * 1.001
+        # nothing further than the window below the step's own operator is recomputed
+        V = si.loss + 1
+        for t in range(1, windowed.r.shape[0]):
+            f = si.bwd_to_fwd[V + t - 1]
+            assert windowed.r[t][:max(0, f - 4)].sum() == 0
+
+
+def test_peak_minimisation_finds_the_floor():
+    g, si = build("multiway_newnode", bs=64)
+    floor = Model(si, budget=None, time_limit=120, mip_rel_gap=0.0).solve()
+    gb = floor.runtime_expected  # objective = peak in GB (+ a negligible run-time tie-break)
+    assert 1.6 / 1024 < gb < 1.7 / 1024
