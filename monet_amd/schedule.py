@@ -383,3 +383,100 @@ def create_schedule(model, sol_file, input_shape=(3, 224, 224)):
     schedule = Schedule(graph, solver_info)
     schedule.init_schedule(solution, solver_info.mode)
     return schedule
+
+
+def _timed_steps(step, warmup, iters):
+    """Mean ms per call of `step` and the peak allocation (MB) over the timed calls."""
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        step()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / iters, torch.cuda.max_memory_allocated() / 2**20
+
+
+def main(argv=None):
+    """`python -m monet_amd.schedule MODEL BATCH_SIZE BUDGET MODE SOLVER --solution_file F
+    (--check_runtime | --check_diff | --run_bs)` (reference: monet/schedule.py:348-517)."""
+    import argparse
+
+    from . import config
+    from .models import build_model
+
+    parser = argparse.ArgumentParser()
+    parser.add_argument('model')
+    parser.add_argument('bs', type=int)
+    parser.add_argument('budget', type=float)
+    parser.add_argument('mode')
+    parser.add_argument('solver', nargs='?', default="HIGHS")
+    parser.add_argument("--solution_file", type=str, required=True)
+    parser.add_argument("--check_runtime", action="store_true",
+                        help="time the schedule (and, with --original, stock autograd)")
+    parser.add_argument("--original", action="store_true")
+    parser.add_argument("--run_bs", action="store_true", help="one step, report peak memory")
+    parser.add_argument("--check_diff", action="store_true",
+                        help="compare output and gradients with stock autograd")
+    parser.add_argument("--warmup", type=int, default=10)
+    parser.add_argument("--iters", type=int, default=20)
+    args = parser.parse_args(argv)
+
+    config.budget = args.budget
+    model, input_shape, model_name = build_model(args.model)
+    if args.check_diff:
+        disable_dropout(model)
+    graph = Graph.create(model, input_shape=input_shape)
+    model.cuda()
+    si, solution = load_solution(args.solution_file)
+    schedule = Schedule(graph, si)
+    schedule.init_schedule(solution, si.mode)
+    input_ = torch.randn((args.bs,) + tuple(input_shape)).cuda()
+    state = lambda: list(model.state_dict(keep_vars=True).values())
+
+    def monet_step():
+        out = schedule.forward(input_, *state())
+        schedule.backward(-torch.ones_like(out))
+        for v in model.parameters():
+            v.grad = None
+
+    if args.check_runtime:
+        ms, mb = _timed_steps(monet_step, args.warmup, args.iters)
+        print("monet: %f ms avg, %8.2f MB" % (ms, mb))
+        if args.original:
+            def plain_step():
+                model(input_).sum().backward()
+                for v in model.parameters():
+                    v.grad = None
+            schedule = None
+            torch.cuda.empty_cache()
+            ms0, mb0 = _timed_steps(plain_step, args.warmup, args.iters)
+            print("original: %f ms avg, %8.2f MB" % (ms0, mb0))
+    elif args.check_diff:
+        ref = copy.deepcopy(model)
+        y0 = ref(input_)
+        y0.sum().backward()
+        y1 = schedule.forward(input_, *state())
+        print('Forward mean absolute difference', float((y0 - y1).abs().mean()))
+        schedule.backward(torch.ones_like(y1))
+        worst = 0.0
+        for (name, p), q in zip(model.named_parameters(), ref.parameters()):
+            rel = float((p.grad - q.grad).abs().max() / q.grad.abs().max().clamp_min(1e-12))
+            worst = max(worst, rel)
+            print("%.3e %s %s" % (rel, name, tuple(p.shape)))
+        print("largest relative gradient difference %.3e" % worst)
+    elif args.run_bs:
+        torch.cuda.reset_peak_memory_stats()
+        from time import time
+        t0 = time()
+        monet_step()
+        torch.cuda.synchronize()
+        print("Ran batch %d with peak memory %8.2fM, %fs" % (
+            args.bs, torch.cuda.max_memory_allocated() / 2**20, time() - t0))
+
+
+if __name__ == '__main__':
+    main()

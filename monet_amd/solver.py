@@ -430,12 +430,14 @@ class Model:
         def val(v):
             return 0.0 if v == -1 else (1.0 if v == -2 else x[v])
 
-        r = np.array([[val(R[t][i]) for i in range(V)] for t in range(T)])
-        pp = np.array([[val(P[t][i]) for i in range(V)] for t in range(T)])
-        s = np.array([[val(S[t][i]) for i in range(V)] for t in range(T + 1)])
-        m = np.array([[val(M[t][p]) for p in range(Y)] for t in range(T)])
-        ip = np.array([[val(IP[t][i]) for i in range(V)] for t in range(T)])
-        rf = np.zeros((T, len(conv), max(n_algos, 1)))
+        # 0/1 tables as bytes: a ResNet-50 solution stays a few hundred KB on disk
+        table = lambda rows: np.array(rows, dtype=np.uint8)
+        r = table([[val(R[t][i]) for i in range(V)] for t in range(T)])
+        pp = table([[val(P[t][i]) for i in range(V)] for t in range(T)])
+        s = table([[val(S[t][i]) for i in range(V)] for t in range(T + 1)])
+        m = table([[val(M[t][p]) for p in range(Y)] for t in range(T)])
+        ip = table([[val(IP[t][i]) for i in range(V)] for t in range(T)])
+        rf = np.zeros((T, len(conv), max(n_algos, 1)), dtype=np.uint8)
         for (c, t, k), v in RF.items():
             rf[t, k, c] = x[v]
         solution = Solution(r, s, m, rf, ip, pp, solve_time, float("nan"), float("nan"),
@@ -444,3 +446,70 @@ class Model:
             with open(out_file, 'wb') as f:
                 pickle.dump([si, solution], f)
         return solution
+
+
+def solution_file_name(model_name, bs, mode, budget):
+    return "solution_%s_%d_%s_%.2f.pkl" % (model_name, bs, mode, budget)
+
+
+def main(argv=None):
+    """`python -m monet_amd.solver MODEL BATCH_SIZE BUDGET MODE SOLVER [--time_limit S]`
+    (reference: monet/cvxpy_solver.py:336-384).  Profiling needs the GPU, solving does not:
+    `--profile_only` stops after writing the profiled solver info to --data_dir, `--si_file`
+    solves from such a file on a machine without a GPU."""
+    import argparse
+
+    import torch
+
+    from .graph import Graph
+    from .models import build_model
+
+    parser = argparse.ArgumentParser()
+    parser.add_argument('model')
+    parser.add_argument('bs', type=int)
+    parser.add_argument('budget', type=float, help="memory budget in GB")
+    parser.add_argument('mode')
+    parser.add_argument('solver', nargs='?', default="HIGHS")
+    parser.add_argument("--ablation", action="store_true", help="no recomputation")
+    parser.add_argument("--time_limit", default=86400, type=int, help="solver time limit, seconds")
+    parser.add_argument("--gap", default=0.01, type=float, help="relative optimality gap")
+    parser.add_argument("--window", default=None, type=int,
+                        help="only recompute forward nodes this close below the running "
+                             "backward step (smaller model, possibly costlier schedule)")
+    parser.add_argument("--data_dir", default="data", help="where profiles and solutions go")
+    parser.add_argument("--si_file", default="", help="profiled solver info to solve from")
+    parser.add_argument("--profile_only", action="store_true")
+    parser.add_argument("--verbose", action="store_true")
+    args = parser.parse_args(argv)
+
+    from pathlib import Path
+    Path(args.data_dir).mkdir(parents=True, exist_ok=True)
+    if args.si_file:
+        with open(args.si_file, 'rb') as f:
+            si = pickle.load(f)
+        model_name = si.model_name
+    else:
+        model, input_shape, model_name = build_model(args.model)
+        graph = Graph.create(model, input_shape=input_shape)
+        model.cuda()
+        input_ = torch.randn([args.bs, *input_shape]).cuda()
+        si = SolverInfo(args.bs, model_name=model_name, mode=args.mode, data_dir=args.data_dir)
+        si.extract(graph, input_, *list(model.state_dict(keep_vars=True).values()))
+        print("profiled %d solver nodes -> %s" % (len(si.nodes), args.data_dir))
+        if args.profile_only:
+            return None
+    print("Memory budget", args.budget, "GB; batch size", si.bs, "; model", model_name,
+          "; mode", args.mode)
+    solver_model = Model(si, args.budget, args.time_limit, args.solver, args.ablation,
+                         mip_rel_gap=args.gap, verbose=args.verbose, recompute_window=args.window)
+    out = Path(args.data_dir) / solution_file_name(model_name, si.bs, args.mode, args.budget)
+    solution = solver_model.solve(out_file=str(out))
+    print("solved in %.1f s, expected run time %.2f ms -> %s" % (
+        solution.solve_time, solution.runtime_expected / CPU_GCD_MULTIPLIER, out))
+    return solution
+
+
+if __name__ == '__main__':
+    # run the module under its real name, so that pickles refer to monet_amd.solver.Solution
+    from monet_amd.solver import main as _main
+    _main()

@@ -133,3 +133,56 @@ def test_wrapper_trains_like_the_plain_model(cuda, tmp_path):
         assert abs(float(la) - float(lb)) < 1e-4 * max(1.0, abs(float(la)))
     for (n, pa), pb in zip(plain.named_parameters(), wrapped.model.parameters()):
         assert _rel(pb, pa, 1e-2) < 1e-3, n
+
+
+def test_bottleneck_resnet_against_float64(cuda):
+    """A residual network under a tight schedule (recomputation, 1-bit masks, in-place ops,
+    kernel-variant choice).  fp32 training of a deep randomly initialised network is
+    ill-conditioned, so both the schedule and stock fp32 autograd are measured against
+    float64 autograd: the schedule may not be further from it than stock fp32 is, within a
+    factor that covers the run-to-run spread of such errors."""
+    from monet_amd.models.resnet import Bottleneck, ResNet
+    from monet_amd.schedule import Schedule
+    from monet_amd.solver import Model
+    torch.manual_seed(0)
+    bs, shape = 16, (3, 64, 64)
+    model = ResNet(Bottleneck, [2, 1, 1, 1], num_classes=10).to(cuda).train()
+    graph, si, free = _solve(model, shape, bs, "inplace_conv_multiway_newnode", 1.0, cuda)
+    total = sum(n.mem for i, n in si.nodes.items() if i < si.loss) + si.nodes[si.loss].fixed_mem
+    sol = None
+    for frac in (0.75, 0.9):
+        print("solving at %.2f of the unconstrained footprint" % frac, flush=True)
+        try:
+            sol = Model(si, frac * total / 2**30, time_limit=40, mip_rel_gap=0.05,
+                        recompute_window=12).solve()
+            break
+        except ValueError:
+            continue
+    assert sol is not None
+    assert sol.r[1:].sum() > 0 or sol.ip.sum() > 0
+    x = torch.randn((bs,) + shape, device=cuda)
+    target = torch.randint(0, 10, (bs,), device=cuda)
+    crit = nn.CrossEntropyLoss()
+
+    def stock(m, xin):
+        m.zero_grad()
+        crit(m(xin), target).backward()
+        return {n: p.grad.detach().double() for n, p in m.named_parameters()}
+
+    g64 = stock(copy.deepcopy(model).double(), x.double())
+    g32 = stock(copy.deepcopy(model), x)
+
+    m = copy.deepcopy(model)
+    sched = Schedule(graph, si)
+    sched.init_schedule(sol, si.mode)
+    y = sched.forward(x, *list(m.state_dict(keep_vars=True).values())).requires_grad_(True)
+    crit(y, target).backward()
+    sched.backward(y.grad)
+    worst_ours = worst_stock = 0.0
+    for n, p in m.named_parameters():
+        scale = g64[n].abs().max().clamp_min(1e-12)
+        worst_ours = max(worst_ours, float((p.grad.double() - g64[n]).abs().max() / scale))
+        worst_stock = max(worst_stock, float((g32[n] - g64[n]).abs().max() / scale))
+    print("largest relative error against float64: schedule %.3e, stock fp32 %.3e" % (
+        worst_ours, worst_stock), flush=True)
+    assert worst_ours <= 4 * worst_stock + 1e-5
