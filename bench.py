@@ -138,12 +138,79 @@ def cpu_baseline(sample_n=23, reps=5):
                       f"CPU ops (torch {torch.__version__}), 1 warm-up + median of {reps}"}
 
 
+E2E_MODE = "inplace_conv_multiway_newnode"
+E2E_BS = 184
+
+
+def _train_ms(model, x, target, iters, warmup):
+    """ms per SGD step (forward, cross entropy, backward, momentum update) and peak MB."""
+    import torch
+    opt = torch.optim.SGD(model.parameters(), lr=0.01, momentum=0.9)
+    crit = torch.nn.CrossEntropyLoss()
+
+    def step():
+        opt.zero_grad(set_to_none=True)
+        crit(model(x), target).backward()
+        opt.step()
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    t0 = torch.cuda.Event(enable_timing=True)
+    t1 = torch.cuda.Event(enable_timing=True)
+    t0.record()
+    for _ in range(iters):
+        step()
+    t1.record()
+    torch.cuda.synchronize()
+    return t0.elapsed_time(t1) / iters, torch.cuda.max_memory_allocated() / 2**20
+
+
+def end_to_end(iters=10, warmup=3):
+    """ResNet-50 (torchvision topology, random init), batch 184, fp32 SGD steps: under the
+    solved 10 GB and 6 GB schedules, under the unconstrained schedule (same kernels, nothing
+    recomputed) and with stock PyTorch autograd.  Overhead is against the unconstrained run."""
+    import torch
+
+    from monet_amd.models import resnet50
+    from monet_amd.monet_wrapper import MONeTWrapper
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    x = torch.randn(E2E_BS, 3, 224, 224, device=dev)
+    target = torch.randint(0, 1000, (E2E_BS,), device=dev)
+    res = {"model": "resnet50", "batch": E2E_BS, "dtype": "f32", "unit": "images/s",
+           "step": "forward + cross entropy + backward + SGD momentum update"}
+    base = None
+    for budget in (100, 10, 6):
+        sol = ROOT / "data" / ("solution_resnet50_%d_%s_%.2f.pkl" % (E2E_BS, E2E_MODE, budget))
+        if not sol.exists():
+            continue
+        model = MONeTWrapper(resnet50(), str(sol), (3, 224, 224)).to(dev)
+        model.train()
+        ms, mb = _train_ms(model, x, target, iters, warmup)
+        key = "unconstrained" if budget == 100 else "budget_%dGB" % budget
+        res[key] = {"images_per_s": round(E2E_BS / ms * 1e3, 1), "ms_per_step": round(ms, 2),
+                    "peak_MB": round(mb, 1)}
+        if budget == 100:
+            base = ms
+        elif base:
+            res[key]["overhead_vs_unconstrained"] = round(ms / base - 1.0, 4)
+        del model
+        torch.cuda.empty_cache()
+    model = resnet50().to(dev).train()
+    ms, mb = _train_ms(model, x, target, iters, warmup)
+    res["stock_pytorch"] = {"images_per_s": round(E2E_BS / ms * 1e3, 1),
+                            "ms_per_step": round(ms, 2), "peak_MB": round(mb, 1)}
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-end-to-end", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
@@ -171,6 +238,8 @@ def main():
                      "frac": bn["frac"], "traffic": None},
         "kernels": kernels,
     }
+    if not args.no_end_to_end:
+        out["end_to_end"] = end_to_end()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
