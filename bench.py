@@ -138,6 +138,52 @@ def cpu_baseline(sample_n=23, reps=5):
                       f"CPU ops (torch {torch.__version__}), 1 warm-up + median of {reps}"}
 
 
+MFMA_F32_PEAK_TFLOPS = 157.3  # MI355X published dense fp32 matrix rate
+CONV_SHAPE = dict(N=184, C=256, K=256, R=3, S=3, H=14, W=14, stride=1, pad=1)  # ResNet-50 layer3
+
+
+def conv_bench(steps, warmup):
+    """Forward / backward-data / backward-weight of the ResNet-50 layer3 3x3 convolution at
+    batch 184, fp32, every kernel variant the solver can select; TFLOP/s counts 2*N*K*P*Q*C*R*S
+    per call against the fp32 matrix-core peak."""
+    import torch
+
+    from monet_amd.lm_ops import conv as cv
+    c = CONV_SHAPE
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    x = torch.randn(c["N"], c["C"], c["H"], c["W"], device=dev)
+    w = torch.randn(c["K"], c["C"], c["R"], c["S"], device=dev) * (2.0 / (c["K"] * 9)) ** 0.5
+    y = cv.conv_forward(x, w, None, c["pad"], c["stride"], 1, 1, 0)
+    dy = torch.randn_like(y)
+    flops = 2.0 * y.numel() * c["C"] * c["R"] * c["S"]
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        a.record()
+        for _ in range(steps):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        ms = a.elapsed_time(b) / steps
+        tf = flops / ms / 1e9
+        return {"ms": round(ms, 4), "TFLOP/s": round(tf, 1), "frac": round(tf / MFMA_F32_PEAK_TFLOPS, 4)}
+
+    res = {"shape": c, "dtype": "f32", "flops_per_call": flops, "peak_TFLOP/s": MFMA_F32_PEAK_TFLOPS}
+    for v in range(cv.n_fwd_algos()):
+        res["fwd_v%d" % v] = timed(lambda: cv.conv_forward(x, w, None, c["pad"], c["stride"], 1, 1, v))
+    for v in range(cv.n_bwd_ip_algos()):
+        res["bwd_data_v%d" % v] = timed(lambda: cv.conv_backward_input(
+            list(x.shape), dy, w, c["pad"], c["stride"], 1, 1, v))
+    for v in range(cv.n_bwd_wt_algos()):
+        res["bwd_weight_v%d" % v] = timed(lambda: cv.conv_backward_weight(
+            list(w.shape), dy, x, c["pad"], c["stride"], 1, 1, v))
+    return res
+
+
 E2E_MODE = "inplace_conv_multiway_newnode"
 E2E_BS = 184
 
@@ -211,6 +257,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-end-to-end", action="store_true")
+    ap.add_argument("--only", choices=["conv"], default=None,
+                    help="run one section alone (for profiling under rocprofv3)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
@@ -220,6 +268,9 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
+    if args.only == "conv":
+        print(json.dumps({"conv": conv_bench(args.steps, args.warmup)}))
+        return
     ms_per_step, kernels = gpu_bench(args.steps, args.warmup)
     value = BYTES_STEP / (ms_per_step * 1e-3) / 1e9
     bn = kernels["bn_bwd_from_output"]
@@ -238,6 +289,7 @@ def main():
                      "frac": bn["frac"], "traffic": None},
         "kernels": kernels,
     }
+    out["conv"] = conv_bench(args.steps, args.warmup)
     if not args.no_end_to_end:
         out["end_to_end"] = end_to_end()
     if not args.no_cpu_baseline:
