@@ -29,6 +29,10 @@ if str(ROOT) not in sys.path:
     sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth, GB/s
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `--only lm_ops`, scaled by
+# what the same counters read for a plain copy of known size (FETCH_SIZE x2.000, WRITE_SIZE x1.000);
+# the counter run cannot happen inside this program, so the figures are recorded here
+TRAFFIC = {"bn_bwd_from_output": 1775456256, "relu_bwd_mask": 1200261120, "maxpool_bwd_idx": 778724352}
 
 N, C, H, W = 184, 256, 56, 56          # BN / ReLU tensor
 PN, PC, PH_IN, PW_IN = 184, 64, 112, 112  # max-pool input
@@ -39,7 +43,7 @@ BYTES_POOL = E * 4 + (E // 4) * 4 + (E // 4) // 2  # write dx, read dy, read pac
 BYTES_STEP = BYTES_BN + BYTES_RELU + BYTES_POOL
 
 
-def gpu_bench(steps, warmup):
+def gpu_bench(steps, warmup, calibrate=False):
     import torch
 
     import monet_amd.lm_ops as lm_ops
@@ -76,6 +80,10 @@ def gpu_bench(steps, warmup):
     def op_pool():
         return pool_ops.max_pool2d_backward_from_packed_indices(pdy, idx4, geo, in_shape)
 
+    if calibrate:
+        # one plain copy of E floats (E*4 bytes read, E*4 written): the yardstick the HBM
+        # traffic counters of the other kernels are scaled by
+        torch.empty_like(dy).copy_(dy)
     ops = [("bn_bwd_from_output", op_bn, BYTES_BN), ("relu_bwd_mask", op_relu, BYTES_RELU),
            ("maxpool_bwd_idx", op_pool, BYTES_POOL)]
     for _ in range(warmup):
@@ -99,7 +107,7 @@ def gpu_bench(steps, warmup):
         ms = sum(a.elapsed_time(b) for a, b in ev[name]) / steps
         gbs = nbytes / (ms * 1e-3) / 1e9
         kernels[name] = {"ms": round(ms, 4), "bytes": nbytes, "GB/s": round(gbs, 1),
-                         "frac": round(gbs / HBM_PEAK_GBS, 4)}
+                         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC[name]}
     return ms_per_step, kernels
 
 
@@ -257,7 +265,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-end-to-end", action="store_true")
-    ap.add_argument("--only", choices=["conv"], default=None,
+    ap.add_argument("--only", choices=["conv", "lm_ops"], default=None,
                     help="run one section alone (for profiling under rocprofv3)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -271,7 +279,10 @@ def main():
     if args.only == "conv":
         print(json.dumps({"conv": conv_bench(args.steps, args.warmup)}))
         return
-    ms_per_step, kernels = gpu_bench(args.steps, args.warmup)
+    ms_per_step, kernels = gpu_bench(args.steps, args.warmup, calibrate=args.only == "lm_ops")
+    if args.only == "lm_ops":
+        print(json.dumps({"ms_per_step": ms_per_step, "kernels": kernels}))
+        return
     value = BYTES_STEP / (ms_per_step * 1e-3) / 1e9
     bn = kernels["bn_bwd_from_output"]
     out = {
@@ -286,7 +297,7 @@ def main():
                    "bytes_per_step": BYTES_STEP},
         "roofline": {"bound": "hbm", "kernel": "bn_bwd_from_output (bn_prepare_kernel + bn_resident_kernel launches)",
                      "achieved": bn["GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": bn["frac"], "traffic": None},
+                     "frac": bn["frac"], "traffic": bn["traffic"]},
         "kernels": kernels,
     }
     out["conv"] = conv_bench(args.steps, args.warmup)
