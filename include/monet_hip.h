@@ -178,9 +178,14 @@ typedef struct mn_conv2d {
  * / n_bwd_wt_algos (monet/lm_ops/conv.cpp:728-730); the variants are this
  * library's own memory / speed tiers, not cuDNN's algorithm list
  * (conv.cpp:21-46):
- *   forward          0 implicit GEMM, no workspace
+ *   forward          0 implicit GEMM, weights read in place, no workspace
+ *                    1 same with the weights repacked [tap][c][k] (k padded
+ *                      to a multiple of 128) into the workspace, so operand
+ *                      tiles load as full 16-byte vectors; channel counts
+ *                      that are not a multiple of 16 run it like variant 0
  *   backward-data    0 implicit GEMM reading the weights through strides
- *                    1 same with a transposed weight copy in the workspace
+ *                    1 same with the weights repacked [tap][k][c] (c padded
+ *                      to a multiple of 128) into the workspace
  *   backward-weight  0 split reduction combined with atomics into a cleared dw
  *                    1 split reduction through per-split partials in the
  *                      workspace, then a fixed-order sum (reproducible) */

@@ -4,10 +4,12 @@
 // Forward and backward-data are the same "gather GEMM":
 //     D[m][col] = sum over (ch, tap)  A(m, ch, tap) * src[n, ch, oh*ish + dh[tap], ow*isw + dw[tap]]
 // with col = (n, oh, ow).  Forward: A = weights, src = x, taps = the R*S window.
-// Backward-data: A = weights read through strides (or a transposed copy in the
-// workspace), src = dy; for stride > 1 the input positions are split by parity
+// Backward-data: A = weights read through strides, src = dy; for stride > 1 the input positions are split by parity
 // class so that every class is a dense stride-1 gather over the taps that can
 // reach it (no multiplies by structural zeros).
+//
+// Variant 1 of both first repacks the weights into the workspace as
+// A'[tap][ch][m] (m contiguous, padded), the order the kernel stages them in.
 //
 // Backward-weight is a GEMM whose reduction runs over (n, p, q); the reduction
 // is split across workgroups (split-K) and combined either with atomics into a
@@ -62,8 +64,8 @@ static FastDiv make_fastdiv(uint32_t d) {
 }
 
 // Multiply one staged k-tile (DEPTH deep, k-major in LDS) into the accumulators.
-template <class TL, int DEPTH>
-__device__ __forceinline__ void mma_tile(const float (*As)[TL::BM + kPad],
+template <class TL, int DEPTH, int LDA = TL::BM + kPad>
+__device__ __forceinline__ void mma_tile(const float (*As)[LDA],
                                          const float (*Bs)[TL::BN + kPad], int wm, int wn,
                                          int lane, float16_t (&acc)[TL::TM][TL::TN]) {
   const int r = lane & 31, half = lane >> 5;
@@ -113,14 +115,21 @@ struct Gather {
 // scalar, and little vector ALU work competes with the matrix cores.
 // Otherwise (e.g. 3 input channels) kk = ch*T + tap and every element is
 // decomposed on its own.  All tensors are < 4 GB (checked by the host).
-template <class TL, bool FAST>
+// PACKED (with FAST): `a` is a repacked copy A'[tap][ch][m] with rows of g.lda
+// floats (a multiple of 128, zero padded), so a k-tile of A is BK contiguous
+// row pieces: one 16-byte load per lane and row piece, no masks, and 8 cache
+// lines per wavefront load instead of the ~20 a strided gather touches.
+constexpr int kPadPacked = 4;  // keeps LDS rows 16-byte aligned for the 128-bit stores
+template <class TL, bool FAST, bool PACKED = false>
 __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
                                                                const float* __restrict__ a,
                                                                const float* __restrict__ src,
                                                                const float* __restrict__ bias,
                                                                float* __restrict__ dst) {
+  static_assert(!PACKED || FAST, "the packed operand is only used with the tap-major path");
   constexpr int BM = TL::BM, BN = TL::BN;
-  __shared__ float lds_a[2][BK][BM + kPad];
+  constexpr int LDA = BM + (PACKED ? kPadPacked : kPad);
+  __shared__ __attribute__((aligned(16))) float lds_a[2][BK][LDA];
   __shared__ float lds_b[2][BK][BN + kPad];
   __shared__ int tdh[kMaxTaps], tdw[kMaxTaps], taoff[kMaxTaps];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -159,12 +168,25 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
   const uint32_t pix_b = img_b + (uint32_t)(ohs * g.Ws + ows) * 4u + brow0 * plane_b;
   uint32_t am_b[kARows];
   uint32_t am_ok = 0;
+  if (!PACKED) {
 #pragma unroll
-  for (int i = 0; i < kARows; ++i) {
-    const int m = m0 + arow0 + kAStep * i;
-    const bool ok = m < g.M;
-    am_b[i] = ok ? (uint32_t)(((long long)m * g.lda + (FAST ? (long long)ak * g.cha : 0)) * 4) : 0u;
-    am_ok |= (ok ? 1u : 0u) << i;
+    for (int i = 0; i < kARows; ++i) {
+      const int m = m0 + arow0 + kAStep * i;
+      const bool ok = m < g.M;
+      am_b[i] = ok ? (uint32_t)(((long long)m * g.lda + (FAST ? (long long)ak * g.cha : 0)) * 4) : 0u;
+      am_ok |= (ok ? 1u : 0u) << i;
+    }
+  }
+  // packed A loader: float4 number f = tid + kThreads*i of the k-tile, row f / (BM/4)
+  constexpr int kA4 = BM * BK / 4 / kThreads;
+  float4_t ra4[kA4 > 0 ? kA4 : 1];
+  uint32_t ap_b[kA4 > 0 ? kA4 : 1];
+  if (PACKED) {
+#pragma unroll
+    for (int i = 0; i < kA4; ++i) {
+      const int f = tid + kThreads * i;
+      ap_b[i] = (uint32_t)(((long long)(f / (BM / 4)) * g.lda + m0 + 4 * (f % (BM / 4))) * 4);
+    }
   }
 
   const char* sp = reinterpret_cast<const char*>(src);
@@ -184,11 +206,18 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
 #pragma unroll
     for (int i = 0; i < kBRows; ++i)
       rb[i] = *reinterpret_cast<const float*>(sp + (base + kBStep * i * plane_b));
-    const uint32_t sa = (uint32_t)(((long long)c0 * g.cha + taoff[t]) * 4);
+    if (PACKED) {
+      const uint32_t sa = (uint32_t)(((long long)taoff[t] * g.Cs + c0) * g.lda * 4);
 #pragma unroll
-    for (int i = 0; i < kARows; ++i) {
-      const bool mok = (am_ok >> i) & 1u;
-      ra[i] = *reinterpret_cast<const float*>(ap + (am_b[i] + (mok ? sa : 0u)));
+      for (int i = 0; i < kA4; ++i)
+        ra4[i] = *reinterpret_cast<const float4_t*>(ap + (ap_b[i] + sa));
+    } else {
+      const uint32_t sa = (uint32_t)(((long long)c0 * g.cha + taoff[t]) * 4);
+#pragma unroll
+      for (int i = 0; i < kARows; ++i) {
+        const bool mok = (am_ok >> i) & 1u;
+        ra[i] = *reinterpret_cast<const float*>(ap + (am_b[i] + (mok ? sa : 0u)));
+      }
     }
   };
   auto fetch_any = [&](int k0) {
@@ -225,9 +254,17 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
 #pragma unroll
     for (int i = 0; i < kBRows; ++i)
       lds_b[buf][brow0 + kBStep * i][bcol] = ((b_ok >> i) & 1u) ? rb[i] : 0.f;
+    if (PACKED) {
 #pragma unroll
-    for (int i = 0; i < kARows; ++i)
-      lds_a[buf][ak][arow0 + kAStep * i] = (a_ok && ((am_ok >> i) & 1u)) ? ra[i] : 0.f;
+      for (int i = 0; i < kA4; ++i) {
+        const int f = tid + kThreads * i;
+        *reinterpret_cast<float4_t*>(&lds_a[buf][f / (BM / 4)][4 * (f % (BM / 4))]) = ra4[i];
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < kARows; ++i)
+        lds_a[buf][ak][arow0 + kAStep * i] = (a_ok && ((am_ok >> i) & 1u)) ? ra[i] : 0.f;
+    }
   };
 
   float16_t acc[TL::TM][TL::TN];
@@ -259,7 +296,7 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
     for (int kt = 0; kt < ktiles; ++kt) {
       const int buf = kt & 1;
       if (kt + 1 < ktiles) fetch_next(kt + 1);
-      mma_tile<TL, BK>(lds_a[buf], lds_b[buf], wm, wn, lane, acc);
+      mma_tile<TL, BK, LDA>(lds_a[buf], lds_b[buf], wm, wn, lane, acc);
       if (kt + 1 < ktiles) stage(buf ^ 1);
       __syncthreads();
     }
@@ -463,19 +500,21 @@ __global__ __launch_bounds__(kThreads) void fill_zero_kernel(float* p, size_t n)
   for (size_t j = n4 * 4 + i; j < n; j += (size_t)gridDim.x * kThreads) p[j] = 0.f;
 }
 
-// wt[c][k][r][s] = w[k][c][r][s]
-__global__ __launch_bounds__(kThreads) void transpose_weights_kernel(const float* __restrict__ w,
-                                                                     float* __restrict__ wt, int K,
-                                                                     int C, int RS) {
+// out[(t*Cs + ch)*Mp + m] = A(m, ch, t) = a[m*lda + ch*cha + t] for m < M, else 0
+__global__ __launch_bounds__(kThreads) void pack_weights_kernel(const float* __restrict__ a,
+                                                                float* __restrict__ out, int M,
+                                                                int Mp, int Cs, int T,
+                                                                long long lda, long long cha) {
   const size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x;
-  const size_t n = (size_t)K * C * RS;
+  const size_t n = (size_t)T * Cs * Mp;
   if (i >= n) return;
-  const int rs = i % RS;
-  const size_t kc = i / RS;
-  const int k = kc % K;
-  const int c = kc / K;
-  wt[i] = w[((size_t)k * C + c) * RS + rs];
+  const int m = (int)(i % Mp);
+  const size_t row = i / Mp;
+  const int ch = (int)(row % Cs), t = (int)(row / Cs);
+  out[i] = m < M ? a[(size_t)m * lda + (size_t)ch * cha + t] : 0.f;
 }
+
+static long long packed_rows(long long M) { return (M + 127) / 128 * 128; }
 
 // ------------------------------------------------------------------ host --
 static int check(const mn_conv2d* g) {
@@ -514,29 +553,34 @@ static int pick_tile(long long M, long long ncols, bool fast) {
   return M <= 64 ? 1 : 2;
 }
 
+static bool fast_path(const Gather& g) { return g.T > 0 && g.Cs % BK == 0; }
+
 template <class TL>
 static void launch_gather_t(const Gather& g, const float* a, const float* src, const float* bias,
-                            float* dst, hipStream_t s) {
+                            float* dst, hipStream_t s, bool packed) {
   dim3 grid((g.ncols + TL::BN - 1) / TL::BN, (g.M + TL::BM - 1) / TL::BM);
-  if (g.T > 0 && g.Cs % BK == 0)
+  if (packed)
+    gather_gemm_kernel<TL, true, true><<<grid, kThreads, 0, s>>>(g, a, src, bias, dst);
+  else if (fast_path(g))
     gather_gemm_kernel<TL, true><<<grid, kThreads, 0, s>>>(g, a, src, bias, dst);
   else
     gather_gemm_kernel<TL, false><<<grid, kThreads, 0, s>>>(g, a, src, bias, dst);
 }
 
+// `packed`: a = the repacked operand (pack_weights_kernel) with rows of g.lda floats.
 static void launch_gather(const Gather& g, const float* a, const float* src, const float* bias,
-                          float* dst, hipStream_t s, int tile = -1) {
+                          float* dst, hipStream_t s, bool packed = false, int tile = -1) {
   if (g.ncols == 0 || g.M == 0) return;
 #ifdef MN_TUNING
   if (const char* e = getenv("MN_CONV_TILE")) tile = atoi(e);
 #endif
   if (tile < 0) tile = pick_tile(g.M, g.ncols, g.T > 0 && g.Cs % BK == 0);
   switch (tile) {
-    case 1: launch_gather_t<T64x256>(g, a, src, bias, dst, s); break;
-    case 2: launch_gather_t<T64x128>(g, a, src, bias, dst, s); break;
-    case 3: launch_gather_t<T128x64>(g, a, src, bias, dst, s); break;
-    case 4: launch_gather_t<T64x64>(g, a, src, bias, dst, s); break;
-    default: launch_gather_t<T128x128>(g, a, src, bias, dst, s); break;
+    case 1: launch_gather_t<T64x256>(g, a, src, bias, dst, s, packed); break;
+    case 2: launch_gather_t<T64x128>(g, a, src, bias, dst, s, packed); break;
+    case 3: launch_gather_t<T128x64>(g, a, src, bias, dst, s, packed); break;
+    case 4: launch_gather_t<T64x64>(g, a, src, bias, dst, s, packed); break;
+    default: launch_gather_t<T128x128>(g, a, src, bias, dst, s, packed); break;
   }
 }
 
@@ -584,7 +628,7 @@ extern "C" {
 int mn_conv_n_variants(int direction) {
   switch (direction) {
     case MN_CONV_FWD:
-      return 1;
+      return 2;
     case MN_CONV_BWD_DATA:
       return 2;
     case MN_CONV_BWD_WEIGHT:
@@ -603,7 +647,11 @@ int mn_conv_ws_bytes(const mn_conv2d* g, int direction, int variant, int dtype, 
   if (dtype != MN_F32) return MN_EUNSUPPORTED;
   if (variant < 0 || variant >= mn_conv_n_variants(direction)) return MN_EUNSUPPORTED;
   const size_t wsize = (size_t)g->K * g->C * g->R * g->S * sizeof(float);
-  if (direction == MN_CONV_BWD_DATA && variant == 1) *bytes = wsize;
+  // variant 1 of the gather directions: the repacked weight operand (rows padded to 128)
+  if (direction == MN_CONV_FWD && variant == 1)
+    *bytes = (size_t)g->R * g->S * g->C * packed_rows(g->K) * sizeof(float);
+  if (direction == MN_CONV_BWD_DATA && variant == 1)
+    *bytes = (size_t)g->R * g->S * g->K * packed_rows(g->C) * sizeof(float);
   if (direction == MN_CONV_BWD_WEIGHT && variant == 1) {
     int splits, tiles;
     wgrad_split(g, &splits, &tiles);
@@ -615,12 +663,10 @@ int mn_conv_ws_bytes(const mn_conv2d* g, int direction, int variant, int dtype, 
 int mn_conv_fwd(const mn_conv2d* g, const void* x, const void* w, const void* bias, void* y,
                 void* ws, size_t ws_bytes, int variant, int dtype, mn_stream_t stream) {
   using namespace mn_conv;
-  (void)ws;
-  (void)ws_bytes;
   const int st = check(g);
   if (st != MN_OK) return st;
   if (dtype != MN_F32) return MN_EUNSUPPORTED;
-  if (variant != 0) return MN_EUNSUPPORTED;
+  if (variant < 0 || variant > 1) return MN_EUNSUPPORTED;
   if (g->N == 0) return MN_OK;
   if (!x || !w || !y) return MN_EINVAL;
   Gather q = {};
@@ -649,8 +695,20 @@ int mn_conv_fwd(const mn_conv2d* g, const void* x, const void* w, const void* bi
       q.dw[t] = (int16_t)(s * g->dW - g->pW);
       q.aoff[t] = t;
     }
-  launch_gather(q, (const float*)w, (const float*)x, (const float*)bias, (float*)y,
-                mn_stream(stream));
+  hipStream_t s = mn_stream(stream);
+  const float* a = (const float*)w;
+  // the repacked operand needs the tap-major path; other shapes run variant 1 like variant 0
+  const bool packed = variant == 1 && fast_path(q);
+  if (packed) {
+    const long long Mp = packed_rows(q.M);
+    const size_t n = (size_t)q.T * q.Cs * Mp;
+    if (!ws || ws_bytes < n * sizeof(float) || !mn_aligned(ws, 16)) return MN_EINVAL;
+    pack_weights_kernel<<<(unsigned)((n + kThreads - 1) / kThreads), kThreads, 0, s>>>(
+        a, (float*)ws, q.M, (int)Mp, q.Cs, q.T, q.lda, q.cha);
+    a = (const float*)ws;
+    q.lda = Mp;
+  }
+  launch_gather(q, a, (const float*)x, (const float*)bias, (float*)y, s, packed);
   return mn_launch_status();
 }
 
@@ -667,14 +725,15 @@ int mn_conv_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void* dx
   const int RS = g->R * g->S;
   const float* a = (const float*)w;
   long long lda = RS, cha = (long long)g->C * RS;  // read w[k][c][r][s] as A(c, k, rs)
-  if (variant == 1) {
-    const size_t n = (size_t)g->K * g->C * RS;
-    if (!ws || ws_bytes < n * sizeof(float) || !mn_aligned(ws, 4)) return MN_EINVAL;
-    transpose_weights_kernel<<<(unsigned)((n + kThreads - 1) / kThreads), kThreads, 0, s>>>(
-        (const float*)w, (float*)ws, g->K, g->C, RS);
+  const bool packed = variant == 1 && g->K % BK == 0;
+  if (packed) {  // A'[rs][k][c], rows of Cp floats
+    const long long Cp = packed_rows(g->C);
+    const size_t n = (size_t)RS * g->K * Cp;
+    if (!ws || ws_bytes < n * sizeof(float) || !mn_aligned(ws, 16)) return MN_EINVAL;
+    pack_weights_kernel<<<(unsigned)((n + kThreads - 1) / kThreads), kThreads, 0, s>>>(
+        a, (float*)ws, g->C, (int)Cp, g->K, RS, lda, cha);
     a = (const float*)ws;
-    lda = (long long)g->K * RS;
-    cha = RS;
+    lda = Cp;
   }
   // Classes no tap can reach (e.g. 1x1 filters with stride 2) are plain zeros: clear dx once
   // with full-width stores instead of scattering zeros class by class.
@@ -729,7 +788,7 @@ int mn_conv_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void* dx
       q.osw = g->sW;
       q.lda = lda;
       q.cha = cha;
-      launch_gather(q, a, (const float*)dy, nullptr, (float*)dx, s);
+      launch_gather(q, a, (const float*)dy, nullptr, (float*)dx, s, packed);
     }
   }
   return mn_launch_status();
