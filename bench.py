@@ -108,6 +108,28 @@ def gpu_bench(steps, warmup, calibrate=False):
         gbs = nbytes / (ms * 1e-3) / 1e9
         kernels[name] = {"ms": round(ms, 4), "bytes": nbytes, "GB/s": round(gbs, 1),
                          "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC[name]}
+    # the forward kernels of the same operators, timed on their own (not part of the step)
+    x = torch.randn(N, C, H, W, device=dev)
+    px = torch.randn(PN, PC, PH_IN, PW_IN, device=dev)
+    fwd = [("relu_fwd_mask", lambda: relu_ops.relu_forward_with_mask(x), 2 * E * 4 + E // 8),
+           ("bn_fwd_train", lambda: bn_ops.bn_forward_train(x, gamma, beta, None, None, 0.1, 1e-5),
+            2 * E * 4),
+           ("maxpool_fwd_idx", lambda: pool_ops.max_pool2d_with_packed_indices(px, 3, 2, 1, 1, False),
+            BYTES_POOL)]
+    for name, fn, nbytes in fwd:
+        for _ in range(warmup):
+            fn()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        a.record()
+        for _ in range(steps):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        ms = a.elapsed_time(b) / steps
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        kernels[name] = {"ms": round(ms, 4), "bytes": nbytes, "GB/s": round(gbs, 1),
+                         "frac": round(gbs / HBM_PEAK_GBS, 4), "in_step": False}
     return ms_per_step, kernels
 
 

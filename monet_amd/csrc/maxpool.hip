@@ -101,6 +101,55 @@ __global__ __launch_bounds__(kThreads) void maxpool_fwd_idx_kernel(
   idx4[j] = (uint8_t)(((i0 & 15u) << 4) | (i1 & 15u));
 }
 
+// Forward for kernel 3, stride 2, pad 1, dilation 1 with even H and W % 4 == 0
+// (PH = H/2, PW = W/2): one workgroup per (n, c) plane, one thread per pair of
+// horizontally adjacent outputs = one index byte.  The pair's two windows span
+// input columns 4q-1 .. 4q+3 of rows 2ph-1 .. 2ph+1: per row one aligned
+// 16-byte load plus the left neighbour.  Scan order and tie rules are those of
+// pool_one, so values and indices are identical to the generic kernel's.
+__global__ __launch_bounds__(kThreads) void maxpool_fwd_k3s2p1_kernel(
+    const float* __restrict__ x, float* __restrict__ y, uint8_t* __restrict__ idx4, int H, int W) {
+  const int PH = H >> 1, PW = W >> 1, QW = W >> 2;
+  const size_t plane = blockIdx.x;
+  const float* xp = x + plane * (size_t)H * W;
+  float* yp = y + plane * (size_t)PH * PW;
+  uint8_t* ip = idx4 + ((plane * (size_t)PH * PW) >> 1);  // PH*PW is even
+  const int items = PH * QW;
+  const int qstep = kThreads / QW, rstep = kThreads - qstep * QW;
+  int ph = threadIdx.x / QW;
+  int q = threadIdx.x - ph * QW;
+  for (int it = threadIdx.x; it < items; it += kThreads) {
+    const bool top = ph > 0, left = q > 0;
+    float m0 = -INFINITY, m1 = -INFINITY;
+    uint32_t i0 = (top ? 0u : 3u) + (left ? 0u : 1u), i1 = top ? 0u : 3u;
+#pragma unroll
+    for (int ch = 0; ch < 3; ++ch) {
+      if (ch == 0 && !top) continue;
+      const float* row = xp + (size_t)(2 * ph - 1 + ch) * W + 4 * q;
+      const float4_t v = *reinterpret_cast<const float4_t*>(row);
+      if (left) {
+        const float l = row[-1];
+        if (l > m0 || l != l) { m0 = l; i0 = ch * 3; }
+      }
+      if (v.x > m0 || v.x != v.x) { m0 = v.x; i0 = ch * 3 + 1; }
+      if (v.y > m0 || v.y != v.y) { m0 = v.y; i0 = ch * 3 + 2; }
+      if (v.y > m1 || v.y != v.y) { m1 = v.y; i1 = ch * 3; }
+      if (v.z > m1 || v.z != v.z) { m1 = v.z; i1 = ch * 3 + 1; }
+      if (v.w > m1 || v.w != v.w) { m1 = v.w; i1 = ch * 3 + 2; }
+    }
+    const int o = ph * PW + 2 * q;  // even
+    float2_t out = {m0, m1};
+    *reinterpret_cast<float2_t*>(yp + o) = out;
+    ip[o >> 1] = (uint8_t)((i0 << 4) | i1);
+    ph += qstep;
+    q += rstep;
+    if (q >= QW) {
+      q -= QW;
+      ++ph;
+    }
+  }
+}
+
 // Range of windows along one axis that cover input coordinate `c`.
 template <class G>
 __device__ __forceinline__ void cover(int c, int pad, int k, int dil, int stride, int pooled,
@@ -296,7 +345,10 @@ int mn_maxpool_fwd_idx_f32(const mn_pool2d* g, const float* x, float* y, uint8_t
   if ((size_t)g->N * g->C == 0) return MN_OK;
   if (!x || !y || !idx4) return MN_EINVAL;
   hipStream_t s = mn_stream(stream);
-  if (is_ct(g, 3, 2, 1))
+  if (is_ct(g, 3, 2, 1) && g->H % 2 == 0 && g->W % 4 == 0 && g->PH == g->H / 2 &&
+      g->PW == g->W / 2 && mn_aligned(x, 16) && mn_aligned(y, 8) && g->W / 4 <= kThreads)
+    maxpool_fwd_k3s2p1_kernel<<<(unsigned)g->N * g->C, kThreads, 0, s>>>(x, y, idx4, g->H, g->W);
+  else if (is_ct(g, 3, 2, 1))
     launch_fwd(CtGeo<3, 2, 1>{}, g, x, y, idx4, s);
   else if (is_ct(g, 2, 2, 0))
     launch_fwd(CtGeo<2, 2, 0>{}, g, x, y, idx4, s);
