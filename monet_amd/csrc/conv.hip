@@ -477,6 +477,114 @@ __global__ __launch_bounds__(kThreads) void wgrad_kernel(const WGrad g,
   }
 }
 
+
+// The same GEMM with the columns ordered tap-major, for C % BN == 0 and K % BM == 0:
+// blockIdx.x = tap * (C / BN) + channel tile, so a column tile lies inside ONE tap.
+// Then the window shift is a per-workgroup scalar, a thread's window test is one
+// comparison per k-tile (its depth lane fixes (p, q)), row addresses are arithmetic
+// progressions instead of per-row tables, and no row needs a bounds mask: fewer
+// vector registers (more resident waves) and far less address arithmetic between
+// the matrix instructions.
+template <class TL, int DEPTH>
+__global__ __launch_bounds__(kThreads) void wgrad_tap_kernel(const WGrad g,
+                                                             const float* __restrict__ dy,
+                                                             const float* __restrict__ x,
+                                                             float* __restrict__ out) {
+  constexpr int BM = TL::BM, BN = TL::BN;
+  __shared__ float lds_a[2][DEPTH][BM + kPad];
+  __shared__ float lds_b[2][DEPTH][BN + kPad];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / TL::WN, wn = wave % TL::WN;
+  const int m0 = blockIdx.y * BM;
+  const uint32_t ctiles = (uint32_t)g.C / BN;
+  const uint32_t tap = blockIdx.x / ctiles;
+  const uint32_t c0 = (blockIdx.x - tap * ctiles) * BN;
+  const uint32_t r = g.divS.div(tap), sx = tap - r * g.S;
+  const int dh = (int)r * g.dH - g.pH, dw = (int)sx * g.dW - g.pW;
+  const uint32_t PQ = (uint32_t)g.P * g.Q;
+
+  constexpr int kStep = kThreads / DEPTH, kRowsA = BM / kStep, kRowsB = BN / kStep;
+  const int kdl = tid % DEPTH, row0 = tid / DEPTH;
+  const uint32_t a_row0 = (uint32_t)(m0 + row0) * PQ * 4u, a_step = (uint32_t)kStep * PQ * 4u;
+  const uint32_t HW4 = (uint32_t)g.H * g.W * 4u;
+  const uint32_t b_row0 = (c0 + row0) * HW4 + (uint32_t)((dh * g.W + dw) * 4), b_step = kStep * HW4;
+
+  const char* dyp = reinterpret_cast<const char*>(dy);
+  const char* xp = reinterpret_cast<const char*>(x);
+  float ra[kRowsA], rb[kRowsB];
+  bool a_ok = false, b_ok = false;
+  auto fetch = [&](uint32_t d0) {
+    const uint32_t d = d0 + kdl;
+    a_ok = d < g.depth;
+    const uint32_t dd = a_ok ? d : 0u;
+    const uint32_t n = dd / PQ;
+    const uint32_t pq = dd - n * PQ;
+    const uint32_t p = pq / g.Q, q = pq - p * g.Q;
+    const uint32_t abase = ((n * (uint32_t)g.K) * PQ + pq) * 4u + a_row0;
+#pragma unroll
+    for (int i = 0; i < kRowsA; ++i)
+      ra[i] = *reinterpret_cast<const float*>(dyp + (abase + a_step * i));
+    const int h0 = (int)p * g.sH, w0 = (int)q * g.sW;
+    b_ok = a_ok && (unsigned)(h0 + dh) < (unsigned)g.H && (unsigned)(w0 + dw) < (unsigned)g.W;
+    // an element outside the window is staged as zero; its load reads the row's first element
+    const uint32_t bbase = b_ok ? ((n * (uint32_t)g.C * g.H + h0) * (uint32_t)g.W + w0) * 4u + b_row0
+                                : (c0 + row0) * HW4;
+#pragma unroll
+    for (int i = 0; i < kRowsB; ++i)
+      rb[i] = *reinterpret_cast<const float*>(xp + (bbase + b_step * i));
+  };
+  auto stage = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < kRowsA; ++i) lds_a[buf][kdl][row0 + kStep * i] = a_ok ? ra[i] : 0.f;
+#pragma unroll
+    for (int i = 0; i < kRowsB; ++i) lds_b[buf][kdl][row0 + kStep * i] = b_ok ? rb[i] : 0.f;
+  };
+
+  float16_t acc[TL::TM][TL::TN];
+#pragma unroll
+  for (int i = 0; i < TL::TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TL::TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  const uint32_t total_tiles = (g.depth + DEPTH - 1) / DEPTH;
+  const uint32_t t_begin = blockIdx.z * (g.tiles_per_split * (WBK / DEPTH));
+  const uint32_t t_end = min(t_begin + g.tiles_per_split * (WBK / DEPTH), total_tiles);
+  if (t_begin < t_end) {
+    fetch(t_begin * DEPTH);
+    stage(0);
+    __syncthreads();
+    for (uint32_t kt = t_begin; kt < t_end; ++kt) {
+      const int buf = (kt - t_begin) & 1;
+      if (kt + 1 < t_end) fetch((kt + 1) * DEPTH);
+      mma_tile<TL, DEPTH>(lds_a[buf], lds_b[buf], wm, wn, lane, acc);
+      if (kt + 1 < t_end) stage(buf ^ 1);
+      __syncthreads();
+    }
+  }
+
+  float* base = out;
+  if (g.mode == 2) base += (size_t)blockIdx.z * g.K * g.ncols;
+  const uint32_t RS = (uint32_t)g.R * g.S;
+#pragma unroll
+  for (int nj = 0; nj < TL::TN; ++nj) {
+    const uint32_t c = c0 + wn * (TL::TN * 32) + nj * 32 + (lane & 31);
+#pragma unroll
+    for (int mi = 0; mi < TL::TM; ++mi) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = m0 + wm * (TL::TM * 32) + mi * 32 + acc_row(v, lane);
+        float* o = base + (size_t)m * g.ncols + c * RS + tap;
+        if (g.mode == 1)
+          atomicAdd(o, acc[mi][nj][v]);
+        else
+          *o = acc[mi][nj][v];
+      }
+    }
+  }
+}
+
 // dw[i] = sum over splits of partial[z][i], fixed order.
 __global__ __launch_bounds__(kThreads) void wgrad_reduce_kernel(const float* __restrict__ partial,
                                                                 float* __restrict__ dw, size_t n,
@@ -541,15 +649,18 @@ static int check(const mn_conv2d* g) {
   return MN_OK;
 }
 
-// Tile choice, from sweeps over the ResNet-50 shapes at batch 184 on MI355X:
-// 64 x 128 is within a few percent of the best tile everywhere (its 6 waves per
-// SIMD hide the staging latency better than the larger tiles' 3), and GEMMs with
-// at most 64 rows want all four wavefronts side by side on the columns.  The
-// element-wise path (channels not a multiple of 16) always takes 64 x 128: the
-// wider tiles spill there.
-static int pick_tile(long long M, long long ncols, bool fast) {
+// Tile choice, from sweeps over the ResNet-50 shapes at batch 184 on MI355X.
+// Weights read in place: 64 x 128 is within a few percent of the best tile everywhere
+// (its 6 waves per SIMD hide the staging latency better than the larger tiles' 3), GEMMs
+// with at most 64 rows want all four wavefronts side by side on the columns, and the
+// element-wise path (channels not a multiple of 16) always takes 64 x 128: the wider
+// tiles spill there.  Repacked weights: the A tile costs one load per lane, so 128 rows
+// per workgroup (each gathered column element reused twice as often) wins from 128 rows
+// up, most of all for strided gathers (stride-2 forward: 51 -> 81, 75 -> 102 TFLOP/s).
+static int pick_tile(long long M, long long ncols, bool fast, bool packed) {
   (void)ncols;
   if (!fast) return 2;
+  if (packed) return M <= 64 ? 2 : 3;
   return M <= 64 ? 1 : 2;
 }
 
@@ -574,7 +685,7 @@ static void launch_gather(const Gather& g, const float* a, const float* src, con
 #ifdef MN_TUNING
   if (const char* e = getenv("MN_CONV_TILE")) tile = atoi(e);
 #endif
-  if (tile < 0) tile = pick_tile(g.M, g.ncols, g.T > 0 && g.Cs % BK == 0);
+  if (tile < 0) tile = pick_tile(g.M, g.ncols, fast_path(g), packed);
   switch (tile) {
     case 1: launch_gather_t<T64x256>(g, a, src, bias, dst, s, packed); break;
     case 2: launch_gather_t<T64x128>(g, a, src, bias, dst, s, packed); break;
@@ -585,14 +696,29 @@ static void launch_gather(const Gather& g, const float* a, const float* src, con
 }
 
 // Split of the (n, p, q) reduction: enough workgroups for ~2 per CU.
-static int wgrad_tile(const mn_conv2d* g) {
+static int wgrad_tile(const mn_conv2d* g, int variant) {
 #ifdef MN_TUNING
   if (const char* e = getenv("MN_WGRAD_TILE")) return atoi(e);
 #endif
   // from the same sweeps: 128 x 128 for windows, 128 x 64 for 1x1 filters, 64 rows for K <= 64
   const long long ncols = (long long)g->C * g->R * g->S;
-  if (g->K <= 64) return ncols <= 64 ? 4 : 2;
-  return (g->R * g->S == 1 || ncols <= 64) ? 3 : 0;
+  int tile;
+  if (g->K <= 64)
+    tile = ncols <= 64 ? 4 : 2;
+  else
+    tile = (g->R * g->S == 1 || ncols <= 64) ? 3 : 0;
+  // a 64-wide column tile where it lets the tap-major kernel run (C a multiple of 64, not 128)
+  if (variant == 1 && g->C % 128 != 0 && g->C % 64 == 0 && g->R * g->S > 1) {
+    if (tile == 2) tile = 4;
+    if (tile == 0) tile = 3;
+  }
+  return tile;
+}
+static bool wgrad_tap_major(const mn_conv2d* g, int bm, int bn) {
+#ifdef MN_TUNING
+  if (const char* e = getenv("MN_WGRAD_TAP")) return atoi(e) != 0 && g->C % bn == 0 && g->K % bm == 0;
+#endif
+  return g->C % bn == 0 && g->K % bm == 0;
 }
 static void tile_dims(int tile, int* bm, int* bn) {
   switch (tile) {
@@ -604,9 +730,9 @@ static void tile_dims(int tile, int* bm, int* bn) {
   }
 }
 // Split of the (n, p, q) reduction: enough workgroups for ~3 per CU.
-static void wgrad_split(const mn_conv2d* g, int* splits, int* tiles_per_split) {
+static void wgrad_split(const mn_conv2d* g, int variant, int* splits, int* tiles_per_split) {
   int bm, bn;
-  tile_dims(wgrad_tile(g), &bm, &bn);
+  tile_dims(wgrad_tile(g, variant), &bm, &bn);
   const long long depth = (long long)g->N * g->P * g->Q;
   const long long total_tiles = (depth + WBK - 1) / WBK;
   const long long out_tiles =
@@ -654,7 +780,7 @@ int mn_conv_ws_bytes(const mn_conv2d* g, int direction, int variant, int dtype, 
     *bytes = (size_t)g->R * g->S * g->K * packed_rows(g->C) * sizeof(float);
   if (direction == MN_CONV_BWD_WEIGHT && variant == 1) {
     int splits, tiles;
-    wgrad_split(g, &splits, &tiles);
+    wgrad_split(g, 1, &splits, &tiles);
     *bytes = splits > 1 ? wsize * splits : 0;
   }
   return MN_OK;
@@ -830,7 +956,7 @@ int mn_conv_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, void* 
   q.divRS = make_fastdiv(g->R * g->S);
   q.divS = make_fastdiv(g->S);
   int splits, tps;
-  wgrad_split(g, &splits, &tps);
+  wgrad_split(g, variant, &splits, &tps);
   q.tiles_per_split = tps;
   float* out = (float*)dw;
   if (splits == 1) {
@@ -843,15 +969,36 @@ int mn_conv_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, void* 
     if (!ws || ws_bytes < nw * sizeof(float) * splits || !mn_aligned(ws, 4)) return MN_EINVAL;
     out = (float*)ws;
   }
-  const int tile = wgrad_tile(g);
+  const int tile = wgrad_tile(g, variant);
   int bm, bn;
   tile_dims(tile, &bm, &bn);
+  // with atomics, a tap-major tile would scatter them R*S floats apart: only for 1x1 filters
+  if (wgrad_tap_major(g, bm, bn) && (q.mode != 1 || g->R * g->S == 1)) {
+    dim3 grid(g->R * g->S * (g->C / bn), g->K / bm, splits);
+    int deep = tile == 0 ? 16 : 32;  // 128 x 128 at depth 32 leaves LDS for 2 workgroups per CU only
+#ifdef MN_TUNING
+    if (const char* e = getenv("MN_WGRAD_DEPTH")) deep = atoi(e);
+#endif
+#define MN_TAP(TL)                                                                               \
+  if (deep == 16)                                                                                \
+    wgrad_tap_kernel<TL, 16><<<grid, kThreads, 0, s>>>(q, (const float*)dy, (const float*)x, out); \
+  else                                                                                           \
+    wgrad_tap_kernel<TL, 32><<<grid, kThreads, 0, s>>>(q, (const float*)dy, (const float*)x, out)
+    switch (tile) {
+      case 2: MN_TAP(T64x128); break;
+      case 3: MN_TAP(T128x64); break;
+      case 4: MN_TAP(T64x64); break;
+      default: MN_TAP(T128x128); break;
+    }
+#undef MN_TAP
+  } else {
   dim3 grid((q.ncols + bn - 1) / bn, (g->K + bm - 1) / bm, splits);
   switch (tile) {
     case 2: wgrad_kernel<T64x128><<<grid, kThreads, 0, s>>>(q, (const float*)dy, (const float*)x, out); break;
     case 3: wgrad_kernel<T128x64><<<grid, kThreads, 0, s>>>(q, (const float*)dy, (const float*)x, out); break;
     case 4: wgrad_kernel<T64x64><<<grid, kThreads, 0, s>>>(q, (const float*)dy, (const float*)x, out); break;
     default: wgrad_kernel<T128x128><<<grid, kThreads, 0, s>>>(q, (const float*)dy, (const float*)x, out); break;
+  }
   }
   if (q.mode == 2)
     wgrad_reduce_kernel<<<(unsigned)((nw + kThreads - 1) / kThreads), kThreads, 0, s>>>(
