@@ -168,7 +168,8 @@ def cpu_baseline(sample_n=23, reps=5):
                       f"CPU ops (torch {torch.__version__}), 1 warm-up + median of {reps}"}
 
 
-MFMA_F32_PEAK_TFLOPS = 157.3  # MI355X published dense fp32 matrix rate
+MFMA_F32_PEAK_TFLOPS = 157.3   # MI355X published dense fp32 matrix rate
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # ... and dense bf16
 CONV_SHAPE = dict(N=184, C=256, K=256, R=3, S=3, H=14, W=14, stride=1, pad=1)  # ResNet-50 layer3
 
 
@@ -188,7 +189,7 @@ def conv_bench(steps, warmup):
     dy = torch.randn_like(y)
     flops = 2.0 * y.numel() * c["C"] * c["R"] * c["S"]
 
-    def timed(fn):
+    def timed(fn, peak):
         for _ in range(warmup):
             fn()
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -200,17 +201,27 @@ def conv_bench(steps, warmup):
         torch.cuda.synchronize()
         ms = a.elapsed_time(b) / steps
         tf = flops / ms / 1e9
-        return {"ms": round(ms, 4), "TFLOP/s": round(tf, 1), "frac": round(tf / MFMA_F32_PEAK_TFLOPS, 4)}
+        return {"ms": round(ms, 4), "TFLOP/s": round(tf, 1), "frac": round(tf / peak, 4)}
+
+    def directions(x, w, dy, peak):
+        out = {}
+        for v in range(cv.n_fwd_algos()):
+            out["fwd_v%d" % v] = timed(
+                lambda: cv.conv_forward(x, w, None, c["pad"], c["stride"], 1, 1, v), peak)
+        for v in range(cv.n_bwd_ip_algos()):
+            out["bwd_data_v%d" % v] = timed(lambda: cv.conv_backward_input(
+                list(x.shape), dy, w, c["pad"], c["stride"], 1, 1, v), peak)
+        for v in range(cv.n_bwd_wt_algos()):
+            out["bwd_weight_v%d" % v] = timed(lambda: cv.conv_backward_weight(
+                list(w.shape), dy, x, c["pad"], c["stride"], 1, 1, v), peak)
+        return out
 
     res = {"shape": c, "dtype": "f32", "flops_per_call": flops, "peak_TFLOP/s": MFMA_F32_PEAK_TFLOPS}
-    for v in range(cv.n_fwd_algos()):
-        res["fwd_v%d" % v] = timed(lambda: cv.conv_forward(x, w, None, c["pad"], c["stride"], 1, 1, v))
-    for v in range(cv.n_bwd_ip_algos()):
-        res["bwd_data_v%d" % v] = timed(lambda: cv.conv_backward_input(
-            list(x.shape), dy, w, c["pad"], c["stride"], 1, 1, v))
-    for v in range(cv.n_bwd_wt_algos()):
-        res["bwd_weight_v%d" % v] = timed(lambda: cv.conv_backward_weight(
-            list(w.shape), dy, x, c["pad"], c["stride"], 1, 1, v))
+    res.update(directions(x, w, dy, MFMA_F32_PEAK_TFLOPS))
+    # the same problem on bf16 channels-last tensors (bf16 matrix cores, fp32 accumulation)
+    cl = lambda t: t.to(torch.bfloat16).contiguous(memory_format=torch.channels_last)
+    res["bf16"] = {"layout": "channels-last", "peak_TFLOP/s": MFMA_BF16_PEAK_TFLOPS}
+    res["bf16"].update(directions(cl(x), cl(w), cl(dy), MFMA_BF16_PEAK_TFLOPS))
     return res
 
 

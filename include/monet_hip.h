@@ -171,7 +171,18 @@ typedef struct mn_conv2d {
 #define MN_CONV_FWD 0
 #define MN_CONV_BWD_DATA 1
 #define MN_CONV_BWD_WEIGHT 2
-#define MN_F32 0 /* fp32 tensors, fp32 matrix-core arithmetic */
+#define MN_F32 0 /* fp32 NCHW tensors, weights [K,C,R,S], fp32 matrix-core arithmetic */
+/* bf16 tensors in channels-last order - activations [N,H,W,C], weights
+ * [K,R,S,C], outputs [N,P,Q,K], bias bf16 - multiplied on the bf16 matrix
+ * cores with fp32 accumulation and rounded once (to nearest even) on output.
+ * Needs channel counts that are multiples of 32 on the reduction side
+ * (forward: C; backward-data: K) and multiples of 64 for backward-weight (C and
+ * K); otherwise MN_EUNSUPPORTED.  Both variant indices of a direction run the
+ * same kernel; backward-data always needs K*C*R*S*2 bytes of workspace (the
+ * transposed weights) and backward-weight its fp32 split partials - ask
+ * mn_conv_ws_bytes.  The reference has no reduced-precision path; this dtype
+ * serves the bf16 configuration of the layer3 benchmark. */
+#define MN_BF16 1
 
 /* Number of kernel variants ("algorithms") per direction; variant 0 always
  * runs and needs no workspace.  Takes the role of n_fwd_algos / n_bwd_ip_algos

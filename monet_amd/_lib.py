@@ -36,6 +36,7 @@ class Conv2d(Structure):
 
 CONV_FWD, CONV_BWD_DATA, CONV_BWD_WEIGHT = 0, 1, 2
 F32 = 0
+BF16 = 1   # bf16 tensors in channels-last order (see include/monet_hip.h)
 
 
 class Pool2d(Structure):

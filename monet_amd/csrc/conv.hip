@@ -25,6 +25,15 @@
 #include <cstdlib>
 #endif
 
+// bf16 / channels-last kernels (conv_bf16.hip)
+int mn_conv16_ws_bytes(const mn_conv2d* g, int direction, size_t* bytes);
+int mn_conv16_fwd(const mn_conv2d* g, const void* x, const void* w, const void* bias, void* y,
+                  hipStream_t s);
+int mn_conv16_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void* dx, void* ws,
+                       size_t ws_bytes, hipStream_t s);
+int mn_conv16_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, void* dw, void* ws,
+                         size_t ws_bytes, hipStream_t s);
+
 namespace mn_conv {
 
 typedef float float16_t __attribute__((ext_vector_type(16)));
@@ -770,8 +779,9 @@ int mn_conv_ws_bytes(const mn_conv2d* g, int direction, int variant, int dtype, 
   *bytes = 0;
   const int st = check(g);
   if (st != MN_OK) return st;
-  if (dtype != MN_F32) return MN_EUNSUPPORTED;
   if (variant < 0 || variant >= mn_conv_n_variants(direction)) return MN_EUNSUPPORTED;
+  if (dtype == MN_BF16) return mn_conv16_ws_bytes(g, direction, bytes);  // same for every variant
+  if (dtype != MN_F32) return MN_EUNSUPPORTED;
   const size_t wsize = (size_t)g->K * g->C * g->R * g->S * sizeof(float);
   // variant 1 of the gather directions: the repacked weight operand (rows padded to 128)
   if (direction == MN_CONV_FWD && variant == 1)
@@ -791,10 +801,11 @@ int mn_conv_fwd(const mn_conv2d* g, const void* x, const void* w, const void* bi
   using namespace mn_conv;
   const int st = check(g);
   if (st != MN_OK) return st;
-  if (dtype != MN_F32) return MN_EUNSUPPORTED;
   if (variant < 0 || variant > 1) return MN_EUNSUPPORTED;
   if (g->N == 0) return MN_OK;
   if (!x || !w || !y) return MN_EINVAL;
+  if (dtype == MN_BF16) return mn_conv16_fwd(g, x, w, bias, y, mn_stream(stream));
+  if (dtype != MN_F32) return MN_EUNSUPPORTED;
   Gather q = {};
   q.M = g->K;
   q.T = g->R * g->S;
@@ -843,11 +854,12 @@ int mn_conv_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void* dx
   using namespace mn_conv;
   const int st = check(g);
   if (st != MN_OK) return st;
-  if (dtype != MN_F32) return MN_EUNSUPPORTED;
   if (variant < 0 || variant > 1) return MN_EUNSUPPORTED;
   if (g->N == 0) return MN_OK;
   if (!dy || !w || !dx) return MN_EINVAL;
   hipStream_t s = mn_stream(stream);
+  if (dtype == MN_BF16) return mn_conv16_bwd_data(g, dy, w, dx, ws, ws_bytes, s);
+  if (dtype != MN_F32) return MN_EUNSUPPORTED;
   const int RS = g->R * g->S;
   const float* a = (const float*)w;
   long long lda = RS, cha = (long long)g->C * RS;  // read w[k][c][r][s] as A(c, k, rs)
@@ -925,10 +937,15 @@ int mn_conv_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, void* 
   using namespace mn_conv;
   const int st = check(g);
   if (st != MN_OK) return st;
-  if (dtype != MN_F32) return MN_EUNSUPPORTED;
+  if (dtype != MN_F32 && dtype != MN_BF16) return MN_EUNSUPPORTED;
   if (variant < 0 || variant > 1) return MN_EUNSUPPORTED;
   if (!dw) return MN_EINVAL;
   hipStream_t s = mn_stream(stream);
+  if (dtype == MN_BF16) {
+    if (g->N == 0) return MN_EUNSUPPORTED;  // nothing to reduce: the caller clears dw itself
+    if (!dy || !x) return MN_EINVAL;
+    return mn_conv16_bwd_weight(g, dy, x, dw, ws, ws_bytes, s);
+  }
   const size_t nw = (size_t)g->K * g->C * g->R * g->S;
   if (g->N == 0) {
     fill_zero_kernel<<<(unsigned)((nw / 4 + kThreads) / kThreads), kThreads, 0, s>>>((float*)dw, nw);

@@ -1,0 +1,617 @@
+// 2-D convolution on bf16 tensors with fp32 accumulation on the gfx950 matrix
+// cores (v_mfma_f32_32x32x16_bf16).
+//
+// Layout: channels-last.  Activations [N, H, W, C], weights [K, R, S, C],
+// outputs [N, P, Q, K] (what torch calls memory_format=channels_last for a
+// logically NCHW tensor).  With the channel innermost, the reduction index of
+// the implicit GEMM is contiguous in memory for BOTH operands of forward and
+// backward-data, which is what the matrix instruction wants: every lane feeds
+// it 8 consecutive reduction elements (16 bytes) per operand, so operand tiles
+// go global -> LDS -> registers as 16-byte vectors with no transposition, and
+// a window shift moves addresses by whole pixels (multiples of 2*C bytes), so
+// taps never break the 16-byte alignment.
+//
+//   forward        D[pix][k] = sum_(tap, c) X[pix @ tap][c] * W[k][tap][c]
+//   backward-data  D[pix][c] = sum_(tap, k) dY[pix @ tap][k] * W'[c][tap][k]
+//                  (W' = weights transposed into the workspace; stride > 1 is
+//                  split by parity class like the fp32 path)
+//   backward-weight dW[k][tap][c] = sum_pix dY[pix][k] * X[pix @ tap][c]
+//                  Here the reduction (pixels) is the STRIDED index, so the
+//                  16-byte chunks (8 channels of one pixel) are scattered into
+//                  LDS as 8 two-byte stores to put pixels innermost.  The
+//                  reduction is split across workgroups; partial sums are fp32
+//                  in the workspace and a second kernel adds them in a fixed
+//                  order and rounds once to bf16.
+//
+// Workgroup = 4 wavefronts (2 x 2); tile 128 rows x BN columns x 32 deep,
+// double buffered in LDS with rows padded to 80 bytes (conflict-free 16-byte
+// reads).  Channel counts must be multiples of 32 (reduction side) or 64
+// (backward-weight columns).
+#include "common.h"
+
+namespace mn_conv16 {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+typedef uint16_t bf16_t;  // storage type
+
+constexpr int kThreads = 256;
+constexpr int BM = 128;     // rows of a workgroup tile (gather kernels)
+constexpr int BK = 32;      // reduction depth of a staged tile
+constexpr int LDK = BK + 8; // LDS row length in elements (80 bytes)
+constexpr int kMaxTaps = 49;
+constexpr uint32_t kNoRow = 0xFFFFFFFFu;
+
+__device__ __forceinline__ bf16_t f2bf(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (bf16_t)((u >> 16) | 0x40u);  // quiet NaN
+  u += 0x7FFFu + ((u >> 16) & 1u);  // round to nearest even
+  return (bf16_t)(u >> 16);
+}
+__device__ __forceinline__ float bf2f(bf16_t h) { return __uint_as_float((uint32_t)h << 16); }
+
+// Row of accumulator register v within a 32x32 MFMA tile (column = lane % 32).
+__device__ __forceinline__ int acc_row(int v, int lane) {
+  return 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+}
+
+// acc[i][j] += A rows (wm-th half) x B rows (wn-th half), both staged [row][k].
+template <int TM, int TN, int ROWS_A, int ROWS_B>
+__device__ __forceinline__ void mma_tile(const bf16_t (*As)[LDK], const bf16_t (*Bs)[LDK], int wm,
+                                         int wn, int lane, float16_t (&acc)[TM][TN]) {
+  const int r = lane & 31, kq = (lane >> 5) * 8;
+#pragma unroll
+  for (int ks = 0; ks < BK; ks += 16) {
+    bf16x8 af[TM], bfr[TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+      af[i] = *reinterpret_cast<const bf16x8*>(&As[wm * (ROWS_A / 2) + 32 * i + r][ks + kq]);
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+      bfr[j] = *reinterpret_cast<const bf16x8*>(&Bs[wn * (ROWS_B / 2) + 32 * j + r][ks + kq]);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+  }
+}
+
+// ---------------------------------------------------- forward / backward-data
+struct GatherH {
+  uint32_t npix;          // rows of this launch = N * OH * OW
+  int OH, OW;
+  int Nout;               // columns = channels of dst
+  int Cs, Hs, Ws;         // source [N, Hs, Ws, Cs]
+  int ish, isw;           // source position = oh*ish + dh[tap]
+  int DH, DW, osh, osw, oh0, ow0;  // dst [N, DH, DW, Nout], position = oh*osh + oh0
+  int T;                  // taps of this launch
+  uint32_t wrow;          // elements between consecutive weight rows
+  int16_t dh[kMaxTaps], dw[kMaxTaps];
+  int32_t woff[kMaxTaps]; // element offset of tap t inside a weight row
+};
+
+template <int BN>
+__global__ __launch_bounds__(kThreads) void gather_bf16_kernel(const GatherH g,
+                                                               const bf16_t* __restrict__ src,
+                                                               const bf16_t* __restrict__ w,
+                                                               const bf16_t* __restrict__ bias,
+                                                               bf16_t* __restrict__ dst) {
+  constexpr int TN = BN / 64;       // MFMA tiles per wavefront along the columns
+  constexpr int kBRows = BN / 64;   // 16-byte chunks of B per thread
+  __shared__ __attribute__((aligned(16))) bf16_t lds_a[2][BM][LDK];
+  __shared__ __attribute__((aligned(16))) bf16_t lds_b[2][BN][LDK];
+  __shared__ int tdh[kMaxTaps], tdw[kMaxTaps], twoff[kMaxTaps];
+  __shared__ uint32_t row_dst[BM];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const uint32_t p0 = blockIdx.x * BM;
+  const int n0 = blockIdx.y * BN;
+  const uint32_t plane = (uint32_t)g.OH * g.OW;
+  if (tid < g.T) {
+    tdh[tid] = g.dh[tid];
+    tdw[tid] = g.dw[tid];
+    twoff[tid] = g.woff[tid];
+  }
+  if (tid < BM) {
+    const uint32_t pix = p0 + tid;
+    uint32_t off = kNoRow;
+    if (pix < g.npix) {
+      const uint32_t n = pix / plane, rem = pix - n * plane;
+      const uint32_t oh = rem / g.OW, ow = rem - oh * g.OW;
+      off = ((n * g.DH + oh * g.osh + g.oh0) * (uint32_t)g.DW + ow * g.osw + g.ow0) * (uint32_t)g.Nout;
+    }
+    row_dst[tid] = off;
+  }
+  // A loader: 16-byte chunk `chunk` of rows arow and arow + 64
+  const int chunk = tid & 3, arow = tid >> 2;
+  int ohs[2], ows[2];
+  uint32_t abase[2];
+  bool aok[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const uint32_t pix = p0 + arow + 64 * i;
+    aok[i] = pix < g.npix;
+    const uint32_t pp = aok[i] ? pix : 0u;
+    const uint32_t n = pp / plane, rem = pp - n * plane;
+    const uint32_t oh = rem / g.OW, ow = rem - oh * g.OW;
+    ohs[i] = oh * g.ish;
+    ows[i] = ow * g.isw;
+    abase[i] = n * (uint32_t)g.Hs * g.Ws;
+  }
+  // B loader: chunk `chunk` of weight rows n0 + arow (+ 64)
+  uint32_t bbase[kBRows];
+  bool bok[kBRows];
+#pragma unroll
+  for (int i = 0; i < kBRows; ++i) {
+    const int col = n0 + arow + 64 * i;
+    bok[i] = col < g.Nout;
+    bbase[i] = (bok[i] ? (uint32_t)col : 0u) * g.wrow + chunk * 8;
+  }
+  __syncthreads();
+
+  uint4_t ra[2], rb[kBRows];
+  bool ra_ok[2];
+  auto fetch = [&](int t, int c0) {  // t, c0 uniform
+    const int dh = tdh[t], dw = tdw[t];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int hh = ohs[i] + dh, ww = ows[i] + dw;
+      ra_ok[i] = aok[i] && (unsigned)hh < (unsigned)g.Hs && (unsigned)ww < (unsigned)g.Ws;
+      const uint32_t e = ra_ok[i] ? (abase[i] + hh * g.Ws + ww) * (uint32_t)g.Cs + c0 + chunk * 8 : 0u;
+      ra[i] = *reinterpret_cast<const uint4_t*>(src + e);
+    }
+    const uint32_t wo = twoff[t] + c0;
+#pragma unroll
+    for (int i = 0; i < kBRows; ++i) rb[i] = *reinterpret_cast<const uint4_t*>(w + bbase[i] + wo);
+  };
+  auto stage = [&](int buf) {
+    const uint4_t z = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      *reinterpret_cast<uint4_t*>(&lds_a[buf][arow + 64 * i][chunk * 8]) = ra_ok[i] ? ra[i] : z;
+#pragma unroll
+    for (int i = 0; i < kBRows; ++i)
+      *reinterpret_cast<uint4_t*>(&lds_b[buf][arow + 64 * i][chunk * 8]) = bok[i] ? rb[i] : z;
+  };
+
+  float16_t acc[2][TN];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  const int per_tap = g.Cs / BK;
+  const int ktiles = g.T * per_tap;
+  if (ktiles > 0) {
+    int t = 0, c0 = 0;
+    auto fetch_next = [&]() {
+      fetch(t, c0);
+      c0 += BK;
+      if (c0 == g.Cs) {
+        c0 = 0;
+        ++t;
+      }
+    };
+    fetch_next();
+    stage(0);
+    __syncthreads();
+    for (int kt = 0; kt < ktiles; ++kt) {
+      const int buf = kt & 1;
+      if (kt + 1 < ktiles) fetch_next();
+      mma_tile<2, TN, BM, BN>(lds_a[buf], lds_b[buf], wm, wn, lane, acc);
+      if (kt + 1 < ktiles) stage(buf ^ 1);
+      __syncthreads();
+    }
+  }
+
+  // epilogue: for a fixed register, lanes 0..31 hold 32 consecutive channels of one position
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int col = n0 + wn * (BN / 2) + 32 * j + (lane & 31);
+    if (col >= g.Nout) continue;
+    const float b = bias ? bf2f(bias[col]) : 0.f;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const uint32_t off = row_dst[wm * 64 + 32 * i + acc_row(v, lane)];
+        if (off != kNoRow) dst[off + col] = f2bf(acc[i][j][v] + b);
+      }
+    }
+  }
+}
+
+// wt[(c*T + t)*K + k] = w[(k*T + t)*C + c]
+__global__ __launch_bounds__(kThreads) void transpose_weights_bf16_kernel(
+    const bf16_t* __restrict__ w, bf16_t* __restrict__ wt, int K, int C, int T) {
+  const size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x;
+  const size_t n = (size_t)K * C * T;
+  if (i >= n) return;
+  const int k = (int)(i % K);
+  const size_t ct = i / K;
+  const int t = (int)(ct % T), c = (int)(ct / T);
+  wt[i] = w[((size_t)k * T + t) * C + c];
+}
+
+__global__ __launch_bounds__(kThreads) void fill_zero_bf16_kernel(bf16_t* p, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < n;
+       i += (size_t)gridDim.x * kThreads)
+    p[i] = 0;
+}
+
+// ------------------------------------------------------------ backward weight
+struct WGradH {
+  int K, C, T, S;            // T = R*S taps
+  int H, W, P, Q;
+  int sH, sW, pH, pW, dH, dW;
+  uint32_t depth;            // N*P*Q
+  uint32_t tiles_per_split;  // 32-position tiles per blockIdx.z
+  int partial;               // 1: fp32 partial[z][K][T][C]; 0: bf16 dw[K][T][C] (single split)
+};
+
+// rows = BMW output channels (k), columns = BNW input channels of ONE tap.
+template <int BMW, int BNW>
+__global__ __launch_bounds__(kThreads) void wgrad_bf16_kernel(const WGradH g,
+                                                              const bf16_t* __restrict__ dy,
+                                                              const bf16_t* __restrict__ x,
+                                                              void* __restrict__ out) {
+  constexpr int TM = BMW / 64, TN = BNW / 64;
+  constexpr int kAChunks = BMW * BK / 8 / kThreads;  // 16-byte chunks per thread and tile
+  constexpr int kBChunks = BNW * BK / 8 / kThreads;
+  __shared__ __attribute__((aligned(16))) bf16_t lds_a[2][BMW][LDK];
+  __shared__ __attribute__((aligned(16))) bf16_t lds_b[2][BNW][LDK];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int m0 = blockIdx.y * BMW;
+  const uint32_t ctiles = (uint32_t)g.C / BNW;
+  const uint32_t tap = blockIdx.x / ctiles;
+  const uint32_t c0 = (blockIdx.x - tap * ctiles) * BNW;
+  const uint32_t r = tap / g.S, sx = tap - r * g.S;
+  const int dh = (int)r * g.dH - g.pH, dw = (int)sx * g.dW - g.pW;
+  const uint32_t PQ = (uint32_t)g.P * g.Q;
+
+  const uint32_t total_tiles = (g.depth + BK - 1) / BK;
+  const uint32_t t_begin = blockIdx.z * g.tiles_per_split;
+  const uint32_t t_end = min(t_begin + g.tiles_per_split, total_tiles);
+
+  // chunk e = tid + kThreads*i of a tile: position e / (rows/8), channel group e % (rows/8)
+  uint32_t a_pos[kAChunks], b_pos[kBChunks];  // position inside the tile
+  uint32_t an[kAChunks], ap[kAChunks], aq[kAChunks];  // (n, p, q) of that position
+  uint32_t bn[kBChunks], bp[kBChunks], bq[kBChunks];
+  auto split = [&](uint32_t d, uint32_t& n, uint32_t& p, uint32_t& q) {
+    n = d / PQ;
+    const uint32_t pq = d - n * PQ;
+    p = pq / g.Q;
+    q = pq - p * g.Q;
+  };
+#pragma unroll
+  for (int i = 0; i < kAChunks; ++i) {
+    a_pos[i] = (tid + kThreads * i) / (BMW / 8);
+    split(t_begin * BK + a_pos[i], an[i], ap[i], aq[i]);
+  }
+#pragma unroll
+  for (int i = 0; i < kBChunks; ++i) {
+    b_pos[i] = (tid + kThreads * i) / (BNW / 8);
+    split(t_begin * BK + b_pos[i], bn[i], bp[i], bq[i]);
+  }
+  auto advance = [&](uint32_t& n, uint32_t& p, uint32_t& q) {  // position += BK
+    q += BK;
+    while (q >= (uint32_t)g.Q) {
+      q -= g.Q;
+      ++p;
+    }
+    while (p >= (uint32_t)g.P) {
+      p -= g.P;
+      ++n;
+    }
+  };
+
+  uint4_t ra[kAChunks], rb[kBChunks];
+  bool ra_ok[kAChunks], rb_ok[kBChunks];
+  auto fetch = [&](uint32_t d0) {
+#pragma unroll
+    for (int i = 0; i < kAChunks; ++i) {
+      const int kc = (tid + kThreads * i) % (BMW / 8);
+      ra_ok[i] = d0 + a_pos[i] < g.depth;
+      const uint32_t e = ra_ok[i] ? ((an[i] * g.P + ap[i]) * (uint32_t)g.Q + aq[i]) * (uint32_t)g.K + m0 + kc * 8 : 0u;
+      ra[i] = *reinterpret_cast<const uint4_t*>(dy + e);
+      advance(an[i], ap[i], aq[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < kBChunks; ++i) {
+      const int cc = (tid + kThreads * i) % (BNW / 8);
+      const int hh = (int)bp[i] * g.sH + dh, ww = (int)bq[i] * g.sW + dw;
+      rb_ok[i] = d0 + b_pos[i] < g.depth && (unsigned)hh < (unsigned)g.H && (unsigned)ww < (unsigned)g.W;
+      const uint32_t e = rb_ok[i] ? ((bn[i] * g.H + hh) * (uint32_t)g.W + ww) * (uint32_t)g.C + c0 + cc * 8 : 0u;
+      rb[i] = *reinterpret_cast<const uint4_t*>(x + e);
+      advance(bn[i], bp[i], bq[i]);
+    }
+  };
+  // scatter a chunk's 8 channels to 8 LDS rows, position innermost
+  auto stage = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < kAChunks; ++i) {
+      const int kc = (tid + kThreads * i) % (BMW / 8);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t wv = ra_ok[i] ? ra[i][j] : 0u;
+        lds_a[buf][kc * 8 + 2 * j][a_pos[i]] = (bf16_t)(wv & 0xFFFFu);
+        lds_a[buf][kc * 8 + 2 * j + 1][a_pos[i]] = (bf16_t)(wv >> 16);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < kBChunks; ++i) {
+      const int cc = (tid + kThreads * i) % (BNW / 8);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t wv = rb_ok[i] ? rb[i][j] : 0u;
+        lds_b[buf][cc * 8 + 2 * j][b_pos[i]] = (bf16_t)(wv & 0xFFFFu);
+        lds_b[buf][cc * 8 + 2 * j + 1][b_pos[i]] = (bf16_t)(wv >> 16);
+      }
+    }
+  };
+
+  float16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  if (t_begin < t_end) {
+    fetch(t_begin * BK);
+    stage(0);
+    __syncthreads();
+    for (uint32_t kt = t_begin; kt < t_end; ++kt) {
+      const int buf = (kt - t_begin) & 1;
+      if (kt + 1 < t_end) fetch((kt + 1) * BK);
+      mma_tile<TM, TN, BMW, BNW>(lds_a[buf], lds_b[buf], wm, wn, lane, acc);
+      if (kt + 1 < t_end) stage(buf ^ 1);
+      __syncthreads();
+    }
+  }
+
+  const size_t row_len = (size_t)g.T * g.C;
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const uint32_t c = c0 + wn * (BNW / 2) + 32 * j + (lane & 31);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = m0 + wm * (BMW / 2) + 32 * i + acc_row(v, lane);
+        const size_t o = (size_t)m * row_len + (size_t)tap * g.C + c;
+        if (g.partial)
+          reinterpret_cast<float*>(out)[(size_t)blockIdx.z * g.K * row_len + o] = acc[i][j][v];
+        else
+          reinterpret_cast<bf16_t*>(out)[o] = f2bf(acc[i][j][v]);
+      }
+    }
+  }
+}
+
+// dw[i] = bf16(sum over splits of partial[z][i]), fixed order
+__global__ __launch_bounds__(kThreads) void wgrad_reduce_bf16_kernel(
+    const float* __restrict__ partial, bf16_t* __restrict__ dw, size_t n, int splits) {
+  const size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x;
+  if (i >= n) return;
+  float s = 0.f;
+  for (int z = 0; z < splits; ++z) s += partial[(size_t)z * n + i];
+  dw[i] = f2bf(s);
+}
+
+// ----------------------------------------------------------------------- host
+static int check16(const mn_conv2d* g) {
+  // every tensor is addressed with 32-bit element offsets
+  const long long lim = 1ll << 31;
+  if ((long long)g->N * g->C * g->H * g->W >= lim || (long long)g->N * g->K * g->P * g->Q >= lim ||
+      (long long)g->K * g->C * g->R * g->S >= lim)
+    return MN_EUNSUPPORTED;
+  if (g->R * g->S > kMaxTaps) return MN_EUNSUPPORTED;
+  return MN_OK;
+}
+
+static void launch_gather16(const GatherH& q, const bf16_t* src, const bf16_t* w, const bf16_t* bias,
+                            bf16_t* dst, hipStream_t s) {
+  if (q.npix == 0 || q.Nout == 0) return;
+  if (q.Nout % 128 == 0) {
+    dim3 grid((q.npix + BM - 1) / BM, q.Nout / 128);
+    gather_bf16_kernel<128><<<grid, kThreads, 0, s>>>(q, src, w, bias, dst);
+  } else {
+    dim3 grid((q.npix + BM - 1) / BM, (q.Nout + 63) / 64);
+    gather_bf16_kernel<64><<<grid, kThreads, 0, s>>>(q, src, w, bias, dst);
+  }
+}
+
+static void wgrad16_tiles(const mn_conv2d* g, int* bm, int* bn) {
+  *bm = g->K % 128 == 0 ? 128 : 64;
+  *bn = g->C % 128 == 0 ? 128 : 64;
+}
+
+static void wgrad16_split(const mn_conv2d* g, int* splits, int* tiles_per_split) {
+  int bm, bn;
+  wgrad16_tiles(g, &bm, &bn);
+  const long long depth = (long long)g->N * g->P * g->Q;
+  const long long total_tiles = (depth + BK - 1) / BK;
+  const long long out_tiles = (long long)g->R * g->S * (g->C / bn) * (g->K / bm);
+  long long want = (1024 + out_tiles - 1) / out_tiles;
+  if (want > total_tiles) want = total_tiles;
+  if (want > 128) want = 128;
+  if (want < 1) want = 1;
+  const long long tps = (total_tiles + want - 1) / want;
+  *tiles_per_split = (int)(tps < 1 ? 1 : tps);
+  *splits = (int)((total_tiles + *tiles_per_split - 1) / (*tiles_per_split));
+  if (*splits < 1) *splits = 1;
+}
+
+}  // namespace mn_conv16
+
+// Entry points used by the dtype dispatch in conv.hip.
+int mn_conv16_ws_bytes(const mn_conv2d* g, int direction, size_t* bytes) {
+  using namespace mn_conv16;
+  *bytes = 0;
+  const int st = check16(g);
+  if (st != MN_OK) return st;
+  if (direction == MN_CONV_FWD) return g->C % BK == 0 ? MN_OK : MN_EUNSUPPORTED;
+  if (direction == MN_CONV_BWD_DATA) {
+    if (g->K % BK != 0) return MN_EUNSUPPORTED;
+    *bytes = (size_t)g->K * g->C * g->R * g->S * sizeof(bf16_t);
+    return MN_OK;
+  }
+  if (g->K % 64 != 0 || g->C % 64 != 0) return MN_EUNSUPPORTED;
+  int splits, tps;
+  wgrad16_split(g, &splits, &tps);
+  if (splits > 1) *bytes = (size_t)splits * g->K * g->C * g->R * g->S * sizeof(float);
+  return MN_OK;
+}
+
+int mn_conv16_fwd(const mn_conv2d* g, const void* x, const void* w, const void* bias, void* y,
+                  hipStream_t s) {
+  using namespace mn_conv16;
+  const int st = check16(g);
+  if (st != MN_OK) return st;
+  if (g->C % BK != 0) return MN_EUNSUPPORTED;
+  if (!mn_aligned(x, 16) || !mn_aligned(w, 16)) return MN_EINVAL;
+  GatherH q = {};
+  q.npix = (uint32_t)((long long)g->N * g->P * g->Q);
+  q.OH = g->P;
+  q.OW = g->Q;
+  q.Nout = g->K;
+  q.Cs = g->C;
+  q.Hs = g->H;
+  q.Ws = g->W;
+  q.ish = g->sH;
+  q.isw = g->sW;
+  q.DH = g->P;
+  q.DW = g->Q;
+  q.osh = q.osw = 1;
+  q.T = g->R * g->S;
+  q.wrow = (uint32_t)q.T * g->C;
+  for (int r = 0; r < g->R; ++r)
+    for (int sx = 0; sx < g->S; ++sx) {
+      const int t = r * g->S + sx;
+      q.dh[t] = (int16_t)(r * g->dH - g->pH);
+      q.dw[t] = (int16_t)(sx * g->dW - g->pW);
+      q.woff[t] = t * g->C;
+    }
+  launch_gather16(q, (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias, (bf16_t*)y, s);
+  return mn_launch_status();
+}
+
+int mn_conv16_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void* dx, void* ws,
+                       size_t ws_bytes, hipStream_t s) {
+  using namespace mn_conv16;
+  const int st = check16(g);
+  if (st != MN_OK) return st;
+  if (g->K % BK != 0) return MN_EUNSUPPORTED;
+  const int T = g->R * g->S;
+  const size_t nw = (size_t)g->K * g->C * T;
+  if (!ws || ws_bytes < nw * sizeof(bf16_t) || !mn_aligned(ws, 16) || !mn_aligned(dy, 16))
+    return MN_EINVAL;
+  transpose_weights_bf16_kernel<<<(unsigned)((nw + kThreads - 1) / kThreads), kThreads, 0, s>>>(
+      (const bf16_t*)w, (bf16_t*)ws, g->K, g->C, T);
+  bool empty_class = false;
+  for (int ca = 0; ca < g->sH && !empty_class; ++ca) {
+    bool any = false;
+    for (int r = 0; r < g->R; ++r) any |= (r * g->dH) % g->sH == ca;
+    empty_class |= !any;
+  }
+  for (int cb = 0; cb < g->sW && !empty_class; ++cb) {
+    bool any = false;
+    for (int sx = 0; sx < g->S; ++sx) any |= (sx * g->dW) % g->sW == cb;
+    empty_class |= !any;
+  }
+  if (empty_class) {
+    const size_t n = (size_t)g->N * g->C * g->H * g->W;
+    fill_zero_bf16_kernel<<<2048, kThreads, 0, s>>>((bf16_t*)dx, n);
+  }
+  for (int ca = 0; ca < g->sH; ++ca) {
+    for (int cb = 0; cb < g->sW; ++cb) {
+      GatherH q = {};
+      q.oh0 = ((ca - g->pH) % g->sH + g->sH) % g->sH;
+      q.ow0 = ((cb - g->pW) % g->sW + g->sW) % g->sW;
+      q.OH = q.oh0 < g->H ? (g->H - q.oh0 + g->sH - 1) / g->sH : 0;
+      q.OW = q.ow0 < g->W ? (g->W - q.ow0 + g->sW - 1) / g->sW : 0;
+      int Tc = 0;
+      for (int r = 0; r < g->R; ++r) {
+        if ((r * g->dH) % g->sH != ca) continue;
+        for (int sx = 0; sx < g->S; ++sx) {
+          if ((sx * g->dW) % g->sW != cb) continue;
+          q.dh[Tc] = (int16_t)((q.oh0 + g->pH - r * g->dH) / g->sH);
+          q.dw[Tc] = (int16_t)((q.ow0 + g->pW - sx * g->dW) / g->sW);
+          q.woff[Tc] = (r * g->S + sx) * g->K;
+          ++Tc;
+        }
+      }
+      if (Tc == 0) continue;  // cleared above
+      q.T = Tc;
+      q.npix = (uint32_t)((long long)g->N * q.OH * q.OW);
+      q.Nout = g->C;
+      q.Cs = g->K;
+      q.Hs = g->P;
+      q.Ws = g->Q;
+      q.ish = q.isw = 1;
+      q.DH = g->H;
+      q.DW = g->W;
+      q.osh = g->sH;
+      q.osw = g->sW;
+      q.wrow = (uint32_t)T * g->K;
+      launch_gather16(q, (const bf16_t*)dy, (const bf16_t*)ws, nullptr, (bf16_t*)dx, s);
+    }
+  }
+  return mn_launch_status();
+}
+
+int mn_conv16_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, void* dw, void* ws,
+                         size_t ws_bytes, hipStream_t s) {
+  using namespace mn_conv16;
+  const int st = check16(g);
+  if (st != MN_OK) return st;
+  if (g->K % 64 != 0 || g->C % 64 != 0) return MN_EUNSUPPORTED;
+  if (!mn_aligned(dy, 16) || !mn_aligned(x, 16)) return MN_EINVAL;
+  WGradH q = {};
+  q.K = g->K;
+  q.C = g->C;
+  q.T = g->R * g->S;
+  q.S = g->S;
+  q.H = g->H;
+  q.W = g->W;
+  q.P = g->P;
+  q.Q = g->Q;
+  q.sH = g->sH;
+  q.sW = g->sW;
+  q.pH = g->pH;
+  q.pW = g->pW;
+  q.dH = g->dH;
+  q.dW = g->dW;
+  q.depth = (uint32_t)((long long)g->N * g->P * g->Q);
+  int splits, tps, bm, bn;
+  wgrad16_split(g, &splits, &tps);
+  wgrad16_tiles(g, &bm, &bn);
+  q.tiles_per_split = tps;
+  q.partial = splits > 1;
+  const size_t nw = (size_t)g->K * g->C * q.T;
+  void* out = dw;
+  if (q.partial) {
+    if (!ws || ws_bytes < nw * sizeof(float) * splits || !mn_aligned(ws, 4)) return MN_EINVAL;
+    out = ws;
+  }
+  dim3 grid(q.T * (g->C / bn), g->K / bm, splits);
+  if (bm == 128 && bn == 128)
+    wgrad_bf16_kernel<128, 128><<<grid, kThreads, 0, s>>>(q, (const bf16_t*)dy, (const bf16_t*)x, out);
+  else if (bm == 128)
+    wgrad_bf16_kernel<128, 64><<<grid, kThreads, 0, s>>>(q, (const bf16_t*)dy, (const bf16_t*)x, out);
+  else if (bn == 128)
+    wgrad_bf16_kernel<64, 128><<<grid, kThreads, 0, s>>>(q, (const bf16_t*)dy, (const bf16_t*)x, out);
+  else
+    wgrad_bf16_kernel<64, 64><<<grid, kThreads, 0, s>>>(q, (const bf16_t*)dy, (const bf16_t*)x, out);
+  if (q.partial)
+    wgrad_reduce_bf16_kernel<<<(unsigned)((nw + kThreads - 1) / kThreads), kThreads, 0, s>>>(
+        (const float*)ws, (bf16_t*)dw, nw, splits);
+  return mn_launch_status();
+}

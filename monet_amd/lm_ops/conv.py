@@ -62,55 +62,86 @@ def n_bwd_wt_algos():
     return _lib.load().mn_conv_n_variants(_lib.CONV_BWD_WEIGHT)
 
 
-def _workspace(geo, direction, variant, device):
+def _workspace(geo, direction, variant, device, dtype=None):
     n = ctypes.c_size_t(0)
-    _lib.call("mn_conv_ws_bytes", geo, direction, variant, _lib.F32, ctypes.byref(n))
+    _lib.call("mn_conv_ws_bytes", geo, direction, variant, _lib.F32 if dtype is None else dtype,
+              ctypes.byref(n))
     if n.value == 0:
         return None, 0
     return torch.empty(n.value, dtype=torch.uint8, device=device), n.value
 
 
 def _prep(t, name):
-    _lib.require_gpu_tensor(t, name, torch.float32)
+    """(tensor the kernels can read, library dtype code).  fp32 tensors are used as dense
+    NCHW; bf16 tensors as channels-last (NHWC memory under the same logical shape)."""
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        _lib.require_gpu_tensor(t, name)
     t = t.detach()
-    return t if t.is_contiguous() else t.contiguous()
+    if t.dtype == torch.bfloat16:
+        if t.dim() == 4:
+            t = t.contiguous(memory_format=torch.channels_last)
+        elif not t.is_contiguous():
+            t = t.contiguous()
+        return t, _lib.BF16
+    _lib.require_gpu_tensor(t, name, torch.float32)
+    return (t if t.is_contiguous() else t.contiguous()), _lib.F32
+
+
+def _same_dtype(*codes):
+    if len(set(codes)) != 1:
+        raise RuntimeError("convolution operands must share one dtype (all fp32 or all bf16)")
+    return codes[0]
+
+
+def _empty(shape, code, device):
+    shape = [int(d) for d in shape]
+    if code == _lib.BF16:
+        return torch.empty(shape, dtype=torch.bfloat16, device=device,
+                           memory_format=torch.channels_last)
+    return torch.empty(shape, dtype=torch.float32, device=device)
 
 
 def conv_forward(input_, weight, bias, padding, stride, dilation, groups, variant):
     """y = conv2d(input, weight) (+ bias) with kernel variant `variant`."""
-    x, w = _prep(input_, "input"), _prep(weight, "weight")
-    b = None if bias is None else _prep(bias, "bias")
+    (x, cx), (w, cw) = _prep(input_, "input"), _prep(weight, "weight")
+    code = _same_dtype(cx, cw)
+    b = None
+    if bias is not None:
+        b, cb = _prep(bias, "bias")
+        _same_dtype(code, cb)
     geo = conv_geometry(x.shape, w.shape, stride, padding, dilation, groups)
-    ws, nbytes = _workspace(geo, _lib.CONV_FWD, variant, x.device)
-    y = torch.empty((geo.N, geo.K, geo.P, geo.Q), dtype=torch.float32, device=x.device)
+    ws, nbytes = _workspace(geo, _lib.CONV_FWD, variant, x.device, code)
+    y = _empty((geo.N, geo.K, geo.P, geo.Q), code, x.device)
     _lib.call("mn_conv_fwd", geo, _lib.ptr(x), _lib.ptr(w), _lib.ptr(b), _lib.ptr(y), _lib.ptr(ws),
-              nbytes, variant, _lib.F32, _lib.stream_ptr(x.device))
+              nbytes, variant, code, _lib.stream_ptr(x.device))
     return y
 
 
 def conv_backward_input(input_shape, grad_output, weight, padding, stride, dilation, groups,
                         variant):
-    g, w = _prep(grad_output, "grad_output"), _prep(weight, "weight")
+    (g, cg), (w, cw) = _prep(grad_output, "grad_output"), _prep(weight, "weight")
+    code = _same_dtype(cg, cw)
     geo = conv_geometry(input_shape, w.shape, stride, padding, dilation, groups)
     if tuple(g.shape) != (geo.N, geo.K, geo.P, geo.Q):
         raise RuntimeError("grad_output does not match the convolution geometry")
-    ws, nbytes = _workspace(geo, _lib.CONV_BWD_DATA, variant, g.device)
-    dx = torch.empty([int(d) for d in input_shape], dtype=torch.float32, device=g.device)
+    ws, nbytes = _workspace(geo, _lib.CONV_BWD_DATA, variant, g.device, code)
+    dx = _empty(input_shape, code, g.device)
     _lib.call("mn_conv_bwd_data", geo, _lib.ptr(g), _lib.ptr(w), _lib.ptr(dx), _lib.ptr(ws), nbytes,
-              variant, _lib.F32, _lib.stream_ptr(g.device))
+              variant, code, _lib.stream_ptr(g.device))
     return dx
 
 
 def conv_backward_weight(weight_shape, grad_output, input_, padding, stride, dilation, groups,
                          variant):
-    g, x = _prep(grad_output, "grad_output"), _prep(input_, "input")
+    (g, cg), (x, cx) = _prep(grad_output, "grad_output"), _prep(input_, "input")
+    code = _same_dtype(cg, cx)
     geo = conv_geometry(x.shape, weight_shape, stride, padding, dilation, groups)
     if tuple(g.shape) != (geo.N, geo.K, geo.P, geo.Q):
         raise RuntimeError("grad_output does not match the convolution geometry")
-    ws, nbytes = _workspace(geo, _lib.CONV_BWD_WEIGHT, variant, g.device)
-    dw = torch.empty([int(d) for d in weight_shape], dtype=torch.float32, device=g.device)
+    ws, nbytes = _workspace(geo, _lib.CONV_BWD_WEIGHT, variant, g.device, code)
+    dw = _empty(weight_shape, code, g.device)
     _lib.call("mn_conv_bwd_weight", geo, _lib.ptr(g), _lib.ptr(x), _lib.ptr(dw), _lib.ptr(ws),
-              nbytes, variant, _lib.F32, _lib.stream_ptr(g.device))
+              nbytes, variant, code, _lib.stream_ptr(g.device))
     return dw
 
 

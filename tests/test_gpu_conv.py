@@ -167,3 +167,70 @@ def test_depthwise_passthrough(cuda):
     di, dw = op.backward(g, [x.detach(), w.detach()])
     torch.testing.assert_close(di, x.grad)
     torch.testing.assert_close(dw, w.grad)
+
+
+# ------------------------------------------------------------------ bf16 path
+# bf16 channels-last tensors, bf16 matrix cores, fp32 accumulation: inputs are rounded to
+# bf16 first and the float64 oracle runs on the ROUNDED values, so what is left is the
+# accumulation order and the single rounding of the output: 2^-9 of the value at worst,
+# checked at 1e-2 of the tensor's scale as the configuration states (a wrong operand layout
+# or tap table gives errors of order 1).
+BF16_TOL = 1e-2
+BF16_CASES = [
+    ((4, 64, 14, 14), (128, 64, 3, 3), 1, 1, 1),
+    ((3, 128, 9, 11), (64, 128, 3, 3), 2, 1, 1),        # strided, odd sizes, ragged row tiles
+    ((2, 64, 8, 8), (64, 64, 1, 1), 1, 0, 1),
+    ((2, 64, 9, 9), (192, 64, 1, 1), 2, 0, 1),          # parity classes no tap reaches; K % 128 != 0
+    ((1, 64, 11, 11), (64, 64, 3, 3), 1, 2, 2),         # dilation
+    ((2, 128, 7, 9), (128, 128, 2, 3), (2, 1), (1, 0), 1),
+    ((8, 256, 14, 14), (256, 256, 3, 3), 1, 1, 1),      # ResNet-50 layer3 shape at a small batch
+    ((2, 64, 56, 56), (256, 64, 1, 1), 1, 0, 1),
+]
+
+
+def bf16_round(a):
+    return torch.from_numpy(np.ascontiguousarray(a, np.float32)).to(torch.bfloat16).float().numpy()
+
+
+def dev16(a, cuda):
+    t = torch.from_numpy(np.ascontiguousarray(a, np.float32)).to(cuda).to(torch.bfloat16)
+    return t.contiguous(memory_format=torch.channels_last) if t.dim() == 4 else t
+
+
+@pytest.mark.parametrize("xs,ws,st,pad,dil", BF16_CASES)
+def test_conv_bf16_all_directions(cuda, xs, ws, st, pad, dil):
+    x, w, b = problem(xs, ws, seed=3)
+    x, w, b = bf16_round(x), bf16_round(w), bf16_round(b)
+    exp = O.conv_fwd(x, w, b, st, pad, dil)
+    rng = np.random.default_rng(5)
+    dy = bf16_round(rng.standard_normal(exp.shape))
+    for v in range(conv_ops.n_fwd_algos()):
+        y = conv_ops.conv_forward(dev16(x, cuda), dev16(w, cuda), dev16(b, cuda), pad, st, dil, 1, v)
+        assert y.dtype == torch.bfloat16 and y.is_contiguous(memory_format=torch.channels_last)
+        assert_rel(host(y.float()), exp, BF16_TOL, f"bf16 forward variant {v}")
+    y = conv_ops.conv_forward(dev16(x, cuda), dev16(w, cuda), None, pad, st, dil, 1, 0)
+    assert_rel(host(y.float()), O.conv_fwd(x, w, None, st, pad, dil), BF16_TOL, "bf16 forward, no bias")
+    exp_dx = O.conv_bwd_data(dy, w, xs, st, pad, dil)
+    for v in range(conv_ops.n_bwd_ip_algos()):
+        dx = conv_ops.conv_backward_input(xs, dev16(dy, cuda), dev16(w, cuda), pad, st, dil, 1, v)
+        assert dx.dtype == torch.bfloat16 and list(dx.shape) == list(xs)
+        assert_rel(host(dx.float()), exp_dx, BF16_TOL, f"bf16 backward-data variant {v}")
+    exp_dw = O.conv_bwd_weight(dy, x, ws, st, pad, dil)
+    for v in range(conv_ops.n_bwd_wt_algos()):
+        dw = conv_ops.conv_backward_weight(ws, dev16(dy, cuda), dev16(x, cuda), pad, st, dil, 1, v)
+        assert dw.dtype == torch.bfloat16 and list(dw.shape) == list(ws)
+        assert_rel(host(dw.float()), exp_dw, BF16_TOL, f"bf16 backward-weight variant {v}")
+    # reproducible: fixed-order reduction of the split partials
+    dw2 = conv_ops.conv_backward_weight(ws, dev16(dy, cuda), dev16(x, cuda), pad, st, dil, 1, 0)
+    assert torch.equal(dw, dw2)
+
+
+def test_conv_bf16_rejects_channel_counts_the_tiles_cannot_hold(cuda):
+    from monet_amd import _lib
+    x = torch.randn(1, 3, 8, 8, device=cuda).to(torch.bfloat16)
+    w = torch.randn(64, 3, 3, 3, device=cuda).to(torch.bfloat16)
+    with pytest.raises(_lib.MonetHipError) as e:
+        conv_ops.conv_forward(x, w, None, 1, 1, 1, 1, 0)
+    assert e.value.status == _lib.MN_EUNSUPPORTED
+    with pytest.raises(RuntimeError):
+        conv_ops.conv_forward(x, w.float(), None, 1, 1, 1, 1, 0)   # mixed dtypes
