@@ -17,8 +17,9 @@
 //                  split by parity class like the fp32 path)
 //   backward-weight dW[k][tap][c] = sum_pix dY[pix][k] * X[pix @ tap][c]
 //                  Here the reduction (pixels) is the STRIDED index, so the
-//                  16-byte chunks (8 channels of one pixel) are scattered into
-//                  LDS as 8 two-byte stores to put pixels innermost.  The
+//                  16-byte chunks (8 channels of one pixel) are transposed on
+//                  their way into LDS (lane-pair exchange + dword stores) to
+//                  put pixels innermost.  The
 //                  reduction is split across workgroups; partial sums are fp32
 //                  in the workspace and a second kernel adds them in a fixed
 //                  order and rounds once to bf16.
@@ -278,7 +279,10 @@ __global__ __launch_bounds__(kThreads) void wgrad_bf16_kernel(const WGradH g,
   const uint32_t t_begin = blockIdx.z * g.tiles_per_split;
   const uint32_t t_end = min(t_begin + g.tiles_per_split, total_tiles);
 
-  // chunk e = tid + kThreads*i of a tile: position e / (rows/8), channel group e % (rows/8)
+  // chunk e = tid + kThreads*i of a tile: position e % BK, channel group e / BK.  Consecutive
+  // lanes take consecutive positions so that their two-byte LDS stores fall into different
+  // banks (8 rows apart is a multiple of all 32 banks); the loads of a channel group's
+  // neighbours come from the same cache lines a moment later.
   uint32_t a_pos[kAChunks], b_pos[kBChunks];  // position inside the tile
   uint32_t an[kAChunks], ap[kAChunks], aq[kAChunks];  // (n, p, q) of that position
   uint32_t bn[kBChunks], bp[kBChunks], bq[kBChunks];
@@ -290,12 +294,12 @@ __global__ __launch_bounds__(kThreads) void wgrad_bf16_kernel(const WGradH g,
   };
 #pragma unroll
   for (int i = 0; i < kAChunks; ++i) {
-    a_pos[i] = (tid + kThreads * i) / (BMW / 8);
+    a_pos[i] = (tid + kThreads * i) % BK;
     split(t_begin * BK + a_pos[i], an[i], ap[i], aq[i]);
   }
 #pragma unroll
   for (int i = 0; i < kBChunks; ++i) {
-    b_pos[i] = (tid + kThreads * i) / (BNW / 8);
+    b_pos[i] = (tid + kThreads * i) % BK;
     split(t_begin * BK + b_pos[i], bn[i], bp[i], bq[i]);
   }
   auto advance = [&](uint32_t& n, uint32_t& p, uint32_t& q) {  // position += BK
@@ -315,7 +319,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_bf16_kernel(const WGradH g,
   auto fetch = [&](uint32_t d0) {
 #pragma unroll
     for (int i = 0; i < kAChunks; ++i) {
-      const int kc = (tid + kThreads * i) % (BMW / 8);
+      const int kc = (tid + kThreads * i) / BK;
       ra_ok[i] = d0 + a_pos[i] < g.depth;
       const uint32_t e = ra_ok[i] ? ((an[i] * g.P + ap[i]) * (uint32_t)g.Q + aq[i]) * (uint32_t)g.K + m0 + kc * 8 : 0u;
       ra[i] = *reinterpret_cast<const uint4_t*>(dy + e);
@@ -323,7 +327,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_bf16_kernel(const WGradH g,
     }
 #pragma unroll
     for (int i = 0; i < kBChunks; ++i) {
-      const int cc = (tid + kThreads * i) % (BNW / 8);
+      const int cc = (tid + kThreads * i) / BK;
       const int hh = (int)bp[i] * g.sH + dh, ww = (int)bq[i] * g.sW + dw;
       rb_ok[i] = d0 + b_pos[i] < g.depth && (unsigned)hh < (unsigned)g.H && (unsigned)ww < (unsigned)g.W;
       const uint32_t e = rb_ok[i] ? ((bn[i] * g.H + hh) * (uint32_t)g.W + ww) * (uint32_t)g.C + c0 + cc * 8 : 0u;
@@ -331,28 +335,28 @@ __global__ __launch_bounds__(kThreads) void wgrad_bf16_kernel(const WGradH g,
       advance(bn[i], bp[i], bq[i]);
     }
   };
-  // scatter a chunk's 8 channels to 8 LDS rows, position innermost
+  // Transposing store: a chunk holds 8 channels of one position, LDS wants positions
+  // innermost.  Neighbouring lanes hold neighbouring positions, so a lane pair first swaps
+  // halves (DPP): the even lane ends up with channel 2j of both positions, the odd lane with
+  // channel 2j+1, and each writes 4 full dwords instead of 8 two-byte pieces.
+  const bool odd = tid & 1;
+  auto scatter = [&](bf16_t (*dstp)[LDK], int group, uint32_t pos, const uint4_t& v, bool ok) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t own = ok ? v[j] : 0u;
+      const uint32_t other = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)own, 0xB1, 0xF, 0xF, true);
+      const uint32_t word = odd ? ((other >> 16) | (own & 0xFFFF0000u))
+                                : ((own & 0xFFFFu) | (other << 16));
+      *reinterpret_cast<uint32_t*>(&dstp[group * 8 + 2 * j + (odd ? 1 : 0)][pos & ~1u]) = word;
+    }
+  };
   auto stage = [&](int buf) {
 #pragma unroll
-    for (int i = 0; i < kAChunks; ++i) {
-      const int kc = (tid + kThreads * i) % (BMW / 8);
+    for (int i = 0; i < kAChunks; ++i)
+      scatter(lds_a[buf], (tid + kThreads * i) / BK, a_pos[i], ra[i], ra_ok[i]);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const uint32_t wv = ra_ok[i] ? ra[i][j] : 0u;
-        lds_a[buf][kc * 8 + 2 * j][a_pos[i]] = (bf16_t)(wv & 0xFFFFu);
-        lds_a[buf][kc * 8 + 2 * j + 1][a_pos[i]] = (bf16_t)(wv >> 16);
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < kBChunks; ++i) {
-      const int cc = (tid + kThreads * i) % (BNW / 8);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const uint32_t wv = rb_ok[i] ? rb[i][j] : 0u;
-        lds_b[buf][cc * 8 + 2 * j][b_pos[i]] = (bf16_t)(wv & 0xFFFFu);
-        lds_b[buf][cc * 8 + 2 * j + 1][b_pos[i]] = (bf16_t)(wv >> 16);
-      }
-    }
+    for (int i = 0; i < kBChunks; ++i)
+      scatter(lds_b[buf], (tid + kThreads * i) / BK, b_pos[i], rb[i], rb_ok[i]);
   };
 
   float16_t acc[TM][TN];
