@@ -312,6 +312,7 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
   }
 
   // epilogue: lane owns columns (nj*32 + lane%32) and 16 rows per MFMA tile
+  const bool dense = g.osh == 1 && g.osw == 1;
 #pragma unroll
   for (int nj = 0; nj < TL::TN; ++nj) {
     const uint32_t c = n0 + wn * (TL::TN * 32) + nj * 32 + (lane & 31);
@@ -330,7 +331,13 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
         if (m < g.M) {
           float r = acc[mi][nj][v];
           if (bias) r += bias[m];
-          out[(size_t)m * plane] = r;
+          // a dense output is written once and not read by this kernel: keep it out of the
+          // caches the operand tiles live in; strided (parity-class) outputs share cache lines
+          // between launches and are better left to the cache
+          if (dense)
+            st_stream(&out[(size_t)m * plane], r);
+          else
+            out[(size_t)m * plane] = r;
         }
       }
     }
