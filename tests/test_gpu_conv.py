@@ -234,3 +234,22 @@ def test_conv_bf16_rejects_channel_counts_the_tiles_cannot_hold(cuda):
     assert e.value.status == _lib.MN_EUNSUPPORTED
     with pytest.raises(RuntimeError):
         conv_ops.conv_forward(x, w.float(), None, 1, 1, 1, 1, 0)   # mixed dtypes
+
+
+def test_conv_bf16_channel_counts_that_only_fit_the_shallow_tiles(cuda):
+    """C = 96 and K = 32 are multiples of 32 but not 64: forward and backward-data stage
+    32-deep tiles there; backward-weight needs multiples of 64 and must say so."""
+    from monet_amd import _lib
+    xs, ws, st, pad, dil = (2, 96, 10, 10), (32, 96, 3, 3), 1, 1, 1
+    x, w, b = problem(xs, ws, seed=7)
+    x, w = bf16_round(x), bf16_round(w)
+    exp = O.conv_fwd(x, w, None, st, pad, dil)
+    y = conv_ops.conv_forward(dev16(x, cuda), dev16(w, cuda), None, pad, st, dil, 1, 0)
+    assert_rel(host(y.float()), exp, BF16_TOL, "bf16 forward, 32-deep tiles")
+    dy = bf16_round(np.random.default_rng(8).standard_normal(exp.shape))
+    dx = conv_ops.conv_backward_input(xs, dev16(dy, cuda), dev16(w, cuda), pad, st, dil, 1, 0)
+    assert_rel(host(dx.float()), O.conv_bwd_data(dy, w, xs, st, pad, dil), BF16_TOL,
+               "bf16 backward-data, 32-deep tiles")
+    with pytest.raises(_lib.MonetHipError) as e:
+        conv_ops.conv_backward_weight(ws, dev16(dy, cuda), dev16(x, cuda), pad, st, dil, 1, 0)
+    assert e.value.status == _lib.MN_EUNSUPPORTED
