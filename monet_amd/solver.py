@@ -95,7 +95,8 @@ class _Builder:
 
 class Model:
     def __init__(self, si: SolverInfo, budget, time_limit=86400, solver="HIGHS", ablation=False,
-                 mip_rel_gap=0.01, verbose=False, presolve=True, recompute_window=None):
+                 mip_rel_gap=0.01, verbose=False, presolve=True, recompute_window=None,
+                 excess_price=EXCESS_PRICE, accept_up_to=None):
         self.si = si
         self.budget = budget
         self.time_limit = time_limit
@@ -105,6 +106,9 @@ class Model:
         self.verbose = verbose
         self.presolve = presolve
         self.recompute_window = recompute_window
+        self.excess_price = excess_price
+        # a schedule is accepted if its peak is within this many GB (default: the budget)
+        self.accept_up_to = budget if accept_up_to is None else accept_up_to
         n = si.nodes
         self.ram = np.array([math.ceil(n[i].mem * MEM_GCD_MULTIPLIER / 1024) for i in n])  # KB
         scale = lambda vals: [math.ceil(v * CPU_GCD_MULTIPLIER) for v in vals]
@@ -398,7 +402,7 @@ class Model:
             const_cost = 0.0
         else:
             total = sum(abs(c) for v, c in obj) + 1.0
-            obj = obj + [(excess, EXCESS_PRICE * total / float(self.budget))]
+            obj = obj + [(excess, self.excess_price * total / float(self.budget))]
         B.minimise(obj)
 
         # ---- solve
@@ -422,7 +426,9 @@ class Model:
         if res.x is None:
             raise ValueError("Model infeasible" if res.status == 2 else
                              f"no schedule found: {res.message}")
-        if excess is not None and res.x[excess] > EXCESS_TOLERANCE * self.budget:
+        self.last_excess = float(res.x[excess]) if excess is not None else 0.0
+        if excess is not None and \
+                self.budget + res.x[excess] > self.accept_up_to * (1.0 + EXCESS_TOLERANCE):
             raise ValueError("Model infeasible: the cheapest schedule found needs %.3f GB, budget "
                              "%.3f GB" % (self.budget + res.x[excess], self.budget))
         x = np.around(res.x)
@@ -440,12 +446,45 @@ class Model:
         rf = np.zeros((T, len(conv), max(n_algos, 1)), dtype=np.uint8)
         for (c, t, k), v in RF.items():
             rf[t, k, c] = x[v]
-        solution = Solution(r, s, m, rf, ip, pp, solve_time, float("nan"), float("nan"),
-                            float(res.fun + const_cost))
+        run_time = float(res.fun + const_cost)
+        if excess is not None:  # without what an accepted overshoot of the target was charged
+            run_time -= float(cvec[excess] * res.x[excess])
+        solution = Solution(r, s, m, rf, ip, pp, solve_time, float("nan"), float("nan"), run_time)
         if out_file is not None:
             with open(out_file, 'wb') as f:
                 pickle.dump([si, solution], f)
         return solution
+
+
+def solve_within_budget(si, budget, time_limit=86400, solver="HIGHS", ablation=False,
+                        out_file=None, rounds=6, **options):
+    """Model(si, budget).solve(), with a fallback for tight budgets.  HiGHS can spend its whole
+    time limit without an incumbent when every schedule it tries overshoots a tight budget at
+    the (deliberately prohibitive) default price.  The fallback solves the same model against
+    a slightly LOWER target with a MODERATE price on the overshoot - any schedule is then an
+    acceptable incumbent and the price steers the search - and tightens the target until a
+    schedule fits the real budget.  What comes out fits the budget; it need not be optimal."""
+    per_solve = max(30.0, time_limit / (rounds + 1.0))
+    try:
+        return Model(si, budget, per_solve if rounds else time_limit, solver, ablation,
+                     **options).solve(out_file=out_file)
+    except ValueError as e:
+        if "cheapest schedule found" not in str(e) or not rounds:
+            raise
+        first_error = e
+    target, price = float(budget), 4.0
+    for _ in range(rounds):
+        m = Model(si, target, per_solve, solver, ablation, excess_price=price,
+                  accept_up_to=budget, **options)
+        try:
+            return m.solve(out_file=out_file)  # fits the real budget (it may overshoot the target)
+        except ValueError as e:
+            if "cheapest schedule found" not in str(e):
+                raise
+        # aim lower by what was missing and make overshooting dearer
+        target = max(0.5 * budget, target - 1.5 * (target + m.last_excess - budget))
+        price *= 3.0
+    raise first_error
 
 
 def solution_file_name(model_name, bs, mode, budget):
@@ -500,10 +539,10 @@ def main(argv=None):
             return None
     print("Memory budget", args.budget, "GB; batch size", si.bs, "; model", model_name,
           "; mode", args.mode)
-    solver_model = Model(si, args.budget, args.time_limit, args.solver, args.ablation,
-                         mip_rel_gap=args.gap, verbose=args.verbose, recompute_window=args.window)
     out = Path(args.data_dir) / solution_file_name(model_name, si.bs, args.mode, args.budget)
-    solution = solver_model.solve(out_file=str(out))
+    solution = solve_within_budget(si, args.budget, args.time_limit, args.solver, args.ablation,
+                                   out_file=str(out), mip_rel_gap=args.gap, verbose=args.verbose,
+                                   recompute_window=args.window)
     print("solved in %.1f s, expected run time %.2f ms -> %s" % (
         solution.solve_time, solution.runtime_expected / CPU_GCD_MULTIPLIER, out))
     return solution

@@ -202,3 +202,31 @@ def test_peak_minimisation_finds_the_floor():
     floor = Model(si, budget=None, time_limit=120, mip_rel_gap=0.0).solve()
     gb = floor.runtime_expected  # objective = peak in GB (+ a negligible run-time tie-break)
     assert 1.6 / 1024 < gb < 1.7 / 1024
+
+
+def test_tight_budget_fallback_returns_a_schedule_within_the_real_budget(monkeypatch):
+    """If the direct solve ends without a fitting incumbent, the tightening-target fallback
+    must still return a schedule whose replayed peak is within the REAL budget."""
+    from monet_amd import solver as S
+    g, si = build("multiway_newnode", bs=64)
+    mb = 1.8
+    real_solve = S.Model.solve
+    calls = {"n": 0}
+
+    def first_call_fails(self, out_file=None):
+        calls["n"] += 1
+        if calls["n"] == 1:
+            self.last_excess = 0.05 * self.budget
+            raise ValueError("Model infeasible: the cheapest schedule found needs more")
+        return real_solve(self, out_file)
+
+    monkeypatch.setattr(S.Model, "solve", first_call_fails)
+    sol = S.solve_within_budget(si, mb / 1024.0, time_limit=300, mip_rel_gap=0.0)
+    assert calls["n"] >= 2
+    sched = Schedule(g, si)
+    sched.init_schedule(sol, si.mode)
+    peak, _ = replay(sched, 64)
+    assert peak <= mb * 2**20 * 1.001
+    # and a budget below the floor is still reported as infeasible
+    with pytest.raises(ValueError):
+        S.solve_within_budget(si, 1.0 / 1024.0, time_limit=60, mip_rel_gap=0.0, rounds=2)
