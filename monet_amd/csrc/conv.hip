@@ -719,8 +719,11 @@ static int wgrad_tile(const mn_conv2d* g, int variant) {
   // from the same sweeps: 128 x 128 for windows, 128 x 64 for 1x1 filters, 64 rows for K <= 64
   const long long ncols = (long long)g->C * g->R * g->S;
   int tile;
-  if (g->K <= 64)
-    tile = ncols <= 64 ? 4 : 2;
+  if (g->K <= 64) {
+    // 64 columns per tile when 128 would mostly pad (the 3-channel stem: 147 columns)
+    const long long pad128 = (ncols + 127) / 128 * 128, pad64 = (ncols + 63) / 64 * 64;
+    tile = (ncols <= 64 || 4 * pad128 >= 5 * pad64) ? 4 : 2;
+  }
   else
     tile = (g->R * g->S == 1 || ncols <= 64) ? 3 : 0;
   // a 64-wide column tile where it lets the tap-major kernel run (C a multiple of 64, not 128)
