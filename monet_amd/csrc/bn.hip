@@ -533,7 +533,8 @@ static size_t ws_floats(int64_t N, int64_t C, int64_t HW) {
   const int64_t p1 = product_pieces(N, HW, 1);
   if (p1 <= kMaxResident && p1 > P) P = p1;
   if (HW % 4 == 0) {
-    const int64_t p4 = product_pieces(N, HW, 4);
+    int64_t p4 = product_pieces(N, HW, 4);
+    if (p4 > kMaxResident) p4 = resident_pieces(N, HW, 4, 16);  // 512-thread workgroups
     if (p4 <= kMaxResident && p4 > P) P = p4;
   }
   return (size_t)C * (2 * (size_t)P + 1);
@@ -560,27 +561,38 @@ static int run(Args& A, int64_t N, int64_t C, int64_t HW, bool aligned16, void* 
   uint32_t* counters = reinterpret_cast<uint32_t*>(A.partial + ws_floats(N, C, HW));
   A.pivot = reinterpret_cast<float*>(counters) - C;  // last C floats of the float area
   A.ticket = counters;
-  const int keep = t.keep > 0 ? t.keep : 8, threads = t.threads > 0 ? t.threads : kThreads;
-  const int64_t rp = resident_pieces(N, HW, vec, (vec == 4 ? keep * threads : 16 * kThreads) / kThreads);
+  int keep = t.keep > 0 ? t.keep : 8, threads = t.threads > 0 ? t.threads : kThreads;
+  int64_t rp = resident_pieces(N, HW, vec, (vec == 4 ? keep * threads : 16 * kThreads) / kThreads);
+  // channels too long for 256 pieces of 256 x 8 vectors (e.g. 64 x 112 x 112 at batch 184):
+  // twice the workgroup size doubles the piece and keeps them in the one-pass kernel
+  bool wide = false;
+  if (vec == 4 && keep == 8 && threads == kThreads && rp > kMaxResident &&
+      resident_pieces(N, HW, 4, 16) <= kMaxResident) {
+    wide = true;
+    threads = 512;
+    rp = resident_pieces(N, HW, 4, 16);
+  }
   if (t.resident && rp <= kMaxResident) {
     fill_shape(N, C, HW, vec, rp, vec == 4 ? (uint64_t)threads * keep : (uint64_t)kThreads * 16, A.sh);
     const unsigned blocks = (unsigned)(C * rp);
     bn_prepare_kernel<<<(blocks + 255) / 256, 256, 0, s>>>(
           reinterpret_cast<uint64_t*>(A.partial), blocks, A.ticket);
     // persistent grid: enough workgroups to fill 256 CUs at this register footprint
-    const unsigned grid = blocks < (unsigned)t.grid ? blocks : (unsigned)t.grid;
+    // (512-thread workgroups: one per CU at this register footprint)
+    const unsigned want = wide ? 256u : (unsigned)t.grid;
+    const unsigned grid = blocks < want ? blocks : want;
 #define MN_BN_RES(V, K, T) bn_resident_kernel<V, MODE, K, T><<<grid, T, 0, s>>>(A, blocks)
     if (vec == 4) {
+      if (wide) MN_BN_RES(4, 8, 512);
 #ifdef MN_TUNING
-      if (keep == 8 && threads == 256) MN_BN_RES(4, 8, 256);
+      else if (keep == 8 && threads == 256) MN_BN_RES(4, 8, 256);
       else if (keep == 4 && threads == 512) MN_BN_RES(4, 4, 512);
       else if (keep == 8 && threads == 512) MN_BN_RES(4, 8, 512);
       else if (keep == 4 && threads == 1024) MN_BN_RES(4, 4, 1024);
       else if (keep == 16 && threads == 256) MN_BN_RES(4, 16, 256);
       else if (keep == 12 && threads == 256) MN_BN_RES(4, 12, 256);
-      else
 #endif
-      MN_BN_RES(4, 8, 256);
+      else MN_BN_RES(4, 8, 256);
     } else {
       MN_BN_RES(1, 16, 256);
     }
