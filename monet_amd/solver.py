@@ -518,6 +518,9 @@ def main(argv=None):
     parser.add_argument("--data_dir", default="data", help="where profiles and solutions go")
     parser.add_argument("--si_file", default="", help="profiled solver info to solve from")
     parser.add_argument("--profile_only", action="store_true")
+    parser.add_argument("--rounds", default=6, type=int,
+                        help="tightening-target rounds to fall back on when the direct solve ends "
+                             "without a fitting schedule (0: one solve with the whole time limit)")
     parser.add_argument("--verbose", action="store_true")
     args = parser.parse_args(argv)
 
@@ -541,7 +544,8 @@ def main(argv=None):
           "; mode", args.mode)
     out = Path(args.data_dir) / solution_file_name(model_name, si.bs, args.mode, args.budget)
     solution = solve_within_budget(si, args.budget, args.time_limit, args.solver, args.ablation,
-                                   out_file=str(out), mip_rel_gap=args.gap, verbose=args.verbose,
+                                   out_file=str(out), rounds=args.rounds, mip_rel_gap=args.gap,
+                                   verbose=args.verbose,
                                    recompute_window=args.window)
     print("solved in %.1f s, expected run time %.2f ms -> %s" % (
         solution.solve_time, solution.runtime_expected / CPU_GCD_MULTIPLIER, out))
