@@ -115,6 +115,7 @@ struct Gather {
   long long cha;
   int16_t dh[kMaxTaps], dw[kMaxTaps];
   int32_t aoff[kMaxTaps];
+  int ksplit, tiles_per_split;  // split reduction (ksplit > 1): grid.z slices of k-tiles
 };
 
 // FAST: the source has a multiple of BK channels.  Then the reduction index
@@ -284,9 +285,18 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-  const int ktiles = (g.Kd + BK - 1) / BK;
-  if (ktiles > 0) {
+  // reduction range of this workgroup: all k-tiles, or slice blockIdx.z of them (split
+  // reduction: the slices are added into a cleared output with atomics)
+  const int all_tiles = (g.Kd + BK - 1) / BK;
+  const int kt_begin = g.ksplit > 1 ? (int)blockIdx.z * g.tiles_per_split : 0;
+  const int ktiles = g.ksplit > 1 ? min(kt_begin + g.tiles_per_split, all_tiles) : all_tiles;
+  if (kt_begin < ktiles) {
     int t = 0, c0 = 0;  // FAST: position of the tile being fetched
+    if (FAST && kt_begin > 0) {
+      const int per_tap = g.Cs / BK;
+      t = kt_begin / per_tap;
+      c0 = (kt_begin - t * per_tap) * BK;
+    }
     auto fetch_next = [&](int kt) {
       if (FAST) {
         fetch_fast(t, c0);
@@ -299,11 +309,11 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
         fetch_any(kt * BK);
       }
     };
-    fetch_next(0);
+    fetch_next(kt_begin);
     stage(0);
     __syncthreads();
-    for (int kt = 0; kt < ktiles; ++kt) {
-      const int buf = kt & 1;
+    for (int kt = kt_begin; kt < ktiles; ++kt) {
+      const int buf = (kt - kt_begin) & 1;
       if (kt + 1 < ktiles) fetch_next(kt + 1);
       mma_tile<TL, BK, LDA>(lds_a[buf], lds_b[buf], wm, wn, lane, acc);
       if (kt + 1 < ktiles) stage(buf ^ 1);
@@ -330,7 +340,11 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
         const int m = m0 + wm * (TL::TM * 32) + mi * 32 + acc_row(v, lane);
         if (m < g.M) {
           float r = acc[mi][nj][v];
-          if (bias) r += bias[m];
+          if (bias && blockIdx.z == 0) r += bias[m];
+          if (g.ksplit > 1) {
+            atomicAdd(&out[(size_t)m * plane], r);
+            continue;
+          }
           // a dense output is written once and not read by this kernel: keep it out of the
           // caches the operand tiles live in; strided (parity-class) outputs share cache lines
           // between launches and are better left to the cache
@@ -685,7 +699,7 @@ static bool fast_path(const Gather& g) { return g.T > 0 && g.Cs % BK == 0; }
 template <class TL>
 static void launch_gather_t(const Gather& g, const float* a, const float* src, const float* bias,
                             float* dst, hipStream_t s, bool packed) {
-  dim3 grid((g.ncols + TL::BN - 1) / TL::BN, (g.M + TL::BM - 1) / TL::BM);
+  dim3 grid((g.ncols + TL::BN - 1) / TL::BN, (g.M + TL::BM - 1) / TL::BM, g.ksplit > 1 ? g.ksplit : 1);
   if (packed)
     gather_gemm_kernel<TL, true, true><<<grid, kThreads, 0, s>>>(g, a, src, bias, dst);
   else if (fast_path(g))
@@ -694,14 +708,52 @@ static void launch_gather_t(const Gather& g, const float* a, const float* src, c
     gather_gemm_kernel<TL, false><<<grid, kThreads, 0, s>>>(g, a, src, bias, dst);
 }
 
+static void tile_dims(int tile, int* bm, int* bn);
+
+// Few, long workgroups quantise badly over 256 CUs (2.2 per CU run as 3 rounds): when a
+// launch has fewer than ~6 workgroups per CU, a long reduction and a dense output, slice the
+// reduction so that there are ~8 per CU and add the slices into a cleared output.
+static void plan_split(Gather& g, int tile, bool allow) {
+  g.ksplit = 1;
+  g.tiles_per_split = 0;
+  if (!allow || g.osh != 1 || g.osw != 1) return;
+#ifdef MN_TUNING
+  if (const char* e = getenv("MN_CONV_SPLIT")) {
+    if (atoi(e) <= 1) return;
+  }
+#endif
+  int bm, bn;
+  tile_dims(tile, &bm, &bn);
+  const long long wgs = ((long long)(g.ncols + bn - 1) / bn) * ((g.M + bm - 1) / bm);
+  const int ktiles = (g.Kd + BK - 1) / BK;
+  if (wgs >= 6 * 256 || ktiles < 32) return;
+  int want = (int)((8 * 256 + wgs - 1) / wgs);
+  if (want > ktiles / 16) want = ktiles / 16;  // at least 16 k-tiles per slice
+  if (want > 8) want = 8;
+#ifdef MN_TUNING
+  if (const char* e = getenv("MN_CONV_SPLIT")) want = atoi(e);
+#endif
+  if (want <= 1) return;
+  g.tiles_per_split = (ktiles + want - 1) / want;
+  g.ksplit = (ktiles + g.tiles_per_split - 1) / g.tiles_per_split;
+  if (g.ksplit <= 1) g.ksplit = 1;
+}
+
 // `packed`: a = the repacked operand (pack_weights_kernel) with rows of g.lda floats.
-static void launch_gather(const Gather& g, const float* a, const float* src, const float* bias,
-                          float* dst, hipStream_t s, bool packed = false, int tile = -1) {
+// `split_ok`: the caller allows a split reduction (dst is then cleared here first).
+static void launch_gather(Gather g, const float* a, const float* src, const float* bias,
+                          float* dst, hipStream_t s, bool packed = false, bool split_ok = false,
+                          int tile = -1) {
   if (g.ncols == 0 || g.M == 0) return;
 #ifdef MN_TUNING
   if (const char* e = getenv("MN_CONV_TILE")) tile = atoi(e);
 #endif
   if (tile < 0) tile = pick_tile(g.M, g.ncols, fast_path(g), packed);
+  plan_split(g, tile, split_ok && packed);
+  if (g.ksplit > 1) {
+    const size_t n = (size_t)g.N * g.M * g.DH * g.DW;
+    fill_zero_kernel<<<(unsigned)((n / 4 + kThreads) / kThreads), kThreads, 0, s>>>(dst, n);
+  }
   switch (tile) {
     case 1: launch_gather_t<T64x256>(g, a, src, bias, dst, s, packed); break;
     case 2: launch_gather_t<T64x128>(g, a, src, bias, dst, s, packed); break;
@@ -855,7 +907,7 @@ int mn_conv_fwd(const mn_conv2d* g, const void* x, const void* w, const void* bi
     a = (const float*)ws;
     q.lda = Mp;
   }
-  launch_gather(q, a, (const float*)x, (const float*)bias, (float*)y, s, packed);
+  launch_gather(q, a, (const float*)x, (const float*)bias, (float*)y, s, packed, packed);
   return mn_launch_status();
 }
 
@@ -936,7 +988,8 @@ int mn_conv_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void* dx
       q.osw = g->sW;
       q.lda = lda;
       q.cha = cha;
-      launch_gather(q, a, (const float*)dy, nullptr, (float*)dx, s, packed);
+      launch_gather(q, a, (const float*)dy, nullptr, (float*)dx, s, packed,
+                    packed && g->sH == 1 && g->sW == 1);
     }
   }
   return mn_launch_status();
