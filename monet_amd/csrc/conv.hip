@@ -808,7 +808,18 @@ static void wgrad_split(const mn_conv2d* g, int variant, int* splits, int* tiles
   const long long total_tiles = (depth + WBK - 1) / WBK;
   const long long out_tiles =
       (((long long)g->C * g->R * g->S + bn - 1) / bn) * (((long long)g->K + bm - 1) / bm);
-  long long want = (768 + out_tiles - 1) / out_tiles;
+  // All workgroups of the launch should be resident at once: one more than the CUs can hold
+  // runs as a second round on its own and nearly doubles the time.  Resident workgroups per
+  // CU by tile (LDS / register footprint): 128x128 2 (3 in the 16-deep tap-major kernel),
+  // 128x64 and 64x128 3, 64x64 4.
+  const int tile = wgrad_tile(g, variant);
+  const bool tap = wgrad_tap_major(g, bm, bn) && (variant == 1 || g->R * g->S == 1);
+  const int per_cu = tile == 0 ? (tap ? 3 : 2) : (tile == 4 ? 4 : 3);
+  long long slots = 256ll * per_cu;
+#ifdef MN_TUNING
+  if (const char* e = getenv("MN_WGRAD_SLOTS")) slots = atoll(e);
+#endif
+  long long want = slots / out_tiles;  // rounded down: never a partial extra round
   if (want > total_tiles) want = total_tiles;
   if (want > 256) want = 256;
   if (want < 1) want = 1;
