@@ -387,11 +387,12 @@ struct Held {
   typename Vec<VEC>::type a[KEEP], b[KEEP];
   int c, piece;
   float sft;
+  float t0, t1;  // SOLO: the piece is the whole channel, these are its totals
 };
 
 // Load a piece, reduce it and publish its partial pair.  Never waits for
 // another workgroup.
-template <int VEC, int MODE, int KEEP, int THREADS>
+template <int VEC, int MODE, int KEEP, int THREADS, bool SOLO = false>
 __device__ __forceinline__ void hold_piece(const Args& A, uint32_t item, Held<VEC, KEEP>& h,
                                            float* lds) {
   typedef CursorT<THREADS> Cursor;
@@ -435,19 +436,25 @@ __device__ __forceinline__ void hold_piece(const Args& A, uint32_t item, Held<VE
     }
   }
   block_sum2<THREADS / MN_WAVE>(s0, s1, lds);
-  if (threadIdx.x == 0)
+  if (SOLO) {
+    h.t0 = s0;
+    h.t1 = s1;
+  } else if (threadIdx.x == 0) {
     publish(reinterpret_cast<uint64_t*>(A.partial) + (size_t)h.c * S + h.piece, s0, s1);
+  }
 }
 
 // Wait for the channel totals of a held piece and write its result.
-template <int VEC, int MODE, int KEEP, int THREADS>
+template <int VEC, int MODE, int KEEP, int THREADS, bool SOLO = false>
 __device__ __forceinline__ void finish_piece(const Args& A, const Held<VEC, KEEP>& h, float* lds) {
   typedef typename Vec<VEC>::type V;
   typedef CursorT<THREADS> Cursor;
   const Shape& sh = A.sh;
-  float t0, t1;
-  __syncthreads();  // lds is free again
-  gather_totals(reinterpret_cast<uint64_t*>(A.partial) + (size_t)h.c * sh.S, sh.S, lds, t0, t1);
+  float t0 = h.t0, t1 = h.t1;
+  if (!SOLO) {
+    __syncthreads();  // lds is free again
+    gather_totals(reinterpret_cast<uint64_t*>(A.partial) + (size_t)h.c * sh.S, sh.S, lds, t0, t1);
+  }
   float s_, proj, gmean, gscale;
   coefficients<MODE>(A, h.c, h.piece, t0, t1, h.sft, s_, proj, gmean, gscale);
   if (!A.out) return;
@@ -499,6 +506,19 @@ __global__ __launch_bounds__(THREADS) void bn_resident_kernel(const Args A, uint
     if (i0 < items) hold_piece<VEC, MODE, KEEP, THREADS>(A, i0, h0, lds);
     finish_piece<VEC, MODE, KEEP, THREADS>(A, h1, lds);
     if (i0 >= items) break;
+  }
+}
+
+// Channels short enough for ONE workgroup's registers (N*HW <= THREADS * KEEP vectors, e.g.
+// 14 x 14 and 7 x 7 planes at batch 184): a workgroup takes whole channels, so there is nothing
+// to publish, poll or prepare - one launch, no workspace traffic, no atomics.
+template <int VEC, int MODE, int KEEP, int THREADS>
+__global__ __launch_bounds__(THREADS) void bn_solo_kernel(const Args A) {
+  __shared__ float lds[2 * (THREADS / MN_WAVE)];
+  Held<VEC, KEEP> h;
+  for (uint32_t c = blockIdx.x; c < (uint32_t)A.sh.C; c += gridDim.x) {
+    hold_piece<VEC, MODE, KEEP, THREADS, true>(A, c, h, lds);
+    finish_piece<VEC, MODE, KEEP, THREADS, true>(A, h, lds);
   }
 }
 
@@ -571,6 +591,21 @@ static int run(Args& A, int64_t N, int64_t C, int64_t HW, bool aligned16, void* 
     wide = true;
     threads = 512;
     rp = resident_pieces(N, HW, 4, 16);
+  }
+  // whole channels in one workgroup's registers
+  const uint64_t chan = (uint64_t)N * (HW / vec);
+  if (t.resident && t.keep == 8 && t.threads == kThreads) {
+    const unsigned grid = (unsigned)(C < 65535 ? C : 65535);
+#define MN_BN_SOLO(V, K, T)                                              \
+  do {                                                                   \
+    fill_shape(N, C, HW, V, 1, (uint64_t)(T) * (K), A.sh);               \
+    bn_solo_kernel<V, MODE, K, T><<<grid, T, 0, s>>>(A);                 \
+    return mn_launch_status();                                           \
+  } while (0)
+    if (vec == 4 && chan <= 256u * 9u) MN_BN_SOLO(4, 9, 256);
+    if (vec == 4 && chan <= 1024u * 9u) MN_BN_SOLO(4, 9, 1024);
+    if (vec == 1 && chan <= 256u * 36u) MN_BN_SOLO(1, 36, 256);
+#undef MN_BN_SOLO
   }
   if (t.resident && rp <= kMaxResident) {
     fill_shape(N, C, HW, vec, rp, vec == 4 ? (uint64_t)threads * keep : (uint64_t)kThreads * 16, A.sh);

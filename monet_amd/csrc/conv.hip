@@ -73,9 +73,9 @@ static FastDiv make_fastdiv(uint32_t d) {
 }
 
 // Multiply one staged k-tile (DEPTH deep, k-major in LDS) into the accumulators.
-template <class TL, int DEPTH, int LDA = TL::BM + kPad>
+template <class TL, int DEPTH, int LDA = TL::BM + kPad, int LDB = TL::BN + kPad>
 __device__ __forceinline__ void mma_tile(const float (*As)[LDA],
-                                         const float (*Bs)[TL::BN + kPad], int wm, int wn,
+                                         const float (*Bs)[LDB], int wm, int wn,
                                          int lane, float16_t (&acc)[TL::TM][TL::TN]) {
   const int r = lane & 31, half = lane >> 5;
   const int arow = wm * (TL::TM * 32) + r, bcol = wn * (TL::TN * 32) + r;
@@ -129,18 +129,22 @@ struct Gather {
 // floats (a multiple of 128, zero padded), so a k-tile of A is BK contiguous
 // row pieces: one 16-byte load per lane and row piece, no masks, and 8 cache
 // lines per wavefront load instead of the ~20 a strided gather touches.
+// POINT (with PACKED): a 1x1 filter, stride 1, no padding - the gather is the identity, a
+// k-tile of B is BK contiguous rows of pixels, loaded and staged as 16-byte vectors too.
 constexpr int kPadPacked = 4;  // keeps LDS rows 16-byte aligned for the 128-bit stores
-template <class TL, bool FAST, bool PACKED = false>
+template <class TL, bool FAST, bool PACKED = false, bool POINT = false>
 __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
                                                                const float* __restrict__ a,
                                                                const float* __restrict__ src,
                                                                const float* __restrict__ bias,
                                                                float* __restrict__ dst) {
   static_assert(!PACKED || FAST, "the packed operand is only used with the tap-major path");
+  static_assert(!POINT || PACKED, "the pointwise path is built on the packed one");
   constexpr int BM = TL::BM, BN = TL::BN;
   constexpr int LDA = BM + (PACKED ? kPadPacked : kPad);
+  constexpr int LDB = BN + (POINT ? kPadPacked : kPad);
   __shared__ __attribute__((aligned(16))) float lds_a[2][BK][LDA];
-  __shared__ float lds_b[2][BK][BN + kPad];
+  __shared__ __attribute__((aligned(16))) float lds_b[2][BK][LDB];
   __shared__ int tdh[kMaxTaps], tdw[kMaxTaps], taoff[kMaxTaps];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / TL::WN, wn = wave % TL::WN;
@@ -199,6 +203,25 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
     }
   }
 
+  // pointwise B loader: float4 number f = tid + kThreads*i of the k-tile, row f / (BN/4)
+  constexpr int kB4 = BN * BK / 4 / kThreads;
+  float4_t rb4[kB4 > 0 ? kB4 : 1];
+  uint32_t bp_b[kB4 > 0 ? kB4 : 1];
+  uint32_t bp_ok = 0;
+  if (POINT) {
+    const uint32_t PQ = (uint32_t)g.OH * g.OW;  // a multiple of 4: a float4 stays inside an image
+#pragma unroll
+    for (int i = 0; i < kB4; ++i) {
+      const int f = tid + kThreads * i;
+      const uint32_t krow = f / (BN / 4), c4 = n0 + 4 * (f % (BN / 4));
+      const bool ok = c4 < g.ncols;
+      const uint32_t im = ok ? c4 / PQ : 0u;
+      const uint32_t px = ok ? c4 - im * PQ : 0u;
+      bp_b[i] = (im * (uint32_t)g.Cs + krow) * plane_b + px * 4u;
+      bp_ok |= (ok ? 1u : 0u) << i;
+    }
+  }
+
   const char* sp = reinterpret_cast<const char*>(src);
   const char* ap = reinterpret_cast<const char*>(a);
   float ra[kARows], rb[kBRows];
@@ -211,11 +234,17 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
     const int hh = ohs + dh, ww = ows + dw;
     const bool ok = col_ok && (unsigned)hh < (unsigned)g.Hs && (unsigned)ww < (unsigned)g.Ws;
     b_ok = ok ? 0xFFFFFFFFu : 0u;
-    const uint32_t sb = (uint32_t)((((long long)c0 * g.Hs + dh) * g.Ws + dw) * 4);
-    const uint32_t base = ok ? pix_b + sb : brow0 * plane_b;
+    if (POINT) {
 #pragma unroll
-    for (int i = 0; i < kBRows; ++i)
-      rb[i] = *reinterpret_cast<const float*>(sp + (base + kBStep * i * plane_b));
+      for (int i = 0; i < kB4; ++i)
+        rb4[i] = *reinterpret_cast<const float4_t*>(sp + (bp_b[i] + (uint32_t)c0 * plane_b));
+    } else {
+      const uint32_t sb = (uint32_t)((((long long)c0 * g.Hs + dh) * g.Ws + dw) * 4);
+      const uint32_t base = ok ? pix_b + sb : brow0 * plane_b;
+#pragma unroll
+      for (int i = 0; i < kBRows; ++i)
+        rb[i] = *reinterpret_cast<const float*>(sp + (base + kBStep * i * plane_b));
+    }
     if (PACKED) {
       const uint32_t sa = (uint32_t)(((long long)taoff[t] * g.Cs + c0) * g.lda * 4);
 #pragma unroll
@@ -261,9 +290,19 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
     }
   };
   auto stage = [&](int buf) {
+    if (POINT) {
+      const float4_t z = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int i = 0; i < kBRows; ++i)
-      lds_b[buf][brow0 + kBStep * i][bcol] = ((b_ok >> i) & 1u) ? rb[i] : 0.f;
+      for (int i = 0; i < kB4; ++i) {
+        const int f = tid + kThreads * i;
+        *reinterpret_cast<float4_t*>(&lds_b[buf][f / (BN / 4)][4 * (f % (BN / 4))]) =
+            ((bp_ok >> i) & 1u) ? rb4[i] : z;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < kBRows; ++i)
+        lds_b[buf][brow0 + kBStep * i][bcol] = ((b_ok >> i) & 1u) ? rb[i] : 0.f;
+    }
     if (PACKED) {
 #pragma unroll
       for (int i = 0; i < kA4; ++i) {
@@ -315,7 +354,7 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
     for (int kt = kt_begin; kt < ktiles; ++kt) {
       const int buf = (kt - kt_begin) & 1;
       if (kt + 1 < ktiles) fetch_next(kt + 1);
-      mma_tile<TL, BK, LDA>(lds_a[buf], lds_b[buf], wm, wn, lane, acc);
+      mma_tile<TL, BK, LDA, LDB>(lds_a[buf], lds_b[buf], wm, wn, lane, acc);
       if (kt + 1 < ktiles) stage(buf ^ 1);
       __syncthreads();
     }
@@ -700,7 +739,13 @@ template <class TL>
 static void launch_gather_t(const Gather& g, const float* a, const float* src, const float* bias,
                             float* dst, hipStream_t s, bool packed) {
   dim3 grid((g.ncols + TL::BN - 1) / TL::BN, (g.M + TL::BM - 1) / TL::BM, g.ksplit > 1 ? g.ksplit : 1);
-  if (packed)
+  // pointwise: the gather is the identity and pixels come in whole float4
+  const bool point = packed && g.T == 1 && g.dh[0] == 0 && g.dw[0] == 0 && g.ish == 1 &&
+                     g.isw == 1 && g.Hs == g.OH && g.Ws == g.OW && (g.OH * g.OW) % 4 == 0 &&
+                     mn_aligned(src, 16);
+  if (point)
+    gather_gemm_kernel<TL, true, true, true><<<grid, kThreads, 0, s>>>(g, a, src, bias, dst);
+  else if (packed)
     gather_gemm_kernel<TL, true, true><<<grid, kThreads, 0, s>>>(g, a, src, bias, dst);
   else if (fast_path(g))
     gather_gemm_kernel<TL, true><<<grid, kThreads, 0, s>>>(g, a, src, bias, dst);

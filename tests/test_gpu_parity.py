@@ -205,6 +205,7 @@ def test_maxpool_rejects_what_a_nibble_cannot_hold(cuda):
 # ----------------------------------------------------------------- batchnorm
 BN_SHAPES = [(4, 3, 5, 5), (2, 8, 7, 3), (16, 4, 6, 6), (8, 64, 56, 56), (32, 16, 7, 7),
              (3, 5, 1, 1), (2, 2, 130, 70), (184, 8, 28, 28),
+             (184, 6, 14, 14), (184, 5, 7, 7),   # whole channel in one workgroup
              (184, 2, 112, 112)]   # channels long enough for the 512-thread one-pass kernel
 
 
