@@ -193,7 +193,10 @@ typedef struct mn_conv2d {
  *                    1 same with the weights repacked [tap][c][k] (k padded
  *                      to a multiple of 128) into the workspace, so operand
  *                      tiles load as full 16-byte vectors; channel counts
- *                      that are not a multiple of 16 run it like variant 0
+ *                      that are not a multiple of 16 run it like variant 0.
+ *                      Launches with few, long workgroups split the reduction
+ *                      and add the slices with atomics (sums may then differ in
+ *                      the last bits from run to run; variant 0 never does)
  *   backward-data    0 implicit GEMM reading the weights through strides
  *                    1 same with the weights repacked [tap][k][c] (c padded
  *                      to a multiple of 128) into the workspace
