@@ -422,7 +422,6 @@ class Model:
                    options={"time_limit": float(self.time_limit), "mip_rel_gap": self.mip_rel_gap,
                             "disp": bool(self.verbose), "presolve": bool(self.presolve)})
         solve_time = time() - t0
-        self.last_problem = (A, np.array(B.lo), np.array(B.hi), res.x)
         if res.x is None:
             raise ValueError("Model infeasible" if res.status == 2 else
                              f"no schedule found: {res.message}")

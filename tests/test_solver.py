@@ -230,3 +230,29 @@ def test_tight_budget_fallback_returns_a_schedule_within_the_real_budget(monkeyp
     # and a budget below the floor is still reported as infeasible
     with pytest.raises(ValueError):
         S.solve_within_budget(si, 1.0 / 1024.0, time_limit=60, mip_rel_gap=0.0, rounds=2)
+
+
+def test_model_definitions_trace_to_the_expected_operators():
+    """The two benchmark networks, traced on the CPU: operator counts of the torchvision
+    ResNet-50 topology and of the U-Net, and the solver graph sizes that follow."""
+    from collections import Counter
+    from monet_amd.models import build_model
+    model, shape, name = build_model("torchvision.models.resnet50()")
+    assert name == "resnet50" and shape == (3, 224, 224)
+    assert sum(p.numel() for p in model.parameters()) == 25557032
+    g = Graph.create(model, shape)
+    ops = Counter(n.op for n in g.nodes if isinstance(n, ComputeNode))
+    assert ops == {"aten::_convolution": 53, "aten::batch_norm": 53, "aten::relu_": 49,
+                   "aten::add_": 16, "aten::max_pool2d": 1, "aten::adaptive_avg_pool2d": 1,
+                   "aten::flatten": 1, "aten::linear": 1}
+    si = SolverInfo(184, name, "inplace_conv_multiway_newnode")
+    si.extract(g, cost_fn=synthetic_cost(si))
+    assert si.loss == 225 and len(si.nodes) == 455
+    assert len(si.conv_list) == 53 * 3 and len(si.inplace_list) == (49 + 16) + 49
+
+    unet, ushape, uname = build_model("unet")
+    assert uname == "unet" and ushape == (3, 416, 608)
+    gu = Graph.create(unet, ushape)
+    uops = Counter(n.op for n in gu.nodes if isinstance(n, ComputeNode))
+    assert uops == {"aten::_convolution": 19, "aten::batch_norm": 18, "aten::relu_": 18,
+                    "aten::max_pool2d": 4, "aten::adaptive_avg_pool2d": 4, "aten::cat": 4}
