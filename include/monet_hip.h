@@ -157,6 +157,28 @@ int mn_softmax_bwd_f32(const float* dy, const float* y, float* dx, int64_t outer
 int mn_xent_bwd_f32(const float* logits, const int64_t* labels, float* dlogits, int64_t outer,
                     int64_t dim, int64_t inner, float scale, mn_stream_t stream);
 
+/* BatchNorm fused with the ReLU that follows it (no counterpart in the
+ * reference, whose executor runs them as two operators, monet/lm_ops/bn.py and
+ * relu.py; fusing saves one read and one write of the activation in each
+ * direction and needs no mask, because the backward recomputes the sign of the
+ * pre-activation from the stored INPUT).
+ *   forward (training):   y = max(BN(x), 0), statistics as mn_bn_fwd_train_f32
+ *   forward (saved stats): y = max((x-mean)*invstd*gamma + beta, 0)
+ *   backward: dy is the gradient of the ReLU OUTPUT; g = dy where
+ *             (x-mean)*invstd*gamma + beta > 0, else 0; then as
+ *             mn_bn_bwd_from_x_f32 with g in place of dy.  dx may alias dy. */
+int mn_bn_relu_fwd_train_f32(const float* x, const float* gamma, const float* beta,
+                             float* running_mean, float* running_var, float* y, float* save_mean,
+                             float* save_invstd, int64_t N, int64_t C, int64_t HW, double momentum,
+                             double eps, void* ws, size_t ws_bytes, mn_stream_t stream);
+int mn_bn_relu_fwd_apply_f32(const float* x, const float* mean, const float* invstd,
+                             const float* gamma, const float* beta, float* y, int64_t N, int64_t C,
+                             int64_t HW, mn_stream_t stream);
+int mn_bn_relu_bwd_from_x_f32(const float* dy, const float* x, const float* gamma,
+                              const float* beta, const float* mean, const float* invstd, float* dx,
+                              float* dgamma, float* dbeta, int64_t N, int64_t C, int64_t HW,
+                              void* ws, size_t ws_bytes, mn_stream_t stream);
+
 /* ----------------------------------------------------------- convolution --
  * 2-D convolution over NCHW tensors, weights [K, C, R, S], groups == 1.
  * P/Q are the output sizes: floor((H + 2*pH - dH*(R-1) - 1) / sH) + 1. */

@@ -126,7 +126,29 @@ struct Args {
   float* pivot;         // [C], forward only
   uint32_t* ticket;     // resident launch only
   float inv_m, unbias, momentum, eps;
+  // Fused ReLU.  Forward: out = max(out, 0).  Backward from the input: the incoming gradient
+  // is that of the ReLU output, so it only counts where the recomputed pre-activation
+  // (b - mean) * (invstd * gamma) + rbeta is positive.
+  int relu;
+  const float* rbeta;
 };
+
+// The ReLU gate of the fused backward, per channel.
+struct Gate {
+  bool on;
+  float k1, beta;
+  __device__ __forceinline__ float operator()(float g, float d) const {
+    return (!on || k1 * d + beta > 0.f) ? g : 0.f;
+  }
+};
+template <int MODE>
+__device__ __forceinline__ Gate make_gate(const Args& A, int c) {
+  Gate r;
+  r.on = MODE == BWD_FROM_X && A.relu;
+  r.k1 = r.on ? A.invstd[c] * (A.gamma ? A.gamma[c] : 1.f) : 0.f;
+  r.beta = (r.on && A.rbeta) ? A.rbeta[c] : 0.f;
+  return r;
+}
 
 // ---------------------------------------------------------------- reduce --
 // (s0, s1) = ( sum a , sum a*(b - shift) )   backward
@@ -138,6 +160,7 @@ __device__ __forceinline__ void reduce_piece(const Args& A, int c, int piece, fl
   const Shape& sh = A.sh;
   s0 = 0.f;
   s1 = 0.f;
+  const Gate gate = make_gate<MODE>(A, c);
   Cursor cur(sh, piece);
   while (cur.valid()) {
     V va[kU], vb[kU];
@@ -162,7 +185,7 @@ __device__ __forceinline__ void reduce_piece(const Args& A, int c, int piece, fl
             s0 += d;
             s1 += d * d;
           } else {
-            const float g = comp(va[u], k);
+            const float g = gate(comp(va[u], k), d);
             s0 += g;
             s1 += g * d;
           }
@@ -186,6 +209,8 @@ __device__ __forceinline__ void apply_piece(const Args& A, int c, int piece, flo
                                             float gmean, float gscale) {
   typedef typename Vec<VEC>::type V;
   const Shape& sh = A.sh;
+  const Gate gate = make_gate<MODE>(A, c);
+  const bool relu = MODE == FWD_TRAIN && A.relu;
   Cursor cur(sh, piece);
   while (cur.valid()) {
     V va[kU], vb[kU];
@@ -207,10 +232,13 @@ __device__ __forceinline__ void apply_piece(const Args& A, int c, int piece, flo
         V r;
 #pragma unroll
         for (int k = 0; k < VEC; ++k) {
-          if (MODE == FWD_TRAIN)
-            setc(r, k, (comp(vb[u], k) - proj) * gscale + gmean);
-          else
-            setc(r, k, (comp(va[u], k) - (comp(vb[u], k) - sft) * proj - gmean) * gscale);
+          if (MODE == FWD_TRAIN) {
+            const float y = (comp(vb[u], k) - proj) * gscale + gmean;
+            setc(r, k, relu ? fmaxf(y, 0.f) : y);
+          } else {
+            const float d = comp(vb[u], k) - sft;
+            setc(r, k, (gate(comp(va[u], k), d) - d * proj - gmean) * gscale);
+          }
         }
         stv<VEC>(A.out + o[u], r);
       }
@@ -415,6 +443,7 @@ __device__ __forceinline__ void hold_piece(const Args& A, uint32_t item, Held<VE
   }
   float s0 = 0.f, s1 = 0.f;
   {
+    const Gate gate = make_gate<MODE>(A, h.c);
     Cursor cur(sh, h.piece);
 #pragma unroll
     for (int k = 0; k < KEEP; ++k) {
@@ -426,7 +455,7 @@ __device__ __forceinline__ void hold_piece(const Args& A, uint32_t item, Held<VE
             s0 += d;
             s1 += d * d;
           } else {
-            const float g = comp(h.a[k], e);
+            const float g = gate(comp(h.a[k], e), d);
             s0 += g;
             s1 += g * d;
           }
@@ -458,6 +487,8 @@ __device__ __forceinline__ void finish_piece(const Args& A, const Held<VEC, KEEP
   float s_, proj, gmean, gscale;
   coefficients<MODE>(A, h.c, h.piece, t0, t1, h.sft, s_, proj, gmean, gscale);
   if (!A.out) return;
+  const Gate gate = make_gate<MODE>(A, h.c);
+  const bool relu = MODE == FWD_TRAIN && A.relu;
   Cursor cur(sh, h.piece);
 #pragma unroll
   for (int k = 0; k < KEEP; ++k) {
@@ -465,10 +496,13 @@ __device__ __forceinline__ void finish_piece(const Args& A, const Held<VEC, KEEP
       V r;
 #pragma unroll
       for (int e = 0; e < VEC; ++e) {
-        if (MODE == FWD_TRAIN)
-          setc(r, e, (comp(h.b[k], e) - proj) * gscale + gmean);
-        else
-          setc(r, e, (comp(h.a[k], e) - (comp(h.b[k], e) - s_) * proj - gmean) * gscale);
+        if (MODE == FWD_TRAIN) {
+          const float y = (comp(h.b[k], e) - proj) * gscale + gmean;
+          setc(r, e, relu ? fmaxf(y, 0.f) : y);
+        } else {
+          const float d = comp(h.b[k], e) - s_;
+          setc(r, e, (gate(comp(h.a[k], e), d) - d * proj - gmean) * gscale);
+        }
       }
       stv<VEC>(A.out + cur.template off<VEC>(sh.C, h.c, sh.HW), r);
     }
@@ -654,7 +688,8 @@ static int run(Args& A, int64_t N, int64_t C, int64_t HW, bool aligned16, void* 
 
 int bwd_launch(bool from_y, const float* dy, const float* t, const float* gamma, const float* shift,
                const float* invstd, float* dx, float* dgamma, float* dbeta, int64_t N, int64_t C,
-               int64_t HW, void* ws, size_t ws_bytes, hipStream_t s, const Tuning& tune) {
+               int64_t HW, void* ws, size_t ws_bytes, hipStream_t s, const Tuning& tune,
+               bool relu = false, const float* relu_beta = nullptr) {
   if (N < 0 || C < 0 || HW < 0) return MN_EINVAL;
   if (N == 0 || C == 0 || HW == 0) return MN_OK;
   if (!dy || !t || !invstd || !ws) return MN_EINVAL;
@@ -671,6 +706,9 @@ int bwd_launch(bool from_y, const float* dy, const float* t, const float* gamma,
   A.vec0 = dgamma;
   A.vec1 = dbeta;
   A.inv_m = 1.f / (float)((double)N * (double)HW);
+  A.relu = relu ? 1 : 0;
+  A.rbeta = relu_beta;
+  if (relu && from_y) return MN_EUNSUPPORTED;
   return from_y ? run<BWD_FROM_Y>(A, N, C, HW, al, ws, tune, s)
                 : run<BWD_FROM_X>(A, N, C, HW, al, ws, tune, s);
 }
@@ -678,7 +716,7 @@ int bwd_launch(bool from_y, const float* dy, const float* t, const float* gamma,
 int fwd_train_launch(const float* x, const float* gamma, const float* beta, float* running_mean,
                      float* running_var, float* y, float* save_mean, float* save_invstd, int64_t N,
                      int64_t C, int64_t HW, double momentum, double eps, void* ws, size_t ws_bytes,
-                     hipStream_t s, const Tuning& tune) {
+                     hipStream_t s, const Tuning& tune, bool relu = false) {
   if (N < 0 || C < 0 || HW < 0) return MN_EINVAL;
   if (N == 0 || C == 0 || HW == 0) return MN_OK;
   if (!x || !y || !save_mean || !save_invstd || !ws) return MN_EINVAL;
@@ -699,6 +737,7 @@ int fwd_train_launch(const float* x, const float* gamma, const float* beta, floa
   A.unbias = M > 1.0 ? (float)(M / (M - 1.0)) : 1.f;
   A.momentum = (float)momentum;
   A.eps = (float)eps;
+  A.relu = relu ? 1 : 0;
   return run<FWD_TRAIN>(A, N, C, HW, al, ws, tune, s);
 }
 
@@ -719,9 +758,9 @@ int mn_bn_fwd_train_f32(const float* x, const float* gamma, const float* beta, f
                                  mn_stream(stream), mn_bn::Tuning());
 }
 
-int mn_bn_fwd_apply_f32(const float* x, const float* mean, const float* invstd, const float* gamma,
+static int bn_fwd_apply(const float* x, const float* mean, const float* invstd, const float* gamma,
                         const float* beta, float* y, int64_t N, int64_t C, int64_t HW,
-                        mn_stream_t stream) {
+                        mn_stream_t stream, bool relu) {
   using namespace mn_bn;
   if (N < 0 || C < 0 || HW < 0) return MN_EINVAL;
   if (N == 0 || C == 0 || HW == 0) return MN_OK;
@@ -741,6 +780,7 @@ int mn_bn_fwd_apply_f32(const float* x, const float* mean, const float* invstd, 
   A.gamma = gamma;
   A.shift = beta;
   A.out = y;
+  A.relu = relu ? 1 : 0;
   const unsigned blocks = (unsigned)C * A.sh.S;
   hipStream_t s = mn_stream(stream);
   if (vec == 4)
@@ -748,6 +788,36 @@ int mn_bn_fwd_apply_f32(const float* x, const float* mean, const float* invstd, 
   else
     bn_fwd_saved_kernel<1><<<blocks, kThreads, 0, s>>>(A, mean, invstd);
   return mn_launch_status();
+}
+
+int mn_bn_fwd_apply_f32(const float* x, const float* mean, const float* invstd, const float* gamma,
+                        const float* beta, float* y, int64_t N, int64_t C, int64_t HW,
+                        mn_stream_t stream) {
+  return bn_fwd_apply(x, mean, invstd, gamma, beta, y, N, C, HW, stream, false);
+}
+
+int mn_bn_relu_fwd_train_f32(const float* x, const float* gamma, const float* beta,
+                             float* running_mean, float* running_var, float* y, float* save_mean,
+                             float* save_invstd, int64_t N, int64_t C, int64_t HW, double momentum,
+                             double eps, void* ws, size_t ws_bytes, mn_stream_t stream) {
+  return mn_bn::fwd_train_launch(x, gamma, beta, running_mean, running_var, y, save_mean,
+                                 save_invstd, N, C, HW, momentum, eps, ws, ws_bytes,
+                                 mn_stream(stream), mn_bn::Tuning(), true);
+}
+
+int mn_bn_relu_fwd_apply_f32(const float* x, const float* mean, const float* invstd,
+                             const float* gamma, const float* beta, float* y, int64_t N, int64_t C,
+                             int64_t HW, mn_stream_t stream) {
+  return bn_fwd_apply(x, mean, invstd, gamma, beta, y, N, C, HW, stream, true);
+}
+
+int mn_bn_relu_bwd_from_x_f32(const float* dy, const float* x, const float* gamma,
+                              const float* beta, const float* mean, const float* invstd, float* dx,
+                              float* dgamma, float* dbeta, int64_t N, int64_t C, int64_t HW,
+                              void* ws, size_t ws_bytes, mn_stream_t stream) {
+  if (!mean) return MN_EINVAL;
+  return mn_bn::bwd_launch(false, dy, x, gamma, mean, invstd, dx, dgamma, dbeta, N, C, HW, ws,
+                           ws_bytes, mn_stream(stream), mn_bn::Tuning(), true, beta);
 }
 
 int mn_bn_bwd_from_x_f32(const float* dy, const float* x, const float* gamma, const float* mean,

@@ -33,25 +33,27 @@ def _workspace(N, C, HW, device):
     return torch.empty(max(nbytes, 4), dtype=torch.uint8, device=device), nbytes
 
 
-def bn_forward_train(x, weight, bias, running_mean, running_var, momentum, eps, out=None):
-    """Training forward -> (y, save_mean, save_invstd)."""
+def bn_forward_train(x, weight, bias, running_mean, running_var, momentum, eps, out=None,
+                     relu=False):
+    """Training forward -> (y, save_mean, save_invstd); relu=True applies max(., 0) to y."""
     xc, N, C, HW = _as_nchw(x, "input")
     y = torch.empty_like(xc) if out is None else out
     save_mean = torch.empty(C, dtype=torch.float32, device=x.device)
     save_invstd = torch.empty(C, dtype=torch.float32, device=x.device)
     ws, nbytes = _workspace(N, C, HW, x.device)
-    _lib.call("mn_bn_fwd_train_f32", _lib.ptr(xc), _lib.ptr(weight), _lib.ptr(bias),
+    _lib.call("mn_bn_relu_fwd_train_f32" if relu else "mn_bn_fwd_train_f32", _lib.ptr(xc), _lib.ptr(weight), _lib.ptr(bias),
               _lib.ptr(running_mean), _lib.ptr(running_var), _lib.ptr(y), _lib.ptr(save_mean),
               _lib.ptr(save_invstd), N, C, HW, float(momentum), float(eps), _lib.ptr(ws), nbytes,
               _lib.stream_ptr(x.device))
     return y, save_mean, save_invstd
 
 
-def bn_forward_apply(x, mean, invstd, weight, bias):
-    """y = (x - mean) * invstd * weight + bias with given per-channel vectors."""
+def bn_forward_apply(x, mean, invstd, weight, bias, relu=False):
+    """y = (x - mean) * invstd * weight + bias with given per-channel vectors (then max(., 0)
+    if relu)."""
     xc, N, C, HW = _as_nchw(x, "input")
     y = torch.empty_like(xc)
-    _lib.call("mn_bn_fwd_apply_f32", _lib.ptr(xc), _lib.ptr(mean), _lib.ptr(invstd),
+    _lib.call("mn_bn_relu_fwd_apply_f32" if relu else "mn_bn_fwd_apply_f32", _lib.ptr(xc), _lib.ptr(mean), _lib.ptr(invstd),
               _lib.ptr(weight), _lib.ptr(bias), _lib.ptr(y), N, C, HW, _lib.stream_ptr(x.device))
     return y
 
@@ -72,6 +74,24 @@ def _bn_backward(entry, grad, t, weight, shift, invstd):
     return dx, dw, db
 
 
+def bn_relu_backward_from_input(grad, x, weight, bias, save_mean, save_invstd):
+    """Backward of relu(BN(x)) from the stored input: `grad` is the gradient of the ReLU
+    output; the kernel recomputes where the pre-activation was positive."""
+    tc, N, C, HW = _as_nchw(x, "stored activation")
+    g = grad if grad.is_contiguous() else grad.contiguous()
+    _lib.require_gpu_tensor(g, "grad_output", torch.float32)
+    if g.shape != tc.shape:
+        raise RuntimeError("grad_output and the stored activation differ in shape")
+    dx = torch.empty_like(tc)
+    dw = torch.empty(C, dtype=torch.float32, device=x.device)
+    db = torch.empty(C, dtype=torch.float32, device=x.device)
+    ws, nbytes = _workspace(N, C, HW, x.device)
+    _lib.call("mn_bn_relu_bwd_from_x_f32", _lib.ptr(g), _lib.ptr(tc), _lib.ptr(weight), _lib.ptr(bias),
+              _lib.ptr(save_mean), _lib.ptr(save_invstd), _lib.ptr(dx), _lib.ptr(dw), _lib.ptr(db),
+              N, C, HW, _lib.ptr(ws), nbytes, _lib.stream_ptr(x.device))
+    return dx, dw, db
+
+
 def bn_backward_from_input(grad, x, weight, save_mean, save_invstd):
     return _bn_backward("mn_bn_bwd_from_x_f32", grad, x, weight, save_mean, save_invstd)
 
@@ -84,6 +104,7 @@ class _BatchNormForward(OP):
     params = None   # (training, eps, save_mean, save_invstd, reserve)
     running_mean = None
     running_var = None
+    fused_relu = False
 
     def forward(self, input_, weight, bias, running_mean, running_var,
                 training=False, momentum=0.1, eps=1e-5, *args, **kwargs):
@@ -94,16 +115,19 @@ class _BatchNormForward(OP):
             if self.params is None:
                 if training:
                     out, save_mean, save_invstd = bn_forward_train(
-                        input_, weight, bias, self.running_mean, self.running_var, momentum, eps)
+                        input_, weight, bias, self.running_mean, self.running_var, momentum, eps,
+                        relu=self.fused_relu)
                 else:
                     # inference statistics: normalise with the running ones
                     save_mean = self.running_mean
                     save_invstd = torch.rsqrt(self.running_var + eps)
-                    out = bn_forward_apply(input_, save_mean, save_invstd, weight, bias)
+                    out = bn_forward_apply(input_, save_mean, save_invstd, weight, bias,
+                                           relu=self.fused_relu)
                 self.params = bool(training), eps, save_mean, save_invstd, None
             else:
                 _, _, save_mean, save_invstd, _ = self.params
-                out = bn_forward_apply(input_, save_mean, save_invstd, weight, bias)
+                out = bn_forward_apply(input_, save_mean, save_invstd, weight, bias,
+                                       relu=self.fused_relu)
             return out
 
 
@@ -136,6 +160,33 @@ class OutputActBatchNorm(_BatchNormForward):
             if not training:
                 raise NotImplementedError
             di, dw, db = bn_backward_from_output(grad_output, output, weight, bias, save_invstd)
+            if not nodel:
+                del stored[4], stored[3], stored[2], stored[1], stored[0]
+            return di, dw, db, None, None
+
+
+FUSED_BN_RELU = 'monet::batch_norm_relu'
+
+
+@implements([FUSED_BN_RELU],
+            ['normal', 'multiway', 'newnode', 'multiway_newnode', 'conv_multiway_newnode',
+             'conv_normal'])
+class InputActBatchNormReLU(_BatchNormForward):
+    """BatchNorm and the ReLU behind it as ONE operator (the tracer's optional fusion pass
+    produces `monet::batch_norm_relu` nodes; the reference has no such operator).  Keeps the
+    BatchNorm INPUT: the backward recomputes where the pre-activation was positive, so no
+    mask and no intermediate tensor exist, and each direction is one pass over the data."""
+    backward_storage = InputStorage(0, 1, 2, 3, 4)
+    fused_relu = True
+
+    def backward(self, grad_output, stored, nodel=False):
+        with torch.no_grad():
+            input_, weight, bias, running_mean, running_var = stored
+            training, eps, save_mean, save_invstd, _ = self.params
+            if not training:
+                raise NotImplementedError
+            di, dw, db = bn_relu_backward_from_input(grad_output, input_, weight, bias, save_mean,
+                                                     save_invstd)
             if not nodel:
                 del stored[4], stored[3], stored[2], stored[1], stored[0]
             return di, dw, db, None, None

@@ -263,6 +263,28 @@ def bn_fwd_apply(x, mean, invstd, gamma, beta, dtype=np.float64):
     return y.reshape(np.shape(x))
 
 
+def bn_relu_fwd_train(x, gamma, beta, running_mean, running_var, momentum, eps, dtype=np.float64):
+    """BatchNorm (training) followed by ReLU, as one operator: the composition of bn_fwd_train
+    and max(., 0).  Returns what bn_fwd_train returns with y replaced by relu(y).  (The
+    reference runs the two operators separately, monet/lm_ops/bn.py:12-54 and relu.py:9-29.)"""
+    out = list(bn_fwd_train(x, gamma, beta, running_mean, running_var, momentum, eps, dtype))
+    out[0] = np.maximum(out[0], 0)
+    return tuple(out)
+
+
+def bn_relu_bwd_from_x(dy, x, gamma, beta, mean, invstd, positive=None, dtype=np.float64):
+    """Backward of relu(BN(x)) given the gradient of the ReLU output: mask dy where the
+    pre-activation is not positive, then bn_bwd_from_x.  `positive` overrides the mask (a
+    caller comparing against another implementation passes that implementation's decisions,
+    so that pre-activations within rounding distance of zero do not count as differences)."""
+    if positive is None:
+        shape = [1, -1] + [1] * (x.ndim - 2)
+        pre = (x.astype(dtype) - mean.astype(dtype).reshape(shape)) * \
+            (invstd.astype(dtype) * gamma.astype(dtype)).reshape(shape) + beta.astype(dtype).reshape(shape)
+        positive = pre > 0
+    return bn_bwd_from_x(np.where(positive, dy, 0).astype(dy.dtype), x, gamma, mean, invstd, dtype)
+
+
 def bn_bwd_from_x(dy, x, gamma, mean, invstd, dtype=np.float64):
     """(dx, dgamma, dbeta) from the input: the standard BatchNorm backward that
     cudnn_batch_norm_backward computes for do_cudnn_backward (lrbn.cpp:43-70).

@@ -254,6 +254,35 @@ def test_bn_forward_train_and_recompute(cuda, shape):
 
 
 @pytest.mark.parametrize("shape", BN_SHAPES)
+def test_bn_relu_fused_forward_backward_and_recompute(cuda, shape):
+    """relu(BN(x)) as one operator: forward against the oracle; backward against the oracle
+    fed the GPU's own sign decisions (a pre-activation within rounding distance of zero may
+    legitimately fall on either side); recomputation from the saved statistics."""
+    x, gamma, beta, dy = bn_problem(shape, 4)
+    oy, omean, oinv, _, _ = O.bn_relu_fwd_train(x, gamma, beta, None, None, 0.1, 1e-5)
+    op = lm_ops.bn.InputActBatchNormReLU()
+    tx, tw, tb, tg = dev(x, cuda), dev(gamma, cuda), dev(beta, cuda), dev(dy, cuda)
+    C = shape[1]
+    rm, rv = torch.zeros(C, device=cuda), torch.ones(C, device=cuda)
+    y = op.forward(tx, tw, tb, rm, rv, True, 0.1, 1e-5)
+    assert_rel(host(y), oy, 1e-5, "relu(bn(x))")
+    assert float(y.min()) >= 0.0
+    # where the oracle is clearly positive / negative the GPU agrees
+    clear = np.abs(O.bn_fwd_train(x, gamma, beta, None, None, 0.1, 1e-5)[0]) > 1e-4
+    assert np.array_equal((host(y) > 0)[clear], (oy > 0)[clear])
+    y2 = op.forward(tx, tw, tb, rm, rv, True, 0.1, 1e-5)          # recomputation
+    assert_rel(host(y2), host(y), 2e-7, "recomputed relu(bn(x))")
+    assert np.array_equal(host(y2) > 0, host(y) > 0)
+    odx, odg, odb = O.bn_relu_bwd_from_x(dy, x, gamma, beta, omean, oinv, positive=host(y) > 0)
+    stored = [tx, tw, tb, rm, rv]
+    dx, dg, db, n1, n2 = op.backward(tg.clone(), stored)
+    assert stored == [] and n1 is None and n2 is None
+    assert_rel(host(dx), odx, 1e-5, "dx")
+    assert_rel(host(dg), odg, 3e-5, "dgamma")
+    assert_rel(host(db), odb, 3e-5, "dbeta")
+
+
+@pytest.mark.parametrize("shape", BN_SHAPES)
 def test_bn_backward_from_input_and_from_output(cuda, shape):
     x, gamma, beta, dy = bn_problem(shape, 1)
     oy, omean, oinv, _, _ = O.bn_fwd_train(x, gamma, beta, None, None, 0.1, 1e-5)

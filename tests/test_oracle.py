@@ -244,6 +244,26 @@ def test_bn_backward_both_forms_match_autograd(shape):
         np.testing.assert_allclose(dx.sum(axis=(0, 2, 3)), 0, atol=1e-9)
 
 
+@pytest.mark.parametrize("shape", [(4, 3, 5, 5), (2, 8, 7, 3), (16, 4, 6, 6)])
+def test_bn_relu_fused_matches_autograd_of_the_composition(shape):
+    x, gamma, beta, dy = _bn_problem(shape, 5)
+    tx = torch.from_numpy(x).requires_grad_(True)
+    tw = torch.from_numpy(gamma).requires_grad_(True)
+    tb = torch.from_numpy(beta).requires_grad_(True)
+    ty = torch.relu(F.batch_norm(tx, None, None, tw, tb, True, 0.1, 1e-5))
+    ty.backward(torch.from_numpy(dy))
+    y, mean, invstd, _, _ = O.bn_relu_fwd_train(x, gamma, beta, None, None, 0.1, 1e-5)
+    np.testing.assert_allclose(y, ty.detach().numpy(), rtol=1e-12, atol=1e-14)
+    assert (y >= 0).all() and (y == 0).any()
+    dx, dg, db = O.bn_relu_bwd_from_x(dy, x, gamma, beta, mean, invstd)
+    np.testing.assert_allclose(dx, tx.grad.numpy(), rtol=1e-9, atol=1e-10)
+    np.testing.assert_allclose(dg, tw.grad.numpy(), rtol=1e-9, atol=1e-10)
+    np.testing.assert_allclose(db, tb.grad.numpy(), rtol=1e-9, atol=1e-10)
+    # an explicit mask replaces the recomputed one
+    dx2, _, _ = O.bn_relu_bwd_from_x(dy, x, gamma, beta, mean, invstd, positive=y > 0)
+    np.testing.assert_allclose(dx2, dx, rtol=1e-12)
+
+
 # ------------------------------------------------------------------- softmax
 @pytest.mark.parametrize("shape,dim", [((7, 10), 1), ((3, 2, 5, 4), 1), ((4, 6, 3), 2), ((5,), 0)])
 def test_softmax_matches_torch(shape, dim):
