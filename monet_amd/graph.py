@@ -94,6 +94,15 @@ class ComputeNode(Node):
         return '<Op %s %s>' % (str(self._op), str(list(self.shape)))
 
 
+FUSED_BN_RELU = "monet::batch_norm_relu"
+
+
+def is_batch_norm(op_name):
+    """BatchNorm, alone or fused with the ReLU behind it: operators whose first forward of a
+    step computes statistics that recomputations and the backward must reuse."""
+    return op_name in ("aten::batch_norm", FUSED_BN_RELU)
+
+
 def two_step_backward(node):
     """Operators whose backward is split into a parameter-gradient step and an
     input-gradient step (non-depthwise convolution and the fully connected
@@ -115,8 +124,50 @@ class Graph:
         self._nodes.append(node)
         return len(self._nodes) - 1
 
+    def fuse_batch_norm_relu(self):
+        """New graph in which every BatchNorm whose only reader is a ReLU forms ONE
+        `monet::batch_norm_relu` node with it (same arguments as the BatchNorm).  The reference
+        has no such pass; it halves the memory passes of the pair and needs no ReLU mask."""
+        nodes = self._nodes
+        readers = [0] * len(nodes)
+        for n in nodes:
+            if isinstance(n, ComputeNode):
+                for a in n.args:
+                    if isinstance(a, ComputeNode.D):
+                        readers[a.index] += 1
+        for o in self._outputs:
+            readers[o] += 1
+        fused_into = {}  # index of the ReLU node -> index of its BatchNorm
+        for j, n in enumerate(nodes):
+            if isinstance(n, ComputeNode) and n.op in ("aten::relu", "aten::relu_"):
+                src = [a.index for a in n.args if isinstance(a, ComputeNode.D)]
+                if len(src) == 1 and isinstance(nodes[src[0]], ComputeNode) and \
+                        nodes[src[0]].op == "aten::batch_norm" and readers[src[0]] == 1:
+                    fused_into[j] = src[0]
+        g = Graph()
+        new_index = {}
+        for k, n in enumerate(nodes):
+            if k in fused_into:
+                new_index[k] = new_index[fused_into[k]]
+                continue
+            if isinstance(n, ComputeNode):
+                args = [ComputeNode.D(new_index[a.index], a.requires_grad)
+                        if isinstance(a, ComputeNode.D) else a for a in n.args]
+                op = FUSED_BN_RELU if k in fused_into.values() else n.op
+                new_index[k] = g._add(ComputeNode(n.shape, len(g._nodes), op, args, n.has_backward,
+                                                  n.is_depthwise))
+            else:
+                new_index[k] = g._add(n)
+        g._outputs = [new_index[o] for o in self._outputs]
+        return g
+
     @classmethod
-    def create(cls, model, input_shape=(3, 224, 224)):
+    def create(cls, model, input_shape=(3, 224, 224), fuse_bn_relu=False):
+        g = cls._trace(model, input_shape)
+        return g.fuse_batch_norm_relu() if fuse_bn_relu else g
+
+    @classmethod
+    def _trace(cls, model, input_shape):
         example = (torch.ones((TRACE_BATCH,) + tuple(input_shape)),)
         trace, _ = torch.jit._get_trace_graph(model, example, _force_outplace=False,
                                               _return_inputs_states=False)

@@ -21,7 +21,7 @@ import numpy as np
 import torch
 
 from . import lm_ops
-from .graph import ComputeNode, Param, two_step_backward
+from .graph import ComputeNode, Param, is_batch_norm, two_step_backward
 
 RUNTIME_SAMPLES = 20
 
@@ -147,7 +147,7 @@ def computeinfo(n, op, graph, bs, bwd_op, conv_mode, inplace_mode, *params):
             runtime_fwd.append(_timed(lambda: op.forward(*args)))
         op.inplace = False
         outs = op.forward(*args)
-    elif n.op == "aten::batch_norm":
+    elif is_batch_norm(n.op):
         def first_forward():
             op.params = None
             return op.forward(*args)
@@ -215,7 +215,7 @@ def meminfo(n, op, graph, bs, bwd_op, conv_mode, inplace_mode, *params):
             outs = None
             ws, outs = _peak_over_outputs(lambda: op.forward(*args))
             fwd_mem.append(ws)
-    elif n.op == "aten::batch_norm":
+    elif is_batch_norm(n.op):
         ws, outs = _peak_over_outputs(lambda: op.forward(*args))       # first forward
         fwd_mem.append(ws)
         outs = None

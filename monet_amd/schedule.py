@@ -34,7 +34,7 @@ from collections import defaultdict, namedtuple
 import torch
 
 from . import lm_ops
-from .graph import ComputeNode, Graph, two_step_backward
+from .graph import ComputeNode, Graph, is_batch_norm, two_step_backward
 from .solver_info import BwdNode, IntNode, SolverInfo
 
 ScheduleType = namedtuple('ScheduleType', 'recompute store_output store_intermediate')
@@ -195,7 +195,7 @@ class Schedule(Graph):
                                 "nor recomputed" % (t, n.op, k, a.index)
                     args = tuple((False, a.value) if isinstance(a, ComputeNode.V)
                                  else (True, (a.index, a.requires_grad)) for a in n.args)
-                    is_bn = n.op == "aten::batch_norm"
+                    is_bn = is_batch_norm(n.op)
                     if is_bn and t == 0:
                         self._ops0.append(op)
                     inplace_src = -1
@@ -377,9 +377,9 @@ def create_schedule(model, sol_file, input_shape=(3, 224, 224)):
     if m._get_name() == 'MobileNetV2':
         m = torch.nn.Sequential(m.features, torch.nn.AdaptiveAvgPool2d((1, 1)),
                                 torch.nn.Flatten(start_dim=1), m.classifier[0], m.classifier[1])
-    graph = Graph.create(m, input_shape)
-    del m
     solver_info, solution = load_solution(sol_file)
+    graph = Graph.create(m, input_shape, fuse_bn_relu=getattr(solver_info, "fuse_bn_relu", False))
+    del m
     schedule = Schedule(graph, solver_info)
     schedule.init_schedule(solution, solver_info.mode)
     return schedule
@@ -429,9 +429,10 @@ def main(argv=None):
     model, input_shape, model_name = build_model(args.model)
     if args.check_diff:
         disable_dropout(model)
-    graph = Graph.create(model, input_shape=input_shape)
-    model.cuda()
     si, solution = load_solution(args.solution_file)
+    graph = Graph.create(model, input_shape=input_shape,
+                         fuse_bn_relu=getattr(si, "fuse_bn_relu", False))
+    model.cuda()
     schedule = Schedule(graph, si)
     schedule.init_schedule(solution, si.mode)
     input_ = torch.randn((args.bs,) + tuple(input_shape)).cuda()

@@ -27,7 +27,7 @@ from pathlib import Path
 import numpy as np
 
 from . import lm_ops
-from .graph import ComputeNode, Graph, Input, Param, two_step_backward
+from .graph import ComputeNode, Graph, Input, Param, is_batch_norm, two_step_backward
 
 MEMORY_MULTIPLIER = 4  # bytes per element: the path is fp32 (solver_info.py:10)
 
@@ -126,7 +126,10 @@ class SolverInfo:
         self.select_conv_algo = "conv" in mode
         self.do_inplace = "inplace" in mode
         self.compute_newnode = "newnode" in mode
-        self.mode = mode.replace("inplace_", "")  # the registry knows nothing of "inplace_"
+        # "fused_": the graph was traced with BatchNorm+ReLU pairs as single operators
+        self.fuse_bn_relu = "fused" in mode
+        # the registry knows nothing of these prefixes
+        self.mode = mode.replace("fused_", "").replace("inplace_", "")
 
     # ------------------------------------------------------------------ build
     def extract(self, graph: Graph, *args, cost_fn=None):
@@ -388,7 +391,7 @@ class SolverInfo:
                         b.workspace_mem.append(bmem[0])
                         b.workspace_compute.append(btime[0])
                         if not (two_step_backward(n) and b.bwd_op == "ip_grad"):
-                            if n.op == "aten::batch_norm":
+                            if is_batch_norm(n.op):
                                 fwd.recompute_workspace_mem.append(fmem_re[0])
                                 fwd.recompute_workspace_compute.append(ftime_re[0])
                             fwd.workspace_mem.append(fmem[0])

@@ -38,7 +38,7 @@ def _solve(model, shape, bs, mode, budget_gb, cuda):
     from monet_amd.graph import Graph
     from monet_amd.solver import Model
     from monet_amd.solver_info import SolverInfo
-    graph = Graph.create(copy.deepcopy(model).cpu(), shape)
+    graph = Graph.create(copy.deepcopy(model).cpu(), shape, fuse_bn_relu="fused" in mode)
     x = torch.randn((bs,) + shape, device=cuda)
     si = SolverInfo(bs, "test", mode)
     si.extract(graph, x, *list(model.state_dict(keep_vars=True).values()))
@@ -58,7 +58,8 @@ def _rel(a, b, floor=1e-30):
 
 
 @pytest.mark.parametrize("mode", ["normal", "multiway_newnode", "conv_multiway_newnode",
-                                  "inplace_conv_multiway_newnode"])
+                                  "inplace_conv_multiway_newnode",
+                                  "fused_inplace_conv_multiway_newnode"])
 def test_schedule_matches_autograd(cuda, mode):
     from monet_amd.schedule import Schedule
     torch.manual_seed(0)
@@ -69,7 +70,7 @@ def test_schedule_matches_autograd(cuda, mode):
     peak_mb = None
     solutions = [("free", free)]
     from monet_amd.solver import Model
-    for frac in (0.8, 0.65, 0.55, 0.5, 0.45):
+    for frac in (0.95, 0.9, 0.8, 0.65, 0.55, 0.5, 0.45):
         total = sum(n.mem for i, n in si.nodes.items() if i < si.loss) + si.nodes[si.loss].fixed_mem
         try:
             solutions.append(("%.2f" % frac,

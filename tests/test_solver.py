@@ -42,7 +42,7 @@ def synthetic_cost(si):
                    ([mb] * nf, [mb * (1.0 - 0.1 * c) for c in range(nb)], [])
         if si.do_inplace and hasattr(op, 'inplace'):
             return ([0.0, 0.0], [0.0], []), ([0.1 * mb, 0.1 * mb], [0.1 * mb], [])
-        if n.op == "aten::batch_norm":
+        if n.op in ("aten::batch_norm", "monet::batch_norm_relu"):
             return ([0.0], [0.0], [0.0]), ([0.2 * mb], [0.3 * mb], [0.1 * mb])
         # implementations that keep an intermediate are a bit slower
         extra = 0.02 * mb if "Binary" in type(op).__name__ or "Indices" in type(op).__name__ else 0
@@ -256,3 +256,23 @@ def test_model_definitions_trace_to_the_expected_operators():
     uops = Counter(n.op for n in gu.nodes if isinstance(n, ComputeNode))
     assert uops == {"aten::_convolution": 19, "aten::batch_norm": 18, "aten::relu_": 18,
                     "aten::max_pool2d": 4, "aten::adaptive_avg_pool2d": 4, "aten::cat": 4}
+
+
+def test_batch_norm_relu_fusion_pass():
+    """BatchNorm nodes whose only reader is a ReLU merge with it; others stay."""
+    g = Graph.create(SmallNet(), (3, 16, 16))
+    f = Graph.create(SmallNet(), (3, 16, 16), fuse_bn_relu=True)
+    kinds = [n.op for n in f.nodes if isinstance(n, ComputeNode)]
+    # b1 -> relu fuses; b2 feeds the residual add, so it stays a plain BatchNorm
+    assert kinds == ["aten::_convolution", "monet::batch_norm_relu", "aten::max_pool2d",
+                     "aten::_convolution", "aten::batch_norm", "aten::add_", "aten::relu_",
+                     "aten::adaptive_avg_pool2d", "aten::flatten", "aten::linear"]
+    assert len(f.nodes) == len(g.nodes) - 1 and f._outputs == [len(f.nodes) - 1]
+    pool = next(n for n in f.nodes if isinstance(n, ComputeNode) and n.op == "aten::max_pool2d")
+    fused = f.nodes[pool.args[0].index]
+    assert fused.op == "monet::batch_norm_relu" and len(fused.args) == 9  # the BatchNorm's arguments
+    si = SolverInfo(16, "small", "fused_inplace_conv_multiway_newnode")
+    si.extract(f, cost_fn=synthetic_cost(si))
+    assert si.fuse_bn_relu and si.mode == "conv_multiway_newnode"
+    sol = Model(si, budget=1.0, time_limit=60, mip_rel_gap=0.0).solve()
+    Schedule(f, si).init_schedule(sol, si.mode)
