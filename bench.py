@@ -267,23 +267,25 @@ def end_to_end(iters=10, warmup=3):
     target = torch.randint(0, 1000, (E2E_BS,), device=dev)
     res = {"model": "resnet50", "batch": E2E_BS, "dtype": "f32", "unit": "images/s",
            "step": "forward + cross entropy + backward + SGD momentum update"}
-    base = None
-    for budget in (100, 10, 6):
-        sol = ROOT / "data" / ("solution_resnet50_%d_%s_%.2f.pkl" % (E2E_BS, E2E_MODE, budget))
-        if not sol.exists():
-            continue
-        model = MONeTWrapper(resnet50(), str(sol), (3, 224, 224)).to(dev)
-        model.train()
-        ms, mb = _train_ms(model, x, target, iters, warmup)
-        key = "unconstrained" if budget == 100 else "budget_%dGB" % budget
-        res[key] = {"images_per_s": round(E2E_BS / ms * 1e3, 1), "ms_per_step": round(ms, 2),
-                    "peak_MB": round(mb, 1)}
-        if budget == 100:
-            base = ms
-        elif base:
-            res[key]["overhead_vs_unconstrained"] = round(ms / base - 1.0, 4)
-        del model
-        torch.cuda.empty_cache()
+    # op set of the reference, then the same with BatchNorm+ReLU pairs fused into one operator
+    for suffix, mode in (("", E2E_MODE), ("_fused", "fused_" + E2E_MODE)):
+        base = None
+        for budget in (100, 10, 6):
+            sol = ROOT / "data" / ("solution_resnet50_%d_%s_%.2f.pkl" % (E2E_BS, mode, budget))
+            if not sol.exists():
+                continue
+            model = MONeTWrapper(resnet50(), str(sol), (3, 224, 224)).to(dev)
+            model.train()
+            ms, mb = _train_ms(model, x, target, iters, warmup)
+            key = ("unconstrained" if budget == 100 else "budget_%dGB" % budget) + suffix
+            res[key] = {"images_per_s": round(E2E_BS / ms * 1e3, 1), "ms_per_step": round(ms, 2),
+                        "peak_MB": round(mb, 1)}
+            if budget == 100:
+                base = ms
+            elif base:
+                res[key]["overhead_vs_unconstrained"] = round(ms / base - 1.0, 4)
+            del model
+            torch.cuda.empty_cache()
     model = resnet50().to(dev).train()
     ms, mb = _train_ms(model, x, target, iters, warmup)
     res["stock_pytorch"] = {"images_per_s": round(E2E_BS / ms * 1e3, 1),
