@@ -157,6 +157,14 @@ int mn_softmax_bwd_f32(const float* dy, const float* y, float* dx, int64_t outer
 int mn_xent_bwd_f32(const float* logits, const int64_t* labels, float* dlogits, int64_t outer,
                     int64_t dim, int64_t inner, float scale, mn_stream_t stream);
 
+/* y = max(a + alpha*b, 0) and, if mask != NULL, the packed 1-bit mask of
+ * (a + alpha*b > 0) in the format of mn_pack_bits: the residual add and the
+ * ReLU behind it in one pass.  y may alias a.  No counterpart in the reference
+ * (it runs AddIP, monet/lm_ops/funcs.py:41-59, then a ReLU operator); the
+ * backward of the pair is mn_relu_bwd_mask_f32 / mn_relu_bwd_ref_f32 on y. */
+int mn_add_relu_fwd_f32(const float* a, const float* b, float alpha, float* y, uint8_t* mask,
+                        size_t n, mn_stream_t stream);
+
 /* BatchNorm fused with the ReLU that follows it (no counterpart in the
  * reference, whose executor runs them as two operators, monet/lm_ops/bn.py and
  * relu.py; fusing saves one read and one write of the activation in each

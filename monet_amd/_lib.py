@@ -56,6 +56,7 @@ _SIGNATURES = {
     "mn_pack_nibbles": (c_int, [_P, _P, c_size_t, _P]),
     "mn_unpack_nibbles": (c_int, [_P, _P, c_size_t, _P]),
     "mn_relu_fwd_mask_f32": (c_int, [_P, _P, _P, c_size_t, _P]),
+    "mn_add_relu_fwd_f32": (c_int, [_P, _P, c_float, _P, _P, c_size_t, _P]),
     "mn_relu_bwd_mask_f32": (c_int, [_P, _P, _P, c_size_t, _P]),
     "mn_relu_bwd_ref_f32": (c_int, [_P, _P, c_float, _P, c_size_t, _P]),
     "mn_pool_out_size": (c_int64, [c_int64, c_int64, c_int64, c_int64, c_int64, c_int]),

@@ -95,6 +95,8 @@ class ComputeNode(Node):
 
 
 FUSED_BN_RELU = "monet::batch_norm_relu"
+FUSED_ADD_RELU = "monet::add_relu"
+_FUSABLE = {"aten::batch_norm": FUSED_BN_RELU, "aten::add_": FUSED_ADD_RELU, "aten::add": FUSED_ADD_RELU}
 
 
 def is_batch_norm(op_name):
@@ -125,9 +127,10 @@ class Graph:
         return len(self._nodes) - 1
 
     def fuse_batch_norm_relu(self):
-        """New graph in which every BatchNorm whose only reader is a ReLU forms ONE
-        `monet::batch_norm_relu` node with it (same arguments as the BatchNorm).  The reference
-        has no such pass; it halves the memory passes of the pair and needs no ReLU mask."""
+        """New graph in which every BatchNorm or residual add whose only reader is a ReLU forms
+        ONE node with it (`monet::batch_norm_relu` / `monet::add_relu`, with the arguments of the
+        first operator).  The reference has no such pass; a fused pair makes one pass over the
+        activation where the two operators make two."""
         nodes = self._nodes
         readers = [0] * len(nodes)
         for n in nodes:
@@ -142,7 +145,8 @@ class Graph:
             if isinstance(n, ComputeNode) and n.op in ("aten::relu", "aten::relu_"):
                 src = [a.index for a in n.args if isinstance(a, ComputeNode.D)]
                 if len(src) == 1 and isinstance(nodes[src[0]], ComputeNode) and \
-                        nodes[src[0]].op == "aten::batch_norm" and readers[src[0]] == 1:
+                        nodes[src[0]].op in _FUSABLE and readers[src[0]] == 1 and \
+                        self._add_is_fusable(nodes[src[0]]):
                     fused_into[j] = src[0]
         g = Graph()
         new_index = {}
@@ -153,13 +157,22 @@ class Graph:
             if isinstance(n, ComputeNode):
                 args = [ComputeNode.D(new_index[a.index], a.requires_grad)
                         if isinstance(a, ComputeNode.D) else a for a in n.args]
-                op = FUSED_BN_RELU if k in fused_into.values() else n.op
+                op = _FUSABLE[n.op] if k in fused_into.values() else n.op
                 new_index[k] = g._add(ComputeNode(n.shape, len(g._nodes), op, args, n.has_backward,
                                                   n.is_depthwise))
             else:
                 new_index[k] = g._add(n)
         g._outputs = [new_index[o] for o in self._outputs]
         return g
+
+    def _add_is_fusable(self, n):
+        """An add fuses only if both operands are activations of the output's shape (no
+        broadcasting, no parameter operand)."""
+        if n.op == "aten::batch_norm":
+            return True
+        ops = [a for a in n.args if isinstance(a, ComputeNode.D)]
+        return len(ops) == 2 and all(isinstance(self._nodes[a.index], ComputeNode) and
+                                     list(self._nodes[a.index].shape) == list(n.shape) for a in ops)
 
     @classmethod
     def create(cls, model, input_shape=(3, 224, 224), fuse_bn_relu=False):

@@ -2,7 +2,9 @@
 monet/lm_ops/funcs.py:7-59).  Bandwidth-bound but stock: they call PyTorch."""
 import torch
 
-from .base import OP, implements
+from .. import _lib
+from .base import OP, IntermediateStorage, OutputStorage, implements
+from .relu import _f32_contig, _numel, relu_backward_from_mask, relu_backward_from_ref
 
 _ALL = ['normal', 'multiway', 'newnode', 'multiway_newnode', 'conv_multiway_newnode', 'conv_normal']
 
@@ -62,3 +64,71 @@ class AddIP(_AddBase):
             if self.inplace:
                 return a.add_(b, alpha=s)
             return torch.add(a, b, alpha=s)
+
+
+FUSED_ADD_RELU = 'monet::add_relu'
+
+
+def add_relu_forward(a, b, alpha, inplace=False, want_mask=False):
+    """(max(a + alpha*b, 0), packed mask of a + alpha*b > 0 or None) in one pass; writes into
+    `a` when `inplace`."""
+    ac, bc = _f32_contig(a, "a"), _f32_contig(b, "b")
+    if ac.shape != bc.shape:
+        raise RuntimeError("the fused add needs operands of one shape")
+    n = ac.numel()
+    y = ac if (inplace and ac is a) else torch.empty_like(ac)
+    mask = torch.empty((n + 7) // 8, dtype=torch.uint8, device=a.device) if want_mask else None
+    _lib.call("mn_add_relu_fwd_f32", _lib.ptr(ac), _lib.ptr(bc), float(alpha), _lib.ptr(y),
+              _lib.ptr(mask), n, _lib.stream_ptr(a.device))
+    if inplace and ac is not a:
+        a.copy_(y)
+        y = a
+    return y, mask
+
+
+class _AddReLUBase(OP):
+    """The residual add and the ReLU behind it as ONE operator (`monet::add_relu` nodes come
+    from the tracer's optional fusion pass; arguments are those of aten::add_: a, b, alpha).
+    Both inputs receive the ReLU-masked gradient (b's scaled by alpha)."""
+    params = None
+    inplace = False
+
+    def _split(self, g):
+        s = self.params
+        return g, (g if s == 1 else g * s)
+
+
+@implements([FUSED_ADD_RELU],
+            ['normal', 'multiway', 'newnode', 'multiway_newnode', 'conv_multiway_newnode',
+             'conv_normal'])
+class OutputActAddReLU(_AddReLUBase):
+    backward_storage = OutputStorage()
+
+    def forward(self, a, b, s):
+        with torch.no_grad():
+            self.params = s
+            return add_relu_forward(a, b, s, inplace=self.inplace)[0]
+
+    def backward(self, grad, stored, nodel=False):
+        with torch.no_grad():
+            out = stored[0]
+            if not nodel:
+                del stored[0]
+            return self._split(relu_backward_from_ref(grad, out))
+
+
+@implements([FUSED_ADD_RELU], ['newnode', 'multiway_newnode', 'conv_multiway_newnode'])
+class BinaryActAddReLU(_AddReLUBase):
+    backward_storage = IntermediateStorage(lambda shape: (_numel(shape) + 7) // 8)
+
+    def forward(self, a, b, s):
+        with torch.no_grad():
+            self.params = s
+            return add_relu_forward(a, b, s, inplace=self.inplace, want_mask=True)
+
+    def backward(self, grad, stored, nodel=False):
+        with torch.no_grad():
+            mask = stored[0]
+            if not nodel:
+                del stored[0]
+            return self._split(relu_backward_from_mask(grad, mask))

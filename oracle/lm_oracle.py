@@ -263,6 +263,14 @@ def bn_fwd_apply(x, mean, invstd, gamma, beta, dtype=np.float64):
     return y.reshape(np.shape(x))
 
 
+def add_relu_fwd(a, b, alpha=1.0):
+    """(max(a + alpha*b, 0), packed 1-bit mask of a + alpha*b > 0) in the operands' dtype: the
+    composition of AddIP (monet/lm_ops/funcs.py:41-59) and a ReLU with BinaryActReLU's mask
+    (relu.py:94-118).  Pinned through relu_fwd_mask and plain numpy addition."""
+    t = (a + np.asarray(alpha, dtype=a.dtype) * b).astype(a.dtype)
+    return relu_fwd_mask(t)
+
+
 def bn_relu_fwd_train(x, gamma, beta, running_mean, running_var, momentum, eps, dtype=np.float64):
     """BatchNorm (training) followed by ReLU, as one operator: the composition of bn_fwd_train
     and max(., 0).  Returns what bn_fwd_train returns with y replaced by relu(y).  (The

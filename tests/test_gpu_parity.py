@@ -253,6 +253,42 @@ def test_bn_forward_train_and_recompute(cuda, shape):
     assert_rel(host(y2), host(y), 2e-7, "recomputed y")
 
 
+@pytest.mark.parametrize("n", [1, 7, 8, 31, 32, 33, 1000, 4099, 1 << 18])
+@pytest.mark.parametrize("cls", ["OutputActAddReLU", "BinaryActAddReLU"])
+def test_add_relu_fused(cuda, cls, n):
+    """relu(a + b) as one operator: output, mask and both gradients exact (alpha = 1 is a plain
+    fp32 addition), out of place and in place; unaligned views take the scalar kernel."""
+    rng = np.random.default_rng(n)
+    a = rng.standard_normal(n + 3).astype(np.float32)
+    b = rng.standard_normal(n + 3).astype(np.float32)
+    b[::5] = -a[::5]                       # exact zeros in the sum
+    dy = rng.standard_normal(n).astype(np.float32)
+    for off in (0, 3):                     # 3: breaks the 16-byte alignment
+        av, bv = a[off:off + n], b[off:off + n]
+        oy, omask = O.add_relu_fwd(av, bv)
+        for inplace in (False, True):
+            op = getattr(lm_ops.funcs, cls)()
+            op.inplace = inplace
+            ta, tb = dev(a, cuda)[off:off + n], dev(b, cuda)[off:off + n]
+            res = op.forward(ta, tb, 1)
+            y, mask = res if isinstance(res, tuple) else (res, None)
+            assert np.array_equal(host(y), oy)
+            if inplace:
+                assert y.data_ptr() == ta.data_ptr()
+            if mask is not None:
+                assert np.array_equal(host(mask), omask)
+            stored = [mask if mask is not None else y]
+            ga, gb = op.backward(dev(dy, cuda), stored)
+            assert stored == []
+            exp = np.where(oy > 0, dy, 0).astype(np.float32)
+            assert np.array_equal(host(ga), exp) and np.array_equal(host(gb), exp)
+    # alpha != 1: the kernel may contract a + alpha*b into one fused multiply-add
+    op = getattr(lm_ops.funcs, cls)()
+    res = op.forward(dev(a[:n], cuda), dev(b[:n], cuda), 0.5)
+    y = res[0] if isinstance(res, tuple) else res
+    np.testing.assert_allclose(host(y), np.maximum(a[:n] + 0.5 * b[:n], 0), rtol=0, atol=1e-6)
+
+
 @pytest.mark.parametrize("shape", BN_SHAPES)
 def test_bn_relu_fused_forward_backward_and_recompute(cuda, shape):
     """relu(BN(x)) as one operator: forward against the oracle; backward against the oracle

@@ -244,6 +244,16 @@ def test_bn_backward_both_forms_match_autograd(shape):
         np.testing.assert_allclose(dx.sum(axis=(0, 2, 3)), 0, atol=1e-9)
 
 
+def test_add_relu_is_the_composition():
+    rng = np.random.default_rng(6)
+    a = rng.standard_normal(1001).astype(np.float32)
+    b = rng.standard_normal(1001).astype(np.float32)
+    y, mask = O.add_relu_fwd(a, b)
+    t = torch.relu(torch.from_numpy(a) + torch.from_numpy(b)).numpy()
+    assert np.array_equal(y, t)
+    assert np.array_equal(O.unpack_bits(mask, 1001), (a + b) > 0)
+
+
 @pytest.mark.parametrize("shape", [(4, 3, 5, 5), (2, 8, 7, 3), (16, 4, 6, 6)])
 def test_bn_relu_fused_matches_autograd_of_the_composition(shape):
     x, gamma, beta, dy = _bn_problem(shape, 5)

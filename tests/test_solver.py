@@ -263,11 +263,12 @@ def test_batch_norm_relu_fusion_pass():
     g = Graph.create(SmallNet(), (3, 16, 16))
     f = Graph.create(SmallNet(), (3, 16, 16), fuse_bn_relu=True)
     kinds = [n.op for n in f.nodes if isinstance(n, ComputeNode)]
-    # b1 -> relu fuses; b2 feeds the residual add, so it stays a plain BatchNorm
+    # b1 -> relu fuses; b2 feeds the residual add, so it stays a plain BatchNorm, and the add
+    # fuses with the ReLU behind it
     assert kinds == ["aten::_convolution", "monet::batch_norm_relu", "aten::max_pool2d",
-                     "aten::_convolution", "aten::batch_norm", "aten::add_", "aten::relu_",
+                     "aten::_convolution", "aten::batch_norm", "monet::add_relu",
                      "aten::adaptive_avg_pool2d", "aten::flatten", "aten::linear"]
-    assert len(f.nodes) == len(g.nodes) - 1 and f._outputs == [len(f.nodes) - 1]
+    assert len(f.nodes) == len(g.nodes) - 2 and f._outputs == [len(f.nodes) - 1]
     pool = next(n for n in f.nodes if isinstance(n, ComputeNode) and n.op == "aten::max_pool2d")
     fused = f.nodes[pool.args[0].index]
     assert fused.op == "monet::batch_norm_relu" and len(fused.args) == 9  # the BatchNorm's arguments
