@@ -246,6 +246,14 @@ int mn_conv_fwd(const mn_conv2d* g, const void* x, const void* w, const void* bi
  * cudnn_convolution_backward_input (conv.cpp:503-515, raw call :409-449). */
 int mn_conv_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void* dx, void* ws,
                      size_t ws_bytes, int variant, int dtype, mn_stream_t stream);
+/* dx += gradient w.r.t. the input (fp32 only): the same kernels with an
+ * accumulating epilogue, for a caller that would otherwise add the result to
+ * a gradient it already holds (a residual join).  cuDNN offers this as beta = 1
+ * in cudnnConvolutionBackwardData; the reference always passes beta = 0
+ * (conv.cpp:409-449) and adds afterwards (monet/schedule.py:295-301). */
+int mn_conv_bwd_data_accumulate(const mn_conv2d* g, const void* dy, const void* w, void* dx,
+                                void* ws, size_t ws_bytes, int variant, int dtype,
+                                mn_stream_t stream);
 /* dw = gradient w.r.t. the weights; writes every element of dw.  Replaces
  * cudnn_convolution_backward_weight (conv.cpp:676-688, raw call :550-591). */
 int mn_conv_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, void* dw, void* ws,

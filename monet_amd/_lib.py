@@ -82,6 +82,8 @@ _SIGNATURES = {
     "mn_conv_ws_bytes": (c_int, [POINTER(Conv2d), c_int, c_int, c_int, POINTER(c_size_t)]),
     "mn_conv_fwd": (c_int, [POINTER(Conv2d), _P, _P, _P, _P, _P, c_size_t, c_int, c_int, _P]),
     "mn_conv_bwd_data": (c_int, [POINTER(Conv2d), _P, _P, _P, _P, c_size_t, c_int, c_int, _P]),
+    "mn_conv_bwd_data_accumulate": (c_int, [POINTER(Conv2d), _P, _P, _P, _P, c_size_t, c_int, c_int,
+                                            _P]),
     "mn_conv_bwd_weight": (c_int, [POINTER(Conv2d), _P, _P, _P, _P, c_size_t, c_int, c_int, _P]),
 }
 # entry points whose int return value is NOT a status code

@@ -116,6 +116,7 @@ struct Gather {
   int16_t dh[kMaxTaps], dw[kMaxTaps];
   int32_t aoff[kMaxTaps];
   int ksplit, tiles_per_split;  // split reduction (ksplit > 1): grid.z slices of k-tiles
+  int accum;                    // add to what dst already holds instead of overwriting it
 };
 
 // FAST: the source has a multiple of BK channels.  Then the reduction index
@@ -382,6 +383,10 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
           if (bias && blockIdx.z == 0) r += bias[m];
           if (g.ksplit > 1) {
             atomicAdd(&out[(size_t)m * plane], r);
+            continue;
+          }
+          if (g.accum) {  // every element belongs to exactly one thread of the launch
+            out[(size_t)m * plane] += r;
             continue;
           }
           // a dense output is written once and not read by this kernel: keep it out of the
@@ -795,7 +800,7 @@ static void launch_gather(Gather g, const float* a, const float* src, const floa
 #endif
   if (tile < 0) tile = pick_tile(g.M, g.ncols, fast_path(g), packed);
   plan_split(g, tile, split_ok && packed);
-  if (g.ksplit > 1) {
+  if (g.ksplit > 1 && !g.accum) {
     const size_t n = (size_t)g.N * g.M * g.DH * g.DW;
     fill_zero_kernel<<<(unsigned)((n / 4 + kThreads) / kThreads), kThreads, 0, s>>>(dst, n);
   }
@@ -967,8 +972,8 @@ int mn_conv_fwd(const mn_conv2d* g, const void* x, const void* w, const void* bi
   return mn_launch_status();
 }
 
-int mn_conv_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void* dx, void* ws,
-                     size_t ws_bytes, int variant, int dtype, mn_stream_t stream) {
+static int conv_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void* dx, void* ws,
+                         size_t ws_bytes, int variant, int dtype, mn_stream_t stream, bool accum) {
   using namespace mn_conv;
   const int st = check(g);
   if (st != MN_OK) return st;
@@ -976,7 +981,8 @@ int mn_conv_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void* dx
   if (g->N == 0) return MN_OK;
   if (!dy || !w || !dx) return MN_EINVAL;
   hipStream_t s = mn_stream(stream);
-  if (dtype == MN_BF16) return mn_conv16_bwd_data(g, dy, w, dx, ws, ws_bytes, s);
+  if (dtype == MN_BF16)
+    return accum ? MN_EUNSUPPORTED : mn_conv16_bwd_data(g, dy, w, dx, ws, ws_bytes, s);
   if (dtype != MN_F32) return MN_EUNSUPPORTED;
   const int RS = g->R * g->S;
   const float* a = (const float*)w;
@@ -1004,7 +1010,7 @@ int mn_conv_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void* dx
     for (int sx = 0; sx < g->S; ++sx) any |= (sx * g->dW) % g->sW == cb;
     empty_class |= !any;
   }
-  if (empty_class) {
+  if (empty_class && !accum) {  // (accumulating: those positions simply keep their values)
     const size_t n = (size_t)g->N * g->C * g->H * g->W;
     fill_zero_kernel<<<(unsigned)((n / 4 + kThreads) / kThreads), kThreads, 0, s>>>((float*)dx, n);
   }
@@ -1044,11 +1050,23 @@ int mn_conv_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void* dx
       q.osw = g->sW;
       q.lda = lda;
       q.cha = cha;
+      q.accum = accum ? 1 : 0;
       launch_gather(q, a, (const float*)dy, nullptr, (float*)dx, s, packed,
                     packed && g->sH == 1 && g->sW == 1);
     }
   }
   return mn_launch_status();
+}
+
+int mn_conv_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void* dx, void* ws,
+                     size_t ws_bytes, int variant, int dtype, mn_stream_t stream) {
+  return conv_bwd_data(g, dy, w, dx, ws, ws_bytes, variant, dtype, stream, false);
+}
+
+int mn_conv_bwd_data_accumulate(const mn_conv2d* g, const void* dy, const void* w, void* dx,
+                                void* ws, size_t ws_bytes, int variant, int dtype,
+                                mn_stream_t stream) {
+  return conv_bwd_data(g, dy, w, dx, ws, ws_bytes, variant, dtype, stream, true);
 }
 
 int mn_conv_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, void* dw, void* ws,

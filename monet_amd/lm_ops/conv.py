@@ -118,13 +118,22 @@ def conv_forward(input_, weight, bias, padding, stride, dilation, groups, varian
 
 
 def conv_backward_input(input_shape, grad_output, weight, padding, stride, dilation, groups,
-                        variant):
+                        variant, accumulate_into=None):
+    """Gradient w.r.t. the input.  `accumulate_into`: an fp32 contiguous tensor of the input's
+    shape that already holds a gradient; the result is then ADDED to it by the kernel's
+    epilogue and that tensor is returned (no separate addition pass)."""
     (g, cg), (w, cw) = _prep(grad_output, "grad_output"), _prep(weight, "weight")
     code = _same_dtype(cg, cw)
     geo = conv_geometry(input_shape, w.shape, stride, padding, dilation, groups)
     if tuple(g.shape) != (geo.N, geo.K, geo.P, geo.Q):
         raise RuntimeError("grad_output does not match the convolution geometry")
     ws, nbytes = _workspace(geo, _lib.CONV_BWD_DATA, variant, g.device, code)
+    acc = accumulate_into
+    if acc is not None and code == _lib.F32 and acc.dtype == torch.float32 and acc.is_cuda and \
+            acc.is_contiguous() and list(acc.shape) == [int(d) for d in input_shape]:
+        _lib.call("mn_conv_bwd_data_accumulate", geo, _lib.ptr(g), _lib.ptr(w), _lib.ptr(acc),
+                  _lib.ptr(ws), nbytes, variant, code, _lib.stream_ptr(g.device))
+        return acc
     dx = _empty(input_shape, code, g.device)
     _lib.call("mn_conv_bwd_data", geo, _lib.ptr(g), _lib.ptr(w), _lib.ptr(dx), _lib.ptr(ws), nbytes,
               variant, code, _lib.stream_ptr(g.device))
@@ -191,7 +200,10 @@ class _ConvBase(OP):
                 return _depthwise_forward(input_, weight, bias, stride, padding, dilation, groups)
             return self._fwd_variant(input_, weight, bias, padding, stride, dilation, groups)
 
-    def backward(self, grad_output, stored, nodel=False):
+    # True: `backward(..., accumulate_into=t)` adds the input gradient to `t` inside the kernel
+    accumulates_input_grad = False
+
+    def backward(self, grad_output, stored, nodel=False, accumulate_into=None):
         with torch.no_grad():
             input_, weight = stored
             stride, padding, dilation, groups, input_shape, weight_shape, do_grad = self.params
@@ -212,8 +224,12 @@ class _ConvBase(OP):
                         db = grad_output.sum([0, 2, 3])
                 del input_
                 if kind in (1, 2) and weight is not None and do_grad[0]:
-                    di = self._bwd_ip_variant(input_shape, grad_output, weight, padding, stride,
-                                              dilation, groups)
+                    if accumulate_into is not None and self.accumulates_input_grad:
+                        di = self._bwd_ip_variant(input_shape, grad_output, weight, padding, stride,
+                                                  dilation, groups, accumulate_into)
+                    else:
+                        di = self._bwd_ip_variant(input_shape, grad_output, weight, padding, stride,
+                                                  dilation, groups)
             if do_grad[3]:  # bias present: one gradient per tensor argument of the forward
                 return di, dw, db
             return di, dw
@@ -222,6 +238,7 @@ class _ConvBase(OP):
 @implements(['aten::_convolution'], ['conv_multiway_newnode', 'conv_normal'])
 class SpecificAlgoConvolution(_ConvBase):
     """Runs exactly the variant in `self.algorithm`; falls back to variant 0."""
+    accumulates_input_grad = True
 
     def _fwd_variant(self, input_, weight, bias, padding, stride, dilation, groups):
         try:
@@ -244,14 +261,16 @@ class SpecificAlgoConvolution(_ConvBase):
             self.algorithm = kind * 10 + DEFAULT_VARIANT
             return out
 
-    def _bwd_ip_variant(self, input_shape, grad, weight, padding, stride, dilation, groups):
+    def _bwd_ip_variant(self, input_shape, grad, weight, padding, stride, dilation, groups,
+                        acc=None):
         kind, algo = self.algorithm // 10, self.algorithm % 10
         try:
             return conv_backward_input(input_shape, grad, weight, padding, stride, dilation, groups,
-                                       algo)
+                                       algo, acc)
         except Exception:
+            # (a variant is refused before anything is launched, so nothing was added yet)
             out = conv_backward_input(input_shape, grad, weight, padding, stride, dilation, groups,
-                                      DEFAULT_VARIANT)
+                                      DEFAULT_VARIANT, acc)
             self.algorithm = kind * 10 + DEFAULT_VARIANT
             return out
 

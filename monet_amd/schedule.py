@@ -231,8 +231,13 @@ class Schedule(Graph):
                             "%d %s t=%d" % (i, k_b, n_b.op, t)
                 drop = tuple(sorted(live - stored))
                 last = not (two_step_backward(n_b) and b.bwd_op == "param_grad")
-                plan.append((_BWD, bop, k_b, tuple(spec), drop, last, tuple(n_b.dependencies),
-                             hasattr(bop, 'params'), isinstance(bop, lm_ops.NativeOP)))
+                # an operator that can add its first input's gradient to one that is already
+                # there (convolution backward-data) is handed that tensor instead of a later add
+                deps_b = tuple(n_b.dependencies)
+                acc = bool(getattr(bop, 'accumulates_input_grad', False)) and len(deps_b) > 0 and \
+                    bool(deps_b[0][1])
+                plan.append((_BWD, bop, k_b, tuple(spec), drop, last, deps_b,
+                             hasattr(bop, 'params'), isinstance(bop, lm_ops.NativeOP), acc))
                 have_int.discard(consumed_int)
             else:
                 # the forward pass: the model output stays until forward() has returned it
@@ -278,7 +283,7 @@ class Schedule(Graph):
             elif code == _FREE_INT:
                 ints[ins[1]] = None
             else:
-                _, op, k, spec, drop, last, deps, has_params, native = ins
+                _, op, k, spec, drop, last, deps, has_params, native, acc = ins
                 stored = []
                 for kind, i, _ in spec:
                     if kind == 0:
@@ -298,8 +303,12 @@ class Schedule(Graph):
                     k, self._nodes[k].op)
                 if last:
                     bw[k] = None
-                outs = op.backward(grad, stored)
-                del grad, stored
+                target = bw[deps[0][0]] if acc else None
+                if target is not None:
+                    outs = op.backward(grad, stored, accumulate_into=target)
+                else:
+                    outs = op.backward(grad, stored)
+                del grad, stored, target
                 if not isinstance(outs, (list, tuple)):
                     outs = (outs,)
                 assert len(outs) == len(deps), \
@@ -309,7 +318,7 @@ class Schedule(Graph):
                     if r and o is not None:
                         if bw[i] is None:
                             bw[i] = o
-                        else:
+                        elif o is not bw[i]:  # (else: the operator already added it in place)
                             bw[i] += o
                 del outs
 

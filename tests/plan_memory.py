@@ -53,7 +53,7 @@ def replay(sched, bs):
             elif ins[0] == S._FREE_INT:
                 ints.pop(ins[1], None)
             else:
-                _, op, k, spec, drop, last, deps, *_ = ins
+                _, op, k, spec, drop, last, deps, *_rest2 = ins
                 held = 0
                 for kind, i, optional in spec:
                     if kind == 1:

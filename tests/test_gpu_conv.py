@@ -253,3 +253,20 @@ def test_conv_bf16_channel_counts_that_only_fit_the_shallow_tiles(cuda):
     with pytest.raises(_lib.MonetHipError) as e:
         conv_ops.conv_backward_weight(ws, dev16(dy, cuda), dev16(x, cuda), pad, st, dil, 1, 0)
     assert e.value.status == _lib.MN_EUNSUPPORTED
+
+
+@pytest.mark.parametrize("xs,ws,st,pad,dil", [CASES[8], CASES[10], CASES[11], CASES[1], CASES[9]])
+def test_conv_backward_data_accumulates_into_an_existing_gradient(cuda, xs, ws, st, pad, dil):
+    """dx += conv_backward_data(dy): every variant, dense and strided (parity-class) outputs,
+    positions no tap reaches keep their value, split reductions add onto what is there."""
+    x, w, _ = problem(xs, ws, seed=11)
+    rng = np.random.default_rng(12)
+    dy = rng.standard_normal(O.conv_fwd(x, w, None, st, pad, dil).shape).astype(np.float32)
+    prior = rng.standard_normal(xs).astype(np.float32)
+    exp = prior.astype(np.float64) + O.conv_bwd_data(dy, w, xs, st, pad, dil)
+    for v in range(conv_ops.n_bwd_ip_algos()):
+        acc = dev(prior, cuda)
+        out = conv_ops.conv_backward_input(xs, dev(dy, cuda), dev(w, cuda), pad, st, dil, 1, v,
+                                           accumulate_into=acc)
+        assert out is acc
+        assert_rel(host(acc), exp, 2e-5, f"accumulating backward-data variant {v}")
