@@ -274,7 +274,8 @@ def add_relu_fwd(a, b, alpha=1.0):
 def bn_relu_fwd_train(x, gamma, beta, running_mean, running_var, momentum, eps, dtype=np.float64):
     """BatchNorm (training) followed by ReLU, as one operator: the composition of bn_fwd_train
     and max(., 0).  Returns what bn_fwd_train returns with y replaced by relu(y).  (The
-    reference runs the two operators separately, monet/lm_ops/bn.py:12-54 and relu.py:9-29.)"""
+    reference runs the two operators separately, monet/lm_ops/bn.py:12-54 and relu.py:9-29.)
+    Pinned by: torch.relu(F.batch_norm(training=True)) on CPU in float64."""
     out = list(bn_fwd_train(x, gamma, beta, running_mean, running_var, momentum, eps, dtype))
     out[0] = np.maximum(out[0], 0)
     return tuple(out)
@@ -284,7 +285,8 @@ def bn_relu_bwd_from_x(dy, x, gamma, beta, mean, invstd, positive=None, dtype=np
     """Backward of relu(BN(x)) given the gradient of the ReLU output: mask dy where the
     pre-activation is not positive, then bn_bwd_from_x.  `positive` overrides the mask (a
     caller comparing against another implementation passes that implementation's decisions,
-    so that pre-activations within rounding distance of zero do not count as differences)."""
+    so that pre-activations within rounding distance of zero do not count as differences).
+    Pinned by: float64 autograd through torch.relu(F.batch_norm(...)) for x, gamma and beta."""
     if positive is None:
         shape = [1, -1] + [1] * (x.ndim - 2)
         pre = (x.astype(dtype) - mean.astype(dtype).reshape(shape)) * \
