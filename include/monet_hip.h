@@ -258,6 +258,15 @@ int mn_conv_bwd_data_accumulate(const mn_conv2d* g, const void* dy, const void* 
  * cudnn_convolution_backward_weight (conv.cpp:676-688, raw call :550-591). */
 int mn_conv_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, void* dw, void* ws,
                        size_t ws_bytes, int variant, int dtype, mn_stream_t stream);
+/* The same, and db[k] = sum over (n, p, q) of dy[n,k,p,q] (fp32, K elements)
+ * from the dy tiles the weight-gradient kernel fetches anyway: no separate
+ * pass over dy.  fp32 only (MN_EUNSUPPORTED for MN_BF16).  The reference
+ * computes the bias gradient with a separate reduction, grad.sum([0,2,3])
+ * (monet/lm_ops/conv.py:314).  Variant 1 stays reproducible run to run
+ * (per-split partial sums in the workspace, added in a fixed order). */
+int mn_conv_bwd_weight_bias(const mn_conv2d* g, const void* dy, const void* x, void* dw, void* db,
+                            void* ws, size_t ws_bytes, int variant, int dtype,
+                            mn_stream_t stream);
 
 #ifdef __cplusplus
 }

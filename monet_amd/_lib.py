@@ -85,6 +85,8 @@ _SIGNATURES = {
     "mn_conv_bwd_data_accumulate": (c_int, [POINTER(Conv2d), _P, _P, _P, _P, c_size_t, c_int, c_int,
                                             _P]),
     "mn_conv_bwd_weight": (c_int, [POINTER(Conv2d), _P, _P, _P, _P, c_size_t, c_int, c_int, _P]),
+    "mn_conv_bwd_weight_bias": (c_int, [POINTER(Conv2d), _P, _P, _P, _P, _P, c_size_t, c_int, c_int,
+                                        _P]),
 }
 # entry points whose int return value is NOT a status code
 _UNCHECKED = {"mn_abi_version", "mn_conv_n_variants"}

@@ -415,11 +415,37 @@ struct WGrad {
   int mode;             // 0: store, 1: atomicAdd into dw, 2: store partial [z][K][ncols]
 };
 
-template <class TL>
+// Row sums of the dy tiles one workgroup has staged: LANES consecutive lanes (one per depth
+// position) hold the partial sums of the same rows; they are added in a fixed order and lane 0
+// of each group hands the result over the same way the tile itself is written (store, atomic
+// add, or one partial per split).
+template <int LANES, int ROWS>
+__device__ __forceinline__ void store_row_sums(float (&row_sum)[ROWS], float* __restrict__ db,
+                                               const WGrad& g, int first_row, int row_step,
+                                               int depth_lane) {
+#pragma unroll
+  for (int i = 0; i < ROWS; ++i) {
+    float v = row_sum[i];
+#pragma unroll
+    for (int off = LANES / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    const int m = first_row + row_step * i;
+    if (depth_lane == 0 && m < g.K) {
+      if (g.mode == 1)
+        atomicAdd(db + m, v);
+      else
+        db[(g.mode == 2 ? (size_t)blockIdx.z * g.K : 0) + m] = v;
+    }
+  }
+}
+
+// DB: the workgroups of the first column tile also reduce the rows of their dy tile (the values
+// they fetch anyway) into the bias gradient db[k] = sum over (n, p, q) of dy[n,k,p,q].
+template <class TL, bool DB = false>
 __global__ __launch_bounds__(kThreads) void wgrad_kernel(const WGrad g,
                                                          const float* __restrict__ dy,
                                                          const float* __restrict__ x,
-                                                         float* __restrict__ out) {
+                                                         float* __restrict__ out,
+                                                         float* __restrict__ db) {
   constexpr int BM = TL::BM, BN = TL::BN;
   __shared__ float lds_a[2][WBK][BM + kPad];
   __shared__ float lds_b[2][WBK][BN + kPad];
@@ -467,6 +493,8 @@ __global__ __launch_bounds__(kThreads) void wgrad_kernel(const WGrad g,
   const char* dyp = reinterpret_cast<const char*>(dy);
   const char* xp = reinterpret_cast<const char*>(x);
   float ra[kRowsA], rb[kRowsB];
+  float row_sum[DB ? kRowsA : 1] = {};
+  const bool sums_rows = DB && blockIdx.x == 0;
   uint32_t a_mask = 0, b_mask = 0;
   auto fetch = [&](uint32_t d0) {
     const uint32_t d = d0 + kdl;
@@ -497,8 +525,13 @@ __global__ __launch_bounds__(kThreads) void wgrad_kernel(const WGrad g,
   };
   auto stage = [&](int buf) {
 #pragma unroll
-    for (int i = 0; i < kRowsA; ++i)
-      lds_a[buf][kdl][row0 + kStep * i] = ((a_mask >> i) & 1u) ? ra[i] : 0.f;
+    for (int i = 0; i < kRowsA; ++i) {
+      const float v = ((a_mask >> i) & 1u) ? ra[i] : 0.f;
+      lds_a[buf][kdl][row0 + kStep * i] = v;
+      if constexpr (DB) {
+        if (sums_rows) row_sum[i] += v;
+      }
+    }
 #pragma unroll
     for (int i = 0; i < kRowsB; ++i)
       lds_b[buf][kdl][row0 + kStep * i] = ((b_mask >> i) & 1u) ? rb[i] : 0.f;
@@ -526,6 +559,9 @@ __global__ __launch_bounds__(kThreads) void wgrad_kernel(const WGrad g,
       if (kt + 1 < t_end) stage(buf ^ 1);
       __syncthreads();
     }
+  }
+  if constexpr (DB) {
+    if (sums_rows) store_row_sums<WBK, kRowsA>(row_sum, db, g, m0 + row0, kStep, kdl);
   }
 
   float* base = out;
@@ -559,11 +595,12 @@ __global__ __launch_bounds__(kThreads) void wgrad_kernel(const WGrad g,
 // progressions instead of per-row tables, and no row needs a bounds mask: fewer
 // vector registers (more resident waves) and far less address arithmetic between
 // the matrix instructions.
-template <class TL, int DEPTH>
+template <class TL, int DEPTH, bool DB = false>
 __global__ __launch_bounds__(kThreads) void wgrad_tap_kernel(const WGrad g,
                                                              const float* __restrict__ dy,
                                                              const float* __restrict__ x,
-                                                             float* __restrict__ out) {
+                                                             float* __restrict__ out,
+                                                             float* __restrict__ db) {
   constexpr int BM = TL::BM, BN = TL::BN;
   __shared__ float lds_a[2][DEPTH][BM + kPad];
   __shared__ float lds_b[2][DEPTH][BN + kPad];
@@ -586,6 +623,8 @@ __global__ __launch_bounds__(kThreads) void wgrad_tap_kernel(const WGrad g,
   const char* dyp = reinterpret_cast<const char*>(dy);
   const char* xp = reinterpret_cast<const char*>(x);
   float ra[kRowsA], rb[kRowsB];
+  float row_sum[DB ? kRowsA : 1] = {};
+  const bool sums_rows = DB && blockIdx.x == 0;
   bool a_ok = false, b_ok = false;
   auto fetch = [&](uint32_t d0) {
     const uint32_t d = d0 + kdl;
@@ -609,7 +648,13 @@ __global__ __launch_bounds__(kThreads) void wgrad_tap_kernel(const WGrad g,
   };
   auto stage = [&](int buf) {
 #pragma unroll
-    for (int i = 0; i < kRowsA; ++i) lds_a[buf][kdl][row0 + kStep * i] = a_ok ? ra[i] : 0.f;
+    for (int i = 0; i < kRowsA; ++i) {
+      const float v = a_ok ? ra[i] : 0.f;
+      lds_a[buf][kdl][row0 + kStep * i] = v;
+      if constexpr (DB) {
+        if (sums_rows) row_sum[i] += v;
+      }
+    }
 #pragma unroll
     for (int i = 0; i < kRowsB; ++i) lds_b[buf][kdl][row0 + kStep * i] = b_ok ? rb[i] : 0.f;
   };
@@ -636,6 +681,9 @@ __global__ __launch_bounds__(kThreads) void wgrad_tap_kernel(const WGrad g,
       if (kt + 1 < t_end) stage(buf ^ 1);
       __syncthreads();
     }
+  }
+  if constexpr (DB) {
+    if (sums_rows) store_row_sums<DEPTH, kRowsA>(row_sum, db, g, m0 + row0, kStep, kdl);
   }
 
   float* base = out;
@@ -914,7 +962,8 @@ int mn_conv_ws_bytes(const mn_conv2d* g, int direction, int variant, int dtype, 
   if (direction == MN_CONV_BWD_WEIGHT && variant == 1) {
     int splits, tiles;
     wgrad_split(g, 1, &splits, &tiles);
-    *bytes = splits > 1 ? wsize * splits : 0;
+    // one partial weight gradient and one partial bias gradient (K floats) per split
+    *bytes = splits > 1 ? (wsize + (size_t)g->K * sizeof(float)) * splits : 0;
   }
   return MN_OK;
 }
@@ -1069,8 +1118,9 @@ int mn_conv_bwd_data_accumulate(const mn_conv2d* g, const void* dy, const void* 
   return conv_bwd_data(g, dy, w, dx, ws, ws_bytes, variant, dtype, stream, true);
 }
 
-int mn_conv_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, void* dw, void* ws,
-                       size_t ws_bytes, int variant, int dtype, mn_stream_t stream) {
+// db_out: where the bias gradient goes (fp32, K elements), or null for the weight gradient alone.
+static int conv_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, void* dw, void* db_out,
+                           void* ws, size_t ws_bytes, int variant, int dtype, mn_stream_t stream) {
   using namespace mn_conv;
   const int st = check(g);
   if (st != MN_OK) return st;
@@ -1079,13 +1129,18 @@ int mn_conv_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, void* 
   if (!dw) return MN_EINVAL;
   hipStream_t s = mn_stream(stream);
   if (dtype == MN_BF16) {
+    if (db_out) return MN_EUNSUPPORTED;     // the bf16 kernel has no bias-gradient epilogue
     if (g->N == 0) return MN_EUNSUPPORTED;  // nothing to reduce: the caller clears dw itself
     if (!dy || !x) return MN_EINVAL;
     return mn_conv16_bwd_weight(g, dy, x, dw, ws, ws_bytes, s);
   }
+  if (db_out && !mn_aligned(db_out, 4)) return MN_EINVAL;
   const size_t nw = (size_t)g->K * g->C * g->R * g->S;
+  const size_t nb = (size_t)g->K;
+  float* db = (float*)db_out;
   if (g->N == 0) {
     fill_zero_kernel<<<(unsigned)((nw / 4 + kThreads) / kThreads), kThreads, 0, s>>>((float*)dw, nw);
+    if (db) fill_zero_kernel<<<(unsigned)((nb / 4 + kThreads) / kThreads), kThreads, 0, s>>>(db, nb);
     return mn_launch_status();
   }
   if (!dy || !x) return MN_EINVAL;
@@ -1113,15 +1168,19 @@ int mn_conv_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, void* 
   wgrad_split(g, variant, &splits, &tps);
   q.tiles_per_split = tps;
   float* out = (float*)dw;
+  float* db_dst = db;  // where the kernel leaves its row sums
   if (splits == 1) {
     q.mode = 0;
   } else if (variant == 0) {
     q.mode = 1;
     fill_zero_kernel<<<(unsigned)((nw / 4 + kThreads) / kThreads), kThreads, 0, s>>>((float*)dw, nw);
+    if (db) fill_zero_kernel<<<(unsigned)((nb / 4 + kThreads) / kThreads), kThreads, 0, s>>>(db, nb);
   } else {
     q.mode = 2;
-    if (!ws || ws_bytes < nw * sizeof(float) * splits || !mn_aligned(ws, 4)) return MN_EINVAL;
+    // partial weight gradients, then (always reserved) one partial bias gradient per split
+    if (!ws || ws_bytes < (nw + nb) * sizeof(float) * splits || !mn_aligned(ws, 4)) return MN_EINVAL;
     out = (float*)ws;
+    if (db) db_dst = (float*)ws + nw * splits;
   }
   const int tile = wgrad_tile(g, variant);
   int bm, bn;
@@ -1133,11 +1192,19 @@ int mn_conv_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, void* 
 #ifdef MN_TUNING
     if (const char* e = getenv("MN_WGRAD_DEPTH")) deep = atoi(e);
 #endif
-#define MN_TAP(TL)                                                                               \
-  if (deep == 16)                                                                                \
-    wgrad_tap_kernel<TL, 16><<<grid, kThreads, 0, s>>>(q, (const float*)dy, (const float*)x, out); \
-  else                                                                                           \
-    wgrad_tap_kernel<TL, 32><<<grid, kThreads, 0, s>>>(q, (const float*)dy, (const float*)x, out)
+#define MN_TAP_D(TL, D)                                                                           \
+  if (db)                                                                                         \
+    wgrad_tap_kernel<TL, D, true><<<grid, kThreads, 0, s>>>(q, (const float*)dy, (const float*)x, \
+                                                            out, db_dst);                         \
+  else                                                                                            \
+    wgrad_tap_kernel<TL, D><<<grid, kThreads, 0, s>>>(q, (const float*)dy, (const float*)x, out,  \
+                                                      nullptr)
+#define MN_TAP(TL)       \
+  if (deep == 16) {      \
+    MN_TAP_D(TL, 16);    \
+  } else {               \
+    MN_TAP_D(TL, 32);    \
+  }
     switch (tile) {
       case 2: MN_TAP(T64x128); break;
       case 3: MN_TAP(T128x64); break;
@@ -1145,19 +1212,43 @@ int mn_conv_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, void* 
       default: MN_TAP(T128x128); break;
     }
 #undef MN_TAP
+#undef MN_TAP_D
   } else {
-  dim3 grid((q.ncols + bn - 1) / bn, (g->K + bm - 1) / bm, splits);
-  switch (tile) {
-    case 2: wgrad_kernel<T64x128><<<grid, kThreads, 0, s>>>(q, (const float*)dy, (const float*)x, out); break;
-    case 3: wgrad_kernel<T128x64><<<grid, kThreads, 0, s>>>(q, (const float*)dy, (const float*)x, out); break;
-    case 4: wgrad_kernel<T64x64><<<grid, kThreads, 0, s>>>(q, (const float*)dy, (const float*)x, out); break;
-    default: wgrad_kernel<T128x128><<<grid, kThreads, 0, s>>>(q, (const float*)dy, (const float*)x, out); break;
+    dim3 grid((q.ncols + bn - 1) / bn, (g->K + bm - 1) / bm, splits);
+#define MN_GEN(TL)                                                                              \
+  if (db)                                                                                       \
+    wgrad_kernel<TL, true><<<grid, kThreads, 0, s>>>(q, (const float*)dy, (const float*)x, out, \
+                                                     db_dst);                                   \
+  else                                                                                          \
+    wgrad_kernel<TL><<<grid, kThreads, 0, s>>>(q, (const float*)dy, (const float*)x, out, nullptr)
+    switch (tile) {
+      case 2: MN_GEN(T64x128); break;
+      case 3: MN_GEN(T128x64); break;
+      case 4: MN_GEN(T64x64); break;
+      default: MN_GEN(T128x128); break;
+    }
+#undef MN_GEN
   }
-  }
-  if (q.mode == 2)
+  if (q.mode == 2) {
     wgrad_reduce_kernel<<<(unsigned)((nw + kThreads - 1) / kThreads), kThreads, 0, s>>>(
         (const float*)ws, (float*)dw, nw, splits);
+    if (db)
+      wgrad_reduce_kernel<<<(unsigned)((nb + kThreads - 1) / kThreads), kThreads, 0, s>>>(
+          db_dst, db, nb, splits);
+  }
   return mn_launch_status();
+}
+
+int mn_conv_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, void* dw, void* ws,
+                       size_t ws_bytes, int variant, int dtype, mn_stream_t stream) {
+  return conv_bwd_weight(g, dy, x, dw, nullptr, ws, ws_bytes, variant, dtype, stream);
+}
+
+int mn_conv_bwd_weight_bias(const mn_conv2d* g, const void* dy, const void* x, void* dw, void* db,
+                            void* ws, size_t ws_bytes, int variant, int dtype,
+                            mn_stream_t stream) {
+  if (!db) return MN_EINVAL;
+  return conv_bwd_weight(g, dy, x, dw, db, ws, ws_bytes, variant, dtype, stream);
 }
 
 }  // extern "C"

@@ -141,7 +141,10 @@ def conv_backward_input(input_shape, grad_output, weight, padding, stride, dilat
 
 
 def conv_backward_weight(weight_shape, grad_output, input_, padding, stride, dilation, groups,
-                         variant):
+                         variant, with_bias_grad=False):
+    """Gradient w.r.t. the weights.  `with_bias_grad`: return (dw, db) with the bias gradient
+    db = grad_output.sum([0, 2, 3]) (conv.py:314) reduced by the same kernel from the tiles of
+    grad_output it fetches anyway (fp32); for bf16 tensors db is a separate reduction."""
     (g, cg), (x, cx) = _prep(grad_output, "grad_output"), _prep(input_, "input")
     code = _same_dtype(cg, cx)
     geo = conv_geometry(x.shape, weight_shape, stride, padding, dilation, groups)
@@ -149,8 +152,15 @@ def conv_backward_weight(weight_shape, grad_output, input_, padding, stride, dil
         raise RuntimeError("grad_output does not match the convolution geometry")
     ws, nbytes = _workspace(geo, _lib.CONV_BWD_WEIGHT, variant, g.device, code)
     dw = _empty(weight_shape, code, g.device)
+    if with_bias_grad and code == _lib.F32:
+        db = torch.empty(geo.K, dtype=torch.float32, device=g.device)
+        _lib.call("mn_conv_bwd_weight_bias", geo, _lib.ptr(g), _lib.ptr(x), _lib.ptr(dw),
+                  _lib.ptr(db), _lib.ptr(ws), nbytes, variant, code, _lib.stream_ptr(g.device))
+        return dw, db
     _lib.call("mn_conv_bwd_weight", geo, _lib.ptr(g), _lib.ptr(x), _lib.ptr(dw), _lib.ptr(ws),
               nbytes, variant, code, _lib.stream_ptr(g.device))
+    if with_bias_grad:
+        return dw, grad_output.sum([0, 2, 3])
     return dw
 
 
@@ -217,10 +227,13 @@ class _ConvBase(OP):
                                              groups, do_grad[:2])
             else:
                 if kind in (0, 2) and input_ is not None:
-                    if do_grad[1]:
+                    if do_grad[1] and do_grad[2]:
+                        dw, db = self._bwd_wt_variant(weight_shape, grad_output, input_, padding,
+                                                      stride, dilation, groups, True)
+                    elif do_grad[1]:
                         dw = self._bwd_wt_variant(weight_shape, grad_output, input_, padding, stride,
                                                   dilation, groups)
-                    if do_grad[2]:
+                    elif do_grad[2]:
                         db = grad_output.sum([0, 2, 3])
                 del input_
                 if kind in (1, 2) and weight is not None and do_grad[0]:
@@ -250,14 +263,15 @@ class SpecificAlgoConvolution(_ConvBase):
             self.algorithm = DEFAULT_VARIANT
             return out
 
-    def _bwd_wt_variant(self, weight_shape, grad, input_, padding, stride, dilation, groups):
+    def _bwd_wt_variant(self, weight_shape, grad, input_, padding, stride, dilation, groups,
+                        with_bias_grad=False):
         kind, algo = self.algorithm // 10, self.algorithm % 10
         try:
             return conv_backward_weight(weight_shape, grad, input_, padding, stride, dilation,
-                                        groups, algo)
+                                        groups, algo, with_bias_grad)
         except Exception:
             out = conv_backward_weight(weight_shape, grad, input_, padding, stride, dilation,
-                                       groups, DEFAULT_VARIANT)
+                                       groups, DEFAULT_VARIANT, with_bias_grad)
             self.algorithm = kind * 10 + DEFAULT_VARIANT
             return out
 
@@ -322,17 +336,18 @@ class GreedyAlgoConvolution(_ConvBase):
             return conv_forward(input_, weight, bias, padding, stride, dilation, groups,
                                 DEFAULT_VARIANT)
 
-    def _bwd_wt_variant(self, weight_shape, grad, input_, padding, stride, dilation, groups):
+    def _bwd_wt_variant(self, weight_shape, grad, input_, padding, stride, dilation, groups,
+                        with_bias_grad=False):
         if self.bwd_wt_algo == -1:
             self.bwd_wt_algo = _autotune(n_bwd_wt_algos(), lambda alg: conv_backward_weight(
                 weight_shape, grad, input_, padding, stride, dilation, groups, alg))
         try:
             return conv_backward_weight(weight_shape, grad, input_, padding, stride, dilation,
-                                        groups, self.bwd_wt_algo)
+                                        groups, self.bwd_wt_algo, with_bias_grad)
         except Exception:
             self.bwd_wt_algo = DEFAULT_VARIANT
             return conv_backward_weight(weight_shape, grad, input_, padding, stride, dilation,
-                                        groups, DEFAULT_VARIANT)
+                                        groups, DEFAULT_VARIANT, with_bias_grad)
 
     def _bwd_ip_variant(self, input_shape, grad, weight, padding, stride, dilation, groups):
         if self.bwd_ip_algo == -1:

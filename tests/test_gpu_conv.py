@@ -270,3 +270,52 @@ def test_conv_backward_data_accumulates_into_an_existing_gradient(cuda, xs, ws, 
                                            accumulate_into=acc)
         assert out is acc
         assert_rel(host(acc), exp, 2e-5, f"accumulating backward-data variant {v}")
+
+
+BIAS_GRAD_CASES = CASES + [
+    ((1, 4, 5, 5), (6, 4, 3, 3), 1, 1, 1),             # one depth tile: a single plain store
+    ((1, 64, 4, 4), (64, 64, 3, 3), 1, 1, 1),          # the same through the tap-major kernel
+    ((1, 1024, 4, 4), (1024, 1024, 3, 3), 1, 1, 1),    # more output tiles than resident slots: no split
+    ((2, 64, 40, 40), (64, 64, 3, 3), 1, 1, 1),        # UNet-like: bias, 64 channels, long reduction
+]
+
+
+@pytest.mark.parametrize("xs,ws,st,pad,dil", BIAS_GRAD_CASES)
+def test_conv_backward_weight_with_bias_gradient(cuda, xs, ws, st, pad, dil):
+    """db = sum of dy over (n, p, q), from the weight-gradient kernel itself: against the
+    float64 sum, every variant; dw unchanged by the extra epilogue; variant 1 reproducible."""
+    x, w, _ = problem(xs, ws, 21)
+    yshape = O.conv_fwd(x, w, None, st, pad, dil).shape
+    dy = np.random.default_rng(22).standard_normal(yshape).astype(np.float32)
+    exp_dw = O.conv_bwd_weight(dy, x, ws, st, pad, dil)
+    exp_db = dy.astype(np.float64).sum(axis=(0, 2, 3))
+    # a sum of M unit-variance terms: tolerance relative to its typical size sqrt(M), not to
+    # the largest of K sums
+    scale_db = np.sqrt(dy.size / ws[0])
+    for v in range(conv_ops.n_bwd_wt_algos()):
+        alone = conv_ops.conv_backward_weight(ws, dev(dy, cuda), dev(x, cuda), pad, st, dil, 1, v)
+        dw, db = conv_ops.conv_backward_weight(ws, dev(dy, cuda), dev(x, cuda), pad, st, dil, 1, v,
+                                               with_bias_grad=True)
+        assert_rel(host(dw), exp_dw, TOL, f"dw with bias gradient, variant {v}")
+        assert list(db.shape) == [ws[0]]
+        err = np.abs(host(db).astype(np.float64) - exp_db).max()
+        assert err <= TOL * scale_db, f"db variant {v}: {err:.3e} vs {scale_db:.3e}"
+        if v == 1:
+            assert torch.equal(dw, alone)
+            dw2, db2 = conv_ops.conv_backward_weight(ws, dev(dy, cuda), dev(x, cuda), pad, st, dil,
+                                                     1, v, with_bias_grad=True)
+            assert torch.equal(db, db2) and torch.equal(dw, dw2)
+
+
+def test_conv_bias_gradient_entry_point_rejects_bf16_and_null(cuda):
+    from monet_amd import _lib
+    geo = conv_ops.conv_geometry((2, 64, 8, 8), (64, 64, 3, 3), 1, 1, 1, 1)
+    buf = torch.zeros(64 * 64 * 9, device=cuda)
+    with pytest.raises(_lib.MonetHipError) as e:
+        _lib.call("mn_conv_bwd_weight_bias", geo, _lib.ptr(buf), _lib.ptr(buf), _lib.ptr(buf),
+                  _lib.ptr(buf), None, 0, 0, _lib.BF16, _lib.stream_ptr(buf.device))
+    assert e.value.status == _lib.MN_EUNSUPPORTED
+    with pytest.raises(_lib.MonetHipError) as e:
+        _lib.call("mn_conv_bwd_weight_bias", geo, _lib.ptr(buf), _lib.ptr(buf), _lib.ptr(buf),
+                  None, None, 0, 0, _lib.F32, _lib.stream_ptr(buf.device))
+    assert e.value.status == _lib.MN_EINVAL
