@@ -228,36 +228,43 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
   float ra[kARows], rb[kBRows];
   uint32_t b_ok = 0;  // bit i: rb[i] holds a window element (else it is staged as zero)
   bool a_ok = true;
-  // Only issues loads: masking happens in stage(), after the multiply of the current
-  // tile, so the loads stay in flight behind the matrix instructions.
-  auto fetch_fast = [&](int t, int c0) {  // t, c0 uniform
+  // FAST: what only changes when the reduction enters a new tap.  tap_b: this thread's byte
+  // offset of (pixel shifted by the tap, channel brow0) or, outside the window, of an
+  // in-bounds dummy whose value is staged as zero; tap_in: inside the window; tap_a: byte
+  // offset of the tap's block of A (uniform).
+  uint32_t tap_b = 0, tap_a = 0;
+  bool tap_in = false;
+  bool b_in = false;  // tap_in at the time of the last fetch: what stage() masks with
+  auto enter_tap = [&](int t) {  // t uniform
     const int dh = tdh[t], dw = tdw[t];
     const int hh = ohs + dh, ww = ows + dw;
-    const bool ok = col_ok && (unsigned)hh < (unsigned)g.Hs && (unsigned)ww < (unsigned)g.Ws;
-    b_ok = ok ? 0xFFFFFFFFu : 0u;
+    tap_in = col_ok && (unsigned)hh < (unsigned)g.Hs && (unsigned)ww < (unsigned)g.Ws;
+    tap_b = tap_in ? pix_b + (uint32_t)((dh * g.Ws + dw) * 4) : brow0 * plane_b;
+    tap_a = PACKED ? (uint32_t)((long long)taoff[t] * g.Cs * g.lda * 4) : (uint32_t)(taoff[t] * 4);
+  };
+  // Only issues loads: masking happens in stage(), after the multiply of the current
+  // tile, so the loads stay in flight behind the matrix instructions.  The per-tile part of
+  // every address is uniform (c0), so it goes into the base pointer and the per-thread
+  // offsets stay put for a whole tap.
+  auto fetch_fast = [&](int c0) {  // c0 uniform
+    b_in = tap_in;
+    const char* spc = sp + (size_t)c0 * plane_b;
     if (POINT) {
 #pragma unroll
-      for (int i = 0; i < kB4; ++i)
-        rb4[i] = *reinterpret_cast<const float4_t*>(sp + (bp_b[i] + (uint32_t)c0 * plane_b));
+      for (int i = 0; i < kB4; ++i) rb4[i] = *reinterpret_cast<const float4_t*>(spc + bp_b[i]);
     } else {
-      const uint32_t sb = (uint32_t)((((long long)c0 * g.Hs + dh) * g.Ws + dw) * 4);
-      const uint32_t base = ok ? pix_b + sb : brow0 * plane_b;
 #pragma unroll
       for (int i = 0; i < kBRows; ++i)
-        rb[i] = *reinterpret_cast<const float*>(sp + (base + kBStep * i * plane_b));
+        rb[i] = *reinterpret_cast<const float*>(spc + (tap_b + kBStep * i * plane_b));
     }
     if (PACKED) {
-      const uint32_t sa = (uint32_t)(((long long)taoff[t] * g.Cs + c0) * g.lda * 4);
+      const char* apc = ap + ((size_t)tap_a + (size_t)c0 * g.lda * 4);
 #pragma unroll
-      for (int i = 0; i < kA4; ++i)
-        ra4[i] = *reinterpret_cast<const float4_t*>(ap + (ap_b[i] + sa));
+      for (int i = 0; i < kA4; ++i) ra4[i] = *reinterpret_cast<const float4_t*>(apc + ap_b[i]);
     } else {
-      const uint32_t sa = (uint32_t)(((long long)c0 * g.cha + taoff[t]) * 4);
+      const char* apc = ap + ((size_t)tap_a + (size_t)c0 * g.cha * 4);
 #pragma unroll
-      for (int i = 0; i < kARows; ++i) {
-        const bool mok = (am_ok >> i) & 1u;
-        ra[i] = *reinterpret_cast<const float*>(ap + (am_b[i] + (mok ? sa : 0u)));
-      }
+      for (int i = 0; i < kARows; ++i) ra[i] = *reinterpret_cast<const float*>(apc + am_b[i]);
     }
   };
   auto fetch_any = [&](int k0) {
@@ -301,8 +308,10 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
       }
     } else {
 #pragma unroll
-      for (int i = 0; i < kBRows; ++i)
-        lds_b[buf][brow0 + kBStep * i][bcol] = ((b_ok >> i) & 1u) ? rb[i] : 0.f;
+      for (int i = 0; i < kBRows; ++i) {
+        const bool in = FAST ? b_in : (((b_ok >> i) & 1u) != 0);
+        lds_b[buf][brow0 + kBStep * i][bcol] = in ? rb[i] : 0.f;
+      }
     }
     if (PACKED) {
 #pragma unroll
@@ -337,13 +346,15 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
       t = kt_begin / per_tap;
       c0 = (kt_begin - t * per_tap) * BK;
     }
+    if (FAST) enter_tap(t);
     auto fetch_next = [&](int kt) {
       if (FAST) {
-        fetch_fast(t, c0);
+        fetch_fast(c0);
         c0 += BK;
         if (c0 == g.Cs) {
           c0 = 0;
           ++t;
+          if (t < g.T) enter_tap(t);
         }
       } else {
         fetch_any(kt * BK);
@@ -403,6 +414,29 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
 }
 
 // ------------------------------------------------------- backward weight --
+// A thread's position d = n*PQ + pq in the (n, p, q) reduction, moved STEP at a time: the
+// image index and the in-image offset are kept up to date by addition instead of two
+// divisions per tile.
+template <int STEP>
+struct DepthPos {
+  uint32_t d, n, pq;
+  __device__ __forceinline__ DepthPos(uint32_t d0, uint32_t PQ) : d(d0), n(d0 / PQ) {
+    pq = d0 - n * PQ;
+  }
+  __device__ __forceinline__ void advance(uint32_t PQ) {
+    d += STEP;
+    pq += STEP;
+    if (PQ < STEP) {  // uniform: images smaller than a step (may cross several per step)
+      const uint32_t k = pq / PQ;
+      n += k;
+      pq -= k * PQ;
+    } else if (pq >= PQ) {
+      pq -= PQ;
+      ++n;
+    }
+  }
+};
+
 // dw[k][c][r][s] = sum over (n, p, q) dy[n,k,p,q] * x[n,c,p*sH + r*dH - pH, q*sW + s*dW - pW]
 // GEMM: rows = k (M = K), columns = (c, r, s) (ncols = C*R*S), depth = (n, p, q).
 struct WGrad {
@@ -410,7 +444,8 @@ struct WGrad {
   int sH, sW, pH, pW, dH, dW;
   uint32_t depth;       // N*P*Q
   uint32_t ncols;       // C*R*S
-  FastDiv divRS, divS;
+  FastDiv divRS, divS, divQ;
+  int exact_div;             // P*Q or Q beyond FastDiv's range: divide the slow way
   uint32_t tiles_per_split;  // k-tiles handled by one blockIdx.z
   int mode;             // 0: store, 1: atomicAdd into dw, 2: store partial [z][K][ncols]
 };
@@ -496,17 +531,18 @@ __global__ __launch_bounds__(kThreads) void wgrad_kernel(const WGrad g,
   float row_sum[DB ? kRowsA : 1] = {};
   const bool sums_rows = DB && blockIdx.x == 0;
   uint32_t a_mask = 0, b_mask = 0;
-  auto fetch = [&](uint32_t d0) {
-    const uint32_t d = d0 + kdl;
-    const bool d_ok = d < g.depth;
-    uint32_t n = 0, p = 0, q = 0;
-    if (d_ok) {
-      n = d / PQ;
-      const uint32_t pq = d - n * PQ;
-      p = pq / g.Q;
-      q = pq - p * g.Q;
-    }
-    const uint32_t abase = ((n * (uint32_t)g.K) * PQ + p * g.Q + q) * 4u;
+  const uint32_t total_tiles = (g.depth + WBK - 1) / WBK;
+  const uint32_t t_begin = blockIdx.z * g.tiles_per_split;
+  const uint32_t t_end = min(t_begin + g.tiles_per_split, total_tiles);
+  DepthPos<WBK> pos(t_begin * WBK + kdl, PQ);
+  // fetches the tile at the current depth position and moves on to the next one
+  auto fetch = [&]() {
+    const bool d_ok = pos.d < g.depth;
+    const uint32_t n = d_ok ? pos.n : 0u, pq = d_ok ? pos.pq : 0u;
+    const uint32_t p = g.exact_div ? pq / (uint32_t)g.Q : g.divQ.div(pq);
+    const uint32_t q = pq - p * g.Q;
+    pos.advance(PQ);
+    const uint32_t abase = ((n * (uint32_t)g.K) * PQ + pq) * 4u;
     a_mask = d_ok ? am_ok : 0u;
 #pragma unroll
     for (int i = 0; i < kRowsA; ++i)
@@ -545,16 +581,13 @@ __global__ __launch_bounds__(kThreads) void wgrad_kernel(const WGrad g,
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-  const uint32_t total_tiles = (g.depth + WBK - 1) / WBK;
-  const uint32_t t_begin = blockIdx.z * g.tiles_per_split;
-  const uint32_t t_end = min(t_begin + g.tiles_per_split, total_tiles);
   if (t_begin < t_end) {
-    fetch(t_begin * WBK);
+    fetch();
     stage(0);
     __syncthreads();
     for (uint32_t kt = t_begin; kt < t_end; ++kt) {
       const int buf = (kt - t_begin) & 1;
-      if (kt + 1 < t_end) fetch((kt + 1) * WBK);
+      if (kt + 1 < t_end) fetch();
       mma_tile<TL, WBK>(lds_a[buf], lds_b[buf], wm, wn, lane, acc);
       if (kt + 1 < t_end) stage(buf ^ 1);
       __syncthreads();
@@ -626,13 +659,17 @@ __global__ __launch_bounds__(kThreads) void wgrad_tap_kernel(const WGrad g,
   float row_sum[DB ? kRowsA : 1] = {};
   const bool sums_rows = DB && blockIdx.x == 0;
   bool a_ok = false, b_ok = false;
-  auto fetch = [&](uint32_t d0) {
-    const uint32_t d = d0 + kdl;
-    a_ok = d < g.depth;
-    const uint32_t dd = a_ok ? d : 0u;
-    const uint32_t n = dd / PQ;
-    const uint32_t pq = dd - n * PQ;
-    const uint32_t p = pq / g.Q, q = pq - p * g.Q;
+  const uint32_t total_tiles = (g.depth + DEPTH - 1) / DEPTH;
+  const uint32_t t_begin = blockIdx.z * (g.tiles_per_split * (WBK / DEPTH));
+  const uint32_t t_end = min(t_begin + g.tiles_per_split * (WBK / DEPTH), total_tiles);
+  DepthPos<DEPTH> pos(t_begin * DEPTH + kdl, PQ);
+  // fetches the tile at the current depth position and moves on to the next one
+  auto fetch = [&]() {
+    a_ok = pos.d < g.depth;
+    const uint32_t n = a_ok ? pos.n : 0u, pq = a_ok ? pos.pq : 0u;
+    const uint32_t p = g.exact_div ? pq / (uint32_t)g.Q : g.divQ.div(pq);
+    const uint32_t q = pq - p * g.Q;
+    pos.advance(PQ);
     const uint32_t abase = ((n * (uint32_t)g.K) * PQ + pq) * 4u + a_row0;
 #pragma unroll
     for (int i = 0; i < kRowsA; ++i)
@@ -667,16 +704,13 @@ __global__ __launch_bounds__(kThreads) void wgrad_tap_kernel(const WGrad g,
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-  const uint32_t total_tiles = (g.depth + DEPTH - 1) / DEPTH;
-  const uint32_t t_begin = blockIdx.z * (g.tiles_per_split * (WBK / DEPTH));
-  const uint32_t t_end = min(t_begin + g.tiles_per_split * (WBK / DEPTH), total_tiles);
   if (t_begin < t_end) {
-    fetch(t_begin * DEPTH);
+    fetch();
     stage(0);
     __syncthreads();
     for (uint32_t kt = t_begin; kt < t_end; ++kt) {
       const int buf = (kt - t_begin) & 1;
-      if (kt + 1 < t_end) fetch((kt + 1) * DEPTH);
+      if (kt + 1 < t_end) fetch();
       mma_tile<TL, DEPTH>(lds_a[buf], lds_b[buf], wm, wn, lane, acc);
       if (kt + 1 < t_end) stage(buf ^ 1);
       __syncthreads();
@@ -1164,6 +1198,8 @@ static int conv_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, vo
   q.ncols = (uint32_t)(g->C * g->R * g->S);
   q.divRS = make_fastdiv(g->R * g->S);
   q.divS = make_fastdiv(g->S);
+  q.divQ = make_fastdiv(g->Q);
+  q.exact_div = ((long long)g->P * g->Q > (1ll << 20) || g->Q >= 4096) ? 1 : 0;
   int splits, tps;
   wgrad_split(g, variant, &splits, &tps);
   q.tiles_per_split = tps;
