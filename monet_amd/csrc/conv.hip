@@ -21,6 +21,7 @@
 // Operand tiles (BK = 16 deep) are staged through LDS k-major, double buffered:
 // the global loads of tile t+1 are in flight while tile t is multiplied.
 #include "common.h"
+#include <type_traits>
 #ifdef MN_TUNING
 #include <cstdlib>
 #endif
@@ -372,43 +373,63 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
     }
   }
 
-  // epilogue: lane owns columns (nj*32 + lane%32) and 16 rows per MFMA tile
-  const bool dense = g.osh == 1 && g.osw == 1;
+  // epilogue: lane owns columns (nj*32 + lane%32) and 16 rows per MFMA tile.  What kind of
+  // store it is and whether the tile has rows beyond M are uniform, so they select one of a
+  // few straight-line copies of the loop instead of being tested per element; an element's
+  // address is a per-thread byte offset plus a compile-time multiple of the plane size.
+  const uint32_t plane4 = (uint32_t)g.DH * g.DW * 4u;
+  char* dstb = reinterpret_cast<char*>(dst);
+  const bool add_bias = bias != nullptr && blockIdx.z == 0;
+  const int mbase = m0 + wm * (TL::TM * 32) + 4 * (lane >> 5);
+  auto emit = [&](auto full_tag, auto how_tag) {
+    constexpr bool kFull = decltype(full_tag)::value;
+    constexpr int kHow = decltype(how_tag)::value;
 #pragma unroll
-  for (int nj = 0; nj < TL::TN; ++nj) {
-    const uint32_t c = n0 + wn * (TL::TN * 32) + nj * 32 + (lane & 31);
-    if (c >= g.ncols) continue;
-    const uint32_t n = c / ((uint32_t)g.OH * g.OW);
-    const uint32_t rem = c - n * (uint32_t)g.OH * g.OW;
-    const uint32_t oh = rem / g.OW, ow = rem - oh * g.OW;
-    const size_t plane = (size_t)g.DH * g.DW;
-    float* out = dst + (size_t)n * g.M * plane + (size_t)(oh * g.osh + g.oh0) * g.DW +
-                 (ow * g.osw + g.ow0);
+    for (int nj = 0; nj < TL::TN; ++nj) {
+      const uint32_t c = n0 + wn * (TL::TN * 32) + nj * 32 + (lane & 31);
+      if (c >= g.ncols) continue;
+      const uint32_t n = c / ((uint32_t)g.OH * g.OW);
+      const uint32_t rem = c - n * (uint32_t)g.OH * g.OW;
+      const uint32_t oh = rem / g.OW, ow = rem - oh * g.OW;
+      const uint32_t col_b =
+          ((n * (uint32_t)g.M * g.DH + (oh * g.osh + g.oh0)) * (uint32_t)g.DW + (ow * g.osw + g.ow0)) * 4u +
+          (uint32_t)mbase * plane4;
 #pragma unroll
-    for (int mi = 0; mi < TL::TM; ++mi) {
+      for (int mi = 0; mi < TL::TM; ++mi) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int m = m0 + wm * (TL::TM * 32) + mi * 32 + acc_row(v, lane);
-        if (m < g.M) {
+        for (int v = 0; v < 16; ++v) {
+          const int dm = mi * 32 + 8 * (v >> 2) + (v & 3);
+          if (!kFull && mbase + dm >= g.M) continue;
           float r = acc[mi][nj][v];
-          if (bias && blockIdx.z == 0) r += bias[m];
-          if (g.ksplit > 1) {
-            atomicAdd(&out[(size_t)m * plane], r);
-            continue;
-          }
-          if (g.accum) {  // every element belongs to exactly one thread of the launch
-            out[(size_t)m * plane] += r;
-            continue;
-          }
-          // a dense output is written once and not read by this kernel: keep it out of the
-          // caches the operand tiles live in; strided (parity-class) outputs share cache lines
-          // between launches and are better left to the cache
-          if (dense)
-            st_stream(&out[(size_t)m * plane], r);
+          if (add_bias) r += bias[mbase + dm];
+          float* o = reinterpret_cast<float*>(dstb + (col_b + (uint32_t)dm * plane4));
+          if (kHow == 1)
+            atomicAdd(o, r);  // split reduction: the slices meet in a cleared output
+          else if (kHow == 2)
+            *o += r;          // accumulate: every element belongs to one thread of the launch
+          else if (kHow == 3)
+            st_stream(o, r);  // dense output, written once and not read here: around the caches
           else
-            out[(size_t)m * plane] = r;
+            *o = r;           // strided (parity-class) outputs share cache lines between launches
         }
       }
+    }
+  };
+  using std::integral_constant;
+  const int how = g.ksplit > 1 ? 1 : (g.accum ? 2 : ((g.osh == 1 && g.osw == 1) ? 3 : 0));
+  if (m0 + BM <= g.M) {
+    switch (how) {
+      case 1: emit(integral_constant<bool, true>{}, integral_constant<int, 1>{}); break;
+      case 2: emit(integral_constant<bool, true>{}, integral_constant<int, 2>{}); break;
+      case 3: emit(integral_constant<bool, true>{}, integral_constant<int, 3>{}); break;
+      default: emit(integral_constant<bool, true>{}, integral_constant<int, 0>{}); break;
+    }
+  } else {
+    switch (how) {
+      case 1: emit(integral_constant<bool, false>{}, integral_constant<int, 1>{}); break;
+      case 2: emit(integral_constant<bool, false>{}, integral_constant<int, 2>{}); break;
+      case 3: emit(integral_constant<bool, false>{}, integral_constant<int, 3>{}); break;
+      default: emit(integral_constant<bool, false>{}, integral_constant<int, 0>{}); break;
     }
   }
 }
