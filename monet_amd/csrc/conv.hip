@@ -642,6 +642,33 @@ __global__ __launch_bounds__(kThreads) void wgrad_kernel(const WGrad g,
 }
 
 
+// Writes a workgroup's accumulators as the (m0.., c0.., tap) piece of dw (tap-major column
+// tiles): plain store, atomic add, or the partial of split blockIdx.z.
+template <class TL>
+__device__ __forceinline__ void store_tap_tile(const WGrad& g, float16_t (&acc)[TL::TM][TL::TN],
+                                               float* __restrict__ out, int m0, uint32_t c0,
+                                               uint32_t tap, int wm, int wn, int lane) {
+  float* base = out;
+  if (g.mode == 2) base += (size_t)blockIdx.z * g.K * g.ncols;
+  const uint32_t RS = (uint32_t)g.R * g.S;
+#pragma unroll
+  for (int nj = 0; nj < TL::TN; ++nj) {
+    const uint32_t c = c0 + wn * (TL::TN * 32) + nj * 32 + (lane & 31);
+#pragma unroll
+    for (int mi = 0; mi < TL::TM; ++mi) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = m0 + wm * (TL::TM * 32) + mi * 32 + acc_row(v, lane);
+        float* o = base + (size_t)m * g.ncols + c * RS + tap;
+        if (g.mode == 1)
+          atomicAdd(o, acc[mi][nj][v]);
+        else
+          *o = acc[mi][nj][v];
+      }
+    }
+  }
+}
+
 // The same GEMM with the columns ordered tap-major, for C % BN == 0 and K % BM == 0:
 // blockIdx.x = tap * (C / BN) + channel tile, so a column tile lies inside ONE tap.
 // Then the window shift is a per-workgroup scalar, a thread's window test is one
@@ -741,25 +768,234 @@ __global__ __launch_bounds__(kThreads) void wgrad_tap_kernel(const WGrad g,
     if (sums_rows) store_row_sums<DEPTH, kRowsA>(row_sum, db, g, m0 + row0, kStep, kdl);
   }
 
-  float* base = out;
-  if (g.mode == 2) base += (size_t)blockIdx.z * g.K * g.ncols;
-  const uint32_t RS = (uint32_t)g.R * g.S;
+  store_tap_tile<TL>(g, acc, out, m0, c0, tap, wm, wn, lane);
+}
+
+// Tap-major backward-weight for images whose P*Q is a multiple of 4 (so is every depth tile
+// boundary, and N*P*Q).  Vector instructions that are not matrix instructions take issue
+// slots from the matrix pipe, so this variant is built to need few of them per tile:
+//  * LDS tiles are ROW-major, [row][DEPTH], the 16-byte chunks of a row XOR-swizzled by the
+//    row so that both the 128-bit fragment reads (8 rows at a time) and the staging writes are
+//    bank-conflict free without padding.  A lane's operands for 8 matrix steps are 2 chunks.
+//    The reduction index a lane feeds into step s is k = half * DEPTH/2 + s (any pairing of
+//    the tile's depths is a valid order of summation, A and B use the same one).
+//  * dy (and x for a 1x1, stride-1, unpadded filter: VECB) is contiguous along the depth, so
+//    it is fetched as float4 and staged with one 128-bit write per fetch; byte offsets are
+//    carried from tile to tile by addition (image wrap: one compare), the row part of an
+//    address sits in a uniform base pointer, and only the last tile masks its tail.
+//  * the gathered x of a windowed filter keeps one (p, q) position per thread, also carried
+//    by addition.
+// Images so small that one tile could cross two of them go to wgrad_tap_kernel instead.
+template <class TL, int DEPTH, bool DB, bool VECB>
+__global__ __launch_bounds__(kThreads) void wgrad_rows_kernel(const WGrad g,
+                                                              const float* __restrict__ dy,
+                                                              const float* __restrict__ x,
+                                                              float* __restrict__ out,
+                                                              float* __restrict__ db) {
+  constexpr int BM = TL::BM, BN = TL::BN;
+  constexpr int CPR = DEPTH / 4;  // 16-byte chunks per staged row
+  constexpr int RP = 32 / DEPTH;  // staged rows per 128 bytes of LDS
+  static_assert(DEPTH == 16 || DEPTH == 32, "row-major staging is laid out for 16 or 32 deep tiles");
+  __shared__ __attribute__((aligned(16))) float lds_a[2][BM * DEPTH];
+  __shared__ __attribute__((aligned(16))) float lds_b[2][BN * DEPTH];
+  auto swz = [](int row) { return (row / RP) & (CPR - 1); };  // chunk c of a row sits at c ^ swz(row)
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / TL::WN, wn = wave % TL::WN;
+  const int m0 = blockIdx.y * BM;
+  const uint32_t ctiles = (uint32_t)g.C / BN;
+  const uint32_t tap = blockIdx.x / ctiles;
+  const uint32_t c0 = (blockIdx.x - tap * ctiles) * BN;
+  const uint32_t r_tap = g.divS.div(tap), s_tap = tap - r_tap * g.S;
+  const int dh = (int)r_tap * g.dH - g.pH, dw = (int)s_tap * g.dW - g.pW;
+  const uint32_t PQ = (uint32_t)g.P * g.Q, PQ4 = PQ * 4u;
+  const uint32_t HW4 = (uint32_t)g.H * g.W * 4u;
+
+  const uint32_t total_tiles = (g.depth + DEPTH - 1) / DEPTH;
+  const uint32_t t_begin = blockIdx.z * (g.tiles_per_split * (WBK / DEPTH));
+  const uint32_t t_end = min(t_begin + g.tiles_per_split * (WBK / DEPTH), total_tiles);
+
+  // float4 loader: float4 number f = tid + kThreads*i of a tile is (row f / CPR, chunk f % CPR)
+  constexpr int kRowsPass = kThreads / CPR;
+  constexpr int kA4 = BM / kRowsPass, kB4 = BN / kRowsPass;
+  const int chunk = tid % CPR, vrow0 = tid / CPR;
+  // scalar loader of the gathered operand: depth lane kdl, rows row0 + kStep*i
+  constexpr int kStep = kThreads / DEPTH, kRowsB = BN / kStep;
+  const int kdl = tid % DEPTH, row0 = tid / DEPTH;
+
+  // depth position of this thread's float4 and the byte offsets that follow it
+  uint32_t vd = t_begin * DEPTH + 4 * chunk;
+  uint32_t vpq, a_off, bv_off = 0;
+  const uint32_t a_safe = (uint32_t)(m0 + vrow0) * PQ4, bv_safe = (c0 + vrow0) * PQ4;
+  {
+    const uint32_t n = vd / PQ;
+    vpq = vd - n * PQ;
+    a_off = (n * (uint32_t)g.K * PQ + vpq) * 4u + a_safe;
+    if (VECB) bv_off = (n * (uint32_t)g.C * PQ + vpq) * 4u + bv_safe;
+  }
+  const uint32_t a_wrap = (uint32_t)(g.K - 1) * PQ4, bv_wrap = (uint32_t)(g.C - 1) * PQ4;
+  // (p, q) of this thread's gathered element, and the byte offset of its image
+  uint32_t bd = t_begin * DEPTH + kdl, bp = 0, bq = 0, img_off = 0;
+  // a step of DEPTH crosses kq whole rows of the image and rq pixels; the host only sends
+  // images here that a step cannot cross twice (P*Q >= DEPTH and kq + 1 <= P)
+  const uint32_t kq = DEPTH / (uint32_t)g.Q, rq = DEPTH - kq * g.Q;
+  const uint32_t chw4 = (uint32_t)g.C * HW4;
+  const uint32_t b_row0 = (c0 + row0) * HW4 + (uint32_t)((dh * g.W + dw) * 4), b_step = kStep * HW4;
+  if (!VECB) {
+    const uint32_t n = bd / PQ, pq = bd - n * PQ;
+    bp = pq / g.Q;
+    bq = pq - bp * g.Q;
+    img_off = n * chw4;
+  }
+
+  const char* dyp = reinterpret_cast<const char*>(dy);
+  const char* xp = reinterpret_cast<const char*>(x);
+  // uniform row bases of the loads (the per-thread part of an address is one 32-bit offset)
+  const char* a_rows[kA4];
 #pragma unroll
-  for (int nj = 0; nj < TL::TN; ++nj) {
-    const uint32_t c = c0 + wn * (TL::TN * 32) + nj * 32 + (lane & 31);
+  for (int i = 0; i < kA4; ++i) a_rows[i] = dyp + (size_t)i * kRowsPass * PQ4;
+  const char* b_rows[VECB ? kB4 : kRowsB];
 #pragma unroll
-    for (int mi = 0; mi < TL::TM; ++mi) {
+  for (int i = 0; i < (VECB ? kB4 : kRowsB); ++i)
+    b_rows[i] = xp + (VECB ? (size_t)i * kRowsPass * PQ4 : (size_t)i * b_step);
+  float4_t ra4[kA4], rb4[VECB ? kB4 : 1];
+  float rb[VECB ? 1 : kRowsB];
+  float row_sum[DB ? kA4 : 1] = {};
+  const bool sums_rows = DB && blockIdx.x == 0;
+  bool a_ok = false, b_ok = false;
+  uint32_t tile_d0 = t_begin * DEPTH;  // uniform: first depth of the tile being fetched
+  bool tail = false;                   // uniform: that tile reaches past the reduction
+  auto fetch = [&]() {
+    tail = tile_d0 + DEPTH > g.depth;
+    tile_d0 += DEPTH;
+    a_ok = vd < g.depth;
+    const uint32_t ao = a_ok ? a_off : a_safe;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int m = m0 + wm * (TL::TM * 32) + mi * 32 + acc_row(v, lane);
-        float* o = base + (size_t)m * g.ncols + c * RS + tap;
-        if (g.mode == 1)
-          atomicAdd(o, acc[mi][nj][v]);
-        else
-          *o = acc[mi][nj][v];
+    for (int i = 0; i < kA4; ++i)
+      ra4[i] = *reinterpret_cast<const float4_t*>(a_rows[i] + ao);
+    if (VECB) {
+      const uint32_t bo = a_ok ? bv_off : bv_safe;
+#pragma unroll
+      for (int i = 0; i < kB4; ++i)
+        rb4[i] = *reinterpret_cast<const float4_t*>(b_rows[i] + bo);
+    } else {
+      const int h0 = (int)__umul24(bp, (uint32_t)g.sH), w0 = (int)__umul24(bq, (uint32_t)g.sW);
+      b_ok = bd < g.depth && (unsigned)(h0 + dh) < (unsigned)g.H && (unsigned)(w0 + dw) < (unsigned)g.W;
+      // an element outside the window is staged as zero; its load reads the row's first element
+      const uint32_t bbase = b_ok ? img_off + (uint32_t)(h0 * g.W + w0) * 4u + b_row0 : (c0 + row0) * HW4;
+#pragma unroll
+      for (int i = 0; i < kRowsB; ++i)
+        rb[i] = *reinterpret_cast<const float*>(b_rows[i] + bbase);
+      // next tile
+      bd += DEPTH;
+      bq += rq;
+      bp += kq;
+      if (bq >= (uint32_t)g.Q) {
+        bq -= g.Q;
+        ++bp;
+      }
+      if (bp >= (uint32_t)g.P) {
+        bp -= g.P;
+        img_off += chw4;
       }
     }
+    vd += DEPTH;
+    vpq += DEPTH;
+    a_off += DEPTH * 4;
+    if (VECB) bv_off += DEPTH * 4;
+    if (vpq >= PQ) {
+      vpq -= PQ;
+      a_off += a_wrap;
+      if (VECB) bv_off += bv_wrap;
+    }
+  };
+  // LDS byte offsets of this thread's staging writes (the swizzle is the same for all its rows)
+  const uint32_t va_w = (uint32_t)(vrow0 * DEPTH + ((chunk ^ swz(vrow0)) << 2));
+  const uint32_t sb_w = (uint32_t)(row0 * DEPTH + ((((kdl >> 2) ^ swz(row0)) << 2) | (kdl & 3)));
+  auto stage = [&](int buf) {
+    const float4_t z = {0.f, 0.f, 0.f, 0.f};
+    if (tail) {  // only the last tile of the reduction; kept a branch (the asm is a barrier to if-conversion)
+      asm volatile("" ::: "memory");
+#pragma unroll
+      for (int i = 0; i < kA4; ++i) ra4[i] = a_ok ? ra4[i] : z;
+      if (VECB) {
+#pragma unroll
+        for (int i = 0; i < kB4; ++i) rb4[i] = a_ok ? rb4[i] : z;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < kA4; ++i) {
+      const float4_t v = ra4[i];
+      *reinterpret_cast<float4_t*>(&lds_a[buf][va_w + i * kRowsPass * DEPTH]) = v;
+      if constexpr (DB) {
+        if (sums_rows) row_sum[i] += (v[0] + v[1]) + (v[2] + v[3]);
+      }
+    }
+    if (VECB) {
+#pragma unroll
+      for (int i = 0; i < kB4; ++i)
+        *reinterpret_cast<float4_t*>(&lds_b[buf][va_w + i * kRowsPass * DEPTH]) = rb4[i];
+    } else {
+#pragma unroll
+      for (int i = 0; i < kRowsB; ++i) lds_b[buf][sb_w + i * kStep * DEPTH] = b_ok ? rb[i] : 0.f;
+    }
+  };
+
+  float16_t acc[TL::TM][TL::TN];
+#pragma unroll
+  for (int i = 0; i < TL::TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TL::TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  // fragment reads: lane (r, half) owns rows r of each 32-row block and depths half*DEPTH/2 ...
+  const int r = lane & 31, half = lane >> 5;
+  const int fa_row = wm * (TL::TM * 32) + r, fb_row = wn * (TL::TN * 32) + r;
+  const int f_swz = swz(r);  // block bases are multiples of 32: the swizzle only depends on r
+  auto multiply = [&](int buf) {
+#pragma unroll
+    for (int g8 = 0; g8 < DEPTH / 16; ++g8) {
+      const int cb = half * (CPR / 2) + 2 * g8;
+      float4_t a4[TL::TM][2], b4[TL::TN][2];
+#pragma unroll
+      for (int i = 0; i < TL::TM; ++i)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+          a4[i][h] = *reinterpret_cast<const float4_t*>(
+              &lds_a[buf][(fa_row + 32 * i) * DEPTH + (((cb + h) ^ f_swz) << 2)]);
+#pragma unroll
+      for (int j = 0; j < TL::TN; ++j)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+          b4[j][h] = *reinterpret_cast<const float4_t*>(
+              &lds_b[buf][(fb_row + 32 * j) * DEPTH + (((cb + h) ^ f_swz) << 2)]);
+#pragma unroll
+      for (int st = 0; st < 8; ++st)
+#pragma unroll
+        for (int i = 0; i < TL::TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TL::TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4[i][st >> 2][st & 3], b4[j][st >> 2][st & 3],
+                                                             acc[i][j], 0, 0, 0);
+    }
+  };
+
+  if (t_begin < t_end) {
+    fetch();
+    stage(0);
+    __syncthreads();
+    for (uint32_t kt = t_begin; kt < t_end; ++kt) {
+      const int buf = (kt - t_begin) & 1;
+      if (kt + 1 < t_end) fetch();
+      multiply(buf);
+      if (kt + 1 < t_end) stage(buf ^ 1);
+      __syncthreads();
+    }
   }
+  if constexpr (DB) {
+    if (sums_rows) store_row_sums<CPR, kA4>(row_sum, db, g, m0 + vrow0, kRowsPass, chunk);
+  }
+  store_tap_tile<TL>(g, acc, out, m0, c0, tap, wm, wn, lane);
 }
 
 // dw[i] = sum over splits of partial[z][i], fixed order.
@@ -1245,6 +1481,41 @@ static int conv_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, vo
   // with atomics, a tap-major tile would scatter them R*S floats apart: only for 1x1 filters
   if (wgrad_tap_major(g, bm, bn) && (q.mode != 1 || g->R * g->S == 1)) {
     dim3 grid(g->R * g->S * (g->C / bn), g->K / bm, splits);
+    // row-major staging with float4 fetches: images of a multiple of 4 pixels, 16-byte aligned
+    // tensors; x too is fetched as float4 where the filter is a plain 1x1
+    const bool vecb = g->R * g->S == 1 && g->sH == 1 && g->sW == 1 && g->pH == 0 && g->pW == 0;
+    bool rows = ((long long)g->P * g->Q) % 4 == 0 && mn_aligned(dy, 16) && (!vecb || mn_aligned(x, 16)) &&
+                (long long)g->P * g->Q >= 32 && 32 / g->Q + 1 <= g->P;
+#ifdef MN_TUNING
+    if (const char* e = getenv("MN_WGRAD_ROWS")) rows = rows && atoi(e) != 0;
+#endif
+    if (rows) {
+#define MN_ROWS_V(TL, D, B, V)                                                                  \
+  wgrad_rows_kernel<TL, D, B, V><<<grid, kThreads, 0, s>>>(q, (const float*)dy, (const float*)x, \
+                                                           out, db_dst)
+#define MN_ROWS(TL, D)              \
+  if (db) {                         \
+    if (vecb) {                     \
+      MN_ROWS_V(TL, D, true, true); \
+    } else {                        \
+      MN_ROWS_V(TL, D, true, false); \
+    }                               \
+  } else {                          \
+    if (vecb) {                     \
+      MN_ROWS_V(TL, D, false, true); \
+    } else {                        \
+      MN_ROWS_V(TL, D, false, false); \
+    }                               \
+  }
+      switch (tile) {
+        case 2: MN_ROWS(T64x128, 32); break;
+        case 3: MN_ROWS(T128x64, 32); break;
+        case 4: MN_ROWS(T64x64, 32); break;
+        default: MN_ROWS(T128x128, 16); break;
+      }
+#undef MN_ROWS
+#undef MN_ROWS_V
+    } else {
     int deep = tile == 0 ? 16 : 32;  // 128 x 128 at depth 32 leaves LDS for 2 workgroups per CU only
 #ifdef MN_TUNING
     if (const char* e = getenv("MN_WGRAD_DEPTH")) deep = atoi(e);
@@ -1270,6 +1541,7 @@ static int conv_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, vo
     }
 #undef MN_TAP
 #undef MN_TAP_D
+    }
   } else {
     dim3 grid((q.ncols + bn - 1) / bn, (g->K + bm - 1) / bm, splits);
 #define MN_GEN(TL)                                                                              \
