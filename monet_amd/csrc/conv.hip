@@ -785,13 +785,16 @@ __global__ __launch_bounds__(kThreads) void wgrad_tap_kernel(const WGrad g,
 //    address sits in a uniform base pointer, and only the last tile masks its tail.
 //  * the gathered x of a windowed filter keeps one (p, q) position per thread, also carried
 //    by addition.
+// Without VECA (P*Q not a multiple of 4, or unaligned tensors) dy is fetched lane by lane
+// like the gathered x, with the same carried addresses and the same LDS layout.
 // Images so small that one tile could cross two of them go to wgrad_tap_kernel instead.
-template <class TL, int DEPTH, bool DB, bool VECB>
+template <class TL, int DEPTH, bool DB, bool VECA, bool VECB_>
 __global__ __launch_bounds__(kThreads) void wgrad_rows_kernel(const WGrad g,
                                                               const float* __restrict__ dy,
                                                               const float* __restrict__ x,
                                                               float* __restrict__ out,
                                                               float* __restrict__ db) {
+  constexpr bool VECB = VECA && VECB_;  // without float4 alignment both operands go lane by lane
   constexpr int BM = TL::BM, BN = TL::BN;
   constexpr int CPR = DEPTH / 4;  // 16-byte chunks per staged row
   constexpr int RP = 32 / DEPTH;  // staged rows per 128 bytes of LDS
@@ -819,7 +822,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_rows_kernel(const WGrad g,
   constexpr int kA4 = BM / kRowsPass, kB4 = BN / kRowsPass;
   const int chunk = tid % CPR, vrow0 = tid / CPR;
   // scalar loader of the gathered operand: depth lane kdl, rows row0 + kStep*i
-  constexpr int kStep = kThreads / DEPTH, kRowsB = BN / kStep;
+  constexpr int kStep = kThreads / DEPTH, kRowsA = BM / kStep, kRowsB = BN / kStep;
   const int kdl = tid % DEPTH, row0 = tid / DEPTH;
 
   // depth position of this thread's float4 and the byte offsets that follow it
@@ -840,26 +843,30 @@ __global__ __launch_bounds__(kThreads) void wgrad_rows_kernel(const WGrad g,
   const uint32_t kq = DEPTH / (uint32_t)g.Q, rq = DEPTH - kq * g.Q;
   const uint32_t chw4 = (uint32_t)g.C * HW4;
   const uint32_t b_row0 = (c0 + row0) * HW4 + (uint32_t)((dh * g.W + dw) * 4), b_step = kStep * HW4;
+  uint32_t as_off = 0;  // scalar dy loader (!VECA): byte offset of (image, pixel, row m0 + row0)
+  const uint32_t as_safe = (uint32_t)(m0 + row0) * PQ4;
   if (!VECB) {
     const uint32_t n = bd / PQ, pq = bd - n * PQ;
     bp = pq / g.Q;
     bq = pq - bp * g.Q;
     img_off = n * chw4;
+    as_off = (n * (uint32_t)g.K * PQ + pq) * 4u + as_safe;
   }
 
   const char* dyp = reinterpret_cast<const char*>(dy);
   const char* xp = reinterpret_cast<const char*>(x);
   // uniform row bases of the loads (the per-thread part of an address is one 32-bit offset)
-  const char* a_rows[kA4];
+  const char* a_rows[VECA ? kA4 : kRowsA];
 #pragma unroll
-  for (int i = 0; i < kA4; ++i) a_rows[i] = dyp + (size_t)i * kRowsPass * PQ4;
+  for (int i = 0; i < (VECA ? kA4 : kRowsA); ++i)
+    a_rows[i] = dyp + (VECA ? (size_t)i * kRowsPass * PQ4 : (size_t)i * kStep * PQ4);
   const char* b_rows[VECB ? kB4 : kRowsB];
 #pragma unroll
   for (int i = 0; i < (VECB ? kB4 : kRowsB); ++i)
     b_rows[i] = xp + (VECB ? (size_t)i * kRowsPass * PQ4 : (size_t)i * b_step);
-  float4_t ra4[kA4], rb4[VECB ? kB4 : 1];
-  float rb[VECB ? 1 : kRowsB];
-  float row_sum[DB ? kA4 : 1] = {};
+  float4_t ra4[VECA ? kA4 : 1], rb4[VECB ? kB4 : 1];
+  float ra[VECA ? 1 : kRowsA], rb[VECB ? 1 : kRowsB];
+  float row_sum[DB ? (VECA ? kA4 : kRowsA) : 1] = {};
   const bool sums_rows = DB && blockIdx.x == 0;
   bool a_ok = false, b_ok = false;
   uint32_t tile_d0 = t_begin * DEPTH;  // uniform: first depth of the tile being fetched
@@ -867,11 +874,17 @@ __global__ __launch_bounds__(kThreads) void wgrad_rows_kernel(const WGrad g,
   auto fetch = [&]() {
     tail = tile_d0 + DEPTH > g.depth;
     tile_d0 += DEPTH;
-    a_ok = vd < g.depth;
-    const uint32_t ao = a_ok ? a_off : a_safe;
+    if (VECA) {
+      a_ok = vd < g.depth;
+      const uint32_t ao = a_ok ? a_off : a_safe;
 #pragma unroll
-    for (int i = 0; i < kA4; ++i)
-      ra4[i] = *reinterpret_cast<const float4_t*>(a_rows[i] + ao);
+      for (int i = 0; i < kA4; ++i) ra4[i] = *reinterpret_cast<const float4_t*>(a_rows[i] + ao);
+    } else {
+      a_ok = bd < g.depth;
+      const uint32_t ao = a_ok ? as_off : as_safe;
+#pragma unroll
+      for (int i = 0; i < kRowsA; ++i) ra[i] = *reinterpret_cast<const float*>(a_rows[i] + ao);
+    }
     if (VECB) {
       const uint32_t bo = a_ok ? bv_off : bv_safe;
 #pragma unroll
@@ -889,23 +902,27 @@ __global__ __launch_bounds__(kThreads) void wgrad_rows_kernel(const WGrad g,
       bd += DEPTH;
       bq += rq;
       bp += kq;
+      if (!VECA) as_off += DEPTH * 4;
       if (bq >= (uint32_t)g.Q) {
         bq -= g.Q;
         ++bp;
       }
-      if (bp >= (uint32_t)g.P) {
+      if (bp >= (uint32_t)g.P) {  // next image
         bp -= g.P;
         img_off += chw4;
+        if (!VECA) as_off += a_wrap;
       }
     }
-    vd += DEPTH;
-    vpq += DEPTH;
-    a_off += DEPTH * 4;
-    if (VECB) bv_off += DEPTH * 4;
-    if (vpq >= PQ) {
-      vpq -= PQ;
-      a_off += a_wrap;
-      if (VECB) bv_off += bv_wrap;
+    if (VECA) {
+      vd += DEPTH;
+      vpq += DEPTH;
+      a_off += DEPTH * 4;
+      if (VECB) bv_off += DEPTH * 4;
+      if (vpq >= PQ) {
+        vpq -= PQ;
+        a_off += a_wrap;
+        if (VECB) bv_off += bv_wrap;
+      }
     }
   };
   // LDS byte offsets of this thread's staging writes (the swizzle is the same for all its rows)
@@ -915,19 +932,34 @@ __global__ __launch_bounds__(kThreads) void wgrad_rows_kernel(const WGrad g,
     const float4_t z = {0.f, 0.f, 0.f, 0.f};
     if (tail) {  // only the last tile of the reduction; kept a branch (the asm is a barrier to if-conversion)
       asm volatile("" ::: "memory");
+      if (VECA) {
 #pragma unroll
-      for (int i = 0; i < kA4; ++i) ra4[i] = a_ok ? ra4[i] : z;
+        for (int i = 0; i < kA4; ++i) ra4[i] = a_ok ? ra4[i] : z;
+      } else {
+#pragma unroll
+        for (int i = 0; i < kRowsA; ++i) ra[i] = a_ok ? ra[i] : 0.f;
+      }
       if (VECB) {
 #pragma unroll
         for (int i = 0; i < kB4; ++i) rb4[i] = a_ok ? rb4[i] : z;
       }
     }
+    if constexpr (VECA) {
 #pragma unroll
-    for (int i = 0; i < kA4; ++i) {
-      const float4_t v = ra4[i];
-      *reinterpret_cast<float4_t*>(&lds_a[buf][va_w + i * kRowsPass * DEPTH]) = v;
-      if constexpr (DB) {
-        if (sums_rows) row_sum[i] += (v[0] + v[1]) + (v[2] + v[3]);
+      for (int i = 0; i < kA4; ++i) {
+        const float4_t v = ra4[i];
+        *reinterpret_cast<float4_t*>(&lds_a[buf][va_w + i * kRowsPass * DEPTH]) = v;
+        if constexpr (DB) {
+          if (sums_rows) row_sum[i] += (v[0] + v[1]) + (v[2] + v[3]);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < kRowsA; ++i) {
+        lds_a[buf][sb_w + i * kStep * DEPTH] = ra[i];
+        if constexpr (DB) {
+          if (sums_rows) row_sum[i] += ra[i];
+        }
       }
     }
     if (VECB) {
@@ -993,7 +1025,12 @@ __global__ __launch_bounds__(kThreads) void wgrad_rows_kernel(const WGrad g,
     }
   }
   if constexpr (DB) {
-    if (sums_rows) store_row_sums<CPR, kA4>(row_sum, db, g, m0 + vrow0, kRowsPass, chunk);
+    if (sums_rows) {
+      if constexpr (VECA)
+        store_row_sums<CPR, kA4>(row_sum, db, g, m0 + vrow0, kRowsPass, chunk);
+      else
+        store_row_sums<DEPTH, kRowsA>(row_sum, db, g, m0 + row0, kStep, kdl);
+    }
   }
   store_tap_tile<TL>(g, acc, out, m0, c0, tap, wm, wn, lane);
 }
@@ -1481,18 +1518,22 @@ static int conv_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, vo
   // with atomics, a tap-major tile would scatter them R*S floats apart: only for 1x1 filters
   if (wgrad_tap_major(g, bm, bn) && (q.mode != 1 || g->R * g->S == 1)) {
     dim3 grid(g->R * g->S * (g->C / bn), g->K / bm, splits);
-    // row-major staging with float4 fetches: images of a multiple of 4 pixels, 16-byte aligned
-    // tensors; x too is fetched as float4 where the filter is a plain 1x1
+    // row-major staging; float4 fetches of dy for images of a multiple of 4 pixels and 16-byte
+    // aligned tensors, of x too where the filter is a plain 1x1
     const bool vecb = g->R * g->S == 1 && g->sH == 1 && g->sW == 1 && g->pH == 0 && g->pW == 0;
-    bool rows = ((long long)g->P * g->Q) % 4 == 0 && mn_aligned(dy, 16) && (!vecb || mn_aligned(x, 16)) &&
-                (long long)g->P * g->Q >= 32 && 32 / g->Q + 1 <= g->P;
+    const bool veca = ((long long)g->P * g->Q) % 4 == 0 && mn_aligned(dy, 16) && (!vecb || mn_aligned(x, 16));
+    bool rows = (long long)g->P * g->Q >= 32 && 32 / g->Q + 1 <= g->P;
 #ifdef MN_TUNING
     if (const char* e = getenv("MN_WGRAD_ROWS")) rows = rows && atoi(e) != 0;
 #endif
     if (rows) {
-#define MN_ROWS_V(TL, D, B, V)                                                                  \
-  wgrad_rows_kernel<TL, D, B, V><<<grid, kThreads, 0, s>>>(q, (const float*)dy, (const float*)x, \
-                                                           out, db_dst)
+#define MN_ROWS_V(TL, D, B, V)                                                                   \
+  if (veca)                                                                                      \
+    wgrad_rows_kernel<TL, D, B, true, V><<<grid, kThreads, 0, s>>>(q, (const float*)dy,          \
+                                                                   (const float*)x, out, db_dst); \
+  else                                                                                           \
+    wgrad_rows_kernel<TL, D, B, false, false><<<grid, kThreads, 0, s>>>(                         \
+        q, (const float*)dy, (const float*)x, out, db_dst)
 #define MN_ROWS(TL, D)              \
   if (db) {                         \
     if (vecb) {                     \

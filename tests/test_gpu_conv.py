@@ -30,6 +30,9 @@ CASES = [
     ((2, 256, 28, 28), (512, 256, 1, 1), 2, 0, 1),     # strided 1x1 (downsample)
     ((2, 3, 64, 64), (64, 3, 7, 7), 2, 3, 1),          # stem
     ((1, 16, 33, 47), (24, 16, 3, 3), 1, 1, 1),        # odd spatial sizes
+    ((5, 128, 7, 7), (128, 128, 3, 3), 1, 1, 1),       # 49-pixel images: no 16-byte alignment along the depth
+    ((5, 128, 7, 7), (256, 128, 1, 1), 1, 0, 1),       # the same, 1x1
+    ((3, 64, 9, 11), (64, 64, 3, 3), 1, 1, 1),         # 99 pixels, 64-channel tiles
 ]
 
 
