@@ -59,7 +59,7 @@ typedef Tile<64, 128, 1, 4> T64x128;
 typedef Tile<128, 64, 4, 1> T128x64;
 typedef Tile<64, 64, 2, 2> T64x64;
 
-// n / d for n < 2^20, d < 4096 (mul = floor(2^32 / d) + 1).
+// n / d, exact while n * d < 2^32 (mul = floor(2^32 / d) + 1): e.g. n < 2^20 and d < 4096.
 struct FastDiv {
   uint32_t mul, d;
   __device__ __forceinline__ uint32_t div(uint32_t n) const {
@@ -118,7 +118,19 @@ struct Gather {
   int32_t aoff[kMaxTaps];
   int ksplit, tiles_per_split;  // split reduction (ksplit > 1): grid.z slices of k-tiles
   int accum;                    // add to what dst already holds instead of overwriting it
+  FastDiv divOHW, divOW;        // column -> (image, row, column) by multiplication ...
+  int exact_div;                // ... unless ncols * OH*OW is beyond FastDiv's exact range
 };
+
+// Column c of the GEMM = output pixel (n, oh, ow).
+__device__ __forceinline__ void split_column(const Gather& g, uint32_t c, uint32_t& n, uint32_t& oh,
+                                             uint32_t& ow) {
+  const uint32_t ohw = (uint32_t)g.OH * g.OW;
+  n = g.exact_div ? c / ohw : g.divOHW.div(c);
+  const uint32_t rem = c - n * ohw;
+  oh = g.exact_div ? rem / (uint32_t)g.OW : g.divOW.div(rem);
+  ow = rem - oh * g.OW;
+}
 
 // FAST: the source has a multiple of BK channels.  Then the reduction index
 // runs tap-major (kk = tap*Cs + ch): a k-tile lies inside one tap, so the
@@ -168,10 +180,8 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
   int ohs = 0, ows = 0;
   uint32_t img = 0;
   {
-    const uint32_t c = col_ok ? col : 0;
-    img = c / ((uint32_t)g.OH * g.OW);
-    const uint32_t rem = c - img * (uint32_t)g.OH * g.OW;
-    const uint32_t oh = rem / g.OW, ow = rem - oh * g.OW;
+    uint32_t oh, ow;
+    split_column(g, col_ok ? col : 0, img, oh, ow);
     ohs = oh * g.ish;
     ows = ow * g.isw;
   }
@@ -217,7 +227,7 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
       const int f = tid + kThreads * i;
       const uint32_t krow = f / (BN / 4), c4 = n0 + 4 * (f % (BN / 4));
       const bool ok = c4 < g.ncols;
-      const uint32_t im = ok ? c4 / PQ : 0u;
+      const uint32_t im = ok ? (g.exact_div ? c4 / PQ : g.divOHW.div(c4)) : 0u;
       const uint32_t px = ok ? c4 - im * PQ : 0u;
       bp_b[i] = (im * (uint32_t)g.Cs + krow) * plane_b + px * 4u;
       bp_ok |= (ok ? 1u : 0u) << i;
@@ -241,22 +251,27 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
     const int hh = ohs + dh, ww = ows + dw;
     tap_in = col_ok && (unsigned)hh < (unsigned)g.Hs && (unsigned)ww < (unsigned)g.Ws;
     tap_b = tap_in ? pix_b + (uint32_t)((dh * g.Ws + dw) * 4) : brow0 * plane_b;
-    tap_a = PACKED ? (uint32_t)((long long)taoff[t] * g.Cs * g.lda * 4) : (uint32_t)(taoff[t] * 4);
+    const int ao = __builtin_amdgcn_readfirstlane(taoff[t]);  // uniform: keep it in a scalar register
+    tap_a = PACKED ? (uint32_t)((long long)ao * g.Cs * g.lda * 4) : (uint32_t)(ao * 4);
   };
   // Only issues loads: masking happens in stage(), after the multiply of the current
   // tile, so the loads stay in flight behind the matrix instructions.  The per-tile part of
   // every address is uniform (c0), so it goes into the base pointer and the per-thread
   // offsets stay put for a whole tap.
+  // uniform bases of the rows one thread gathers (row i is channel brow0 + kBStep*i of the tile)
+  const char* b_rows[kBRows];
+#pragma unroll
+  for (int i = 0; i < kBRows; ++i) b_rows[i] = sp + (size_t)(kBStep * i) * plane_b;
   auto fetch_fast = [&](int c0) {  // c0 uniform
     b_in = tap_in;
-    const char* spc = sp + (size_t)c0 * plane_b;
     if (POINT) {
+      const char* spc = sp + (size_t)c0 * plane_b;
 #pragma unroll
       for (int i = 0; i < kB4; ++i) rb4[i] = *reinterpret_cast<const float4_t*>(spc + bp_b[i]);
     } else {
+      const uint32_t off = tap_b + (uint32_t)c0 * plane_b;
 #pragma unroll
-      for (int i = 0; i < kBRows; ++i)
-        rb[i] = *reinterpret_cast<const float*>(spc + (tap_b + kBStep * i * plane_b));
+      for (int i = 0; i < kBRows; ++i) rb[i] = *reinterpret_cast<const float*>(b_rows[i] + off);
     }
     if (PACKED) {
       const char* apc = ap + ((size_t)tap_a + (size_t)c0 * g.lda * 4);
@@ -388,9 +403,8 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
     for (int nj = 0; nj < TL::TN; ++nj) {
       const uint32_t c = n0 + wn * (TL::TN * 32) + nj * 32 + (lane & 31);
       if (c >= g.ncols) continue;
-      const uint32_t n = c / ((uint32_t)g.OH * g.OW);
-      const uint32_t rem = c - n * (uint32_t)g.OH * g.OW;
-      const uint32_t oh = rem / g.OW, ow = rem - oh * g.OW;
+      uint32_t n, oh, ow;
+      split_column(g, c, n, oh, ow);
       const uint32_t col_b =
           ((n * (uint32_t)g.M * g.DH + (oh * g.osh + g.oh0)) * (uint32_t)g.DW + (ow * g.osw + g.ow0)) * 4u +
           (uint32_t)mbase * plane4;
@@ -1171,6 +1185,10 @@ static void launch_gather(Gather g, const float* a, const float* src, const floa
                           float* dst, hipStream_t s, bool packed = false, bool split_ok = false,
                           int tile = -1) {
   if (g.ncols == 0 || g.M == 0) return;
+  g.divOHW = make_fastdiv((uint32_t)(g.OH * g.OW));
+  g.divOW = make_fastdiv((uint32_t)g.OW);
+  // multiplication by the reciprocal is exact while dividend * divisor < 2^32
+  g.exact_div = ((unsigned long long)(g.ncols + 256) * (unsigned long long)(g.OH * g.OW) >= (1ull << 32)) ? 1 : 0;
 #ifdef MN_TUNING
   if (const char* e = getenv("MN_CONV_TILE")) tile = atoi(e);
 #endif
