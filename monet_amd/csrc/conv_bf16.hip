@@ -89,11 +89,21 @@ struct GatherH {
   int DH, DW, osh, osw, oh0, ow0;  // dst [N, DH, DW, Nout], position = oh*osh + oh0
   int T;                  // taps of this launch
   uint32_t wrow;          // elements between consecutive weight rows
+  uint32_t src_bytes, w_bytes;  // sizes of the two operand tensors (set by the launcher)
   int16_t dh[kMaxTaps], dw[kMaxTaps];
   int32_t woff[kMaxTaps]; // element offset of tap t inside a weight row
 };
 
 // DEPTH = reduction elements staged per barrier.
+// A bf16 matrix instruction is short (a workgroup tile of 128 x 128 x 32 is 8 of them per
+// wavefront, ~256 cycles), so anything else a wavefront has to issue per tile shows directly,
+// and a load must be in flight for more than one tile to be hidden.  Hence:
+//  * operands are fetched with raw buffer loads: the per-thread byte offset of a row is fixed
+//    for a whole tap (a row outside the window or the tensor gets an offset beyond the buffer
+//    and reads as zero: no masks when staging), the per-tile part (channel offset) is the
+//    scalar offset of the instruction: no vector arithmetic per tile;
+//  * two register sets: the loads of tile t+2 are issued before tile t is multiplied and
+//    are staged during tile t+1.
 template <int BN, int DEPTH>
 __global__ __launch_bounds__(kThreads) void gather_bf16_kernel(const GatherH g,
                                                                const bf16_t* __restrict__ src,
@@ -105,6 +115,7 @@ __global__ __launch_bounds__(kThreads) void gather_bf16_kernel(const GatherH g,
   constexpr int kRPP = kThreads / kCPR;       // rows covered by one pass of the workgroup
   constexpr int kARows = BM / kRPP, kBRows = BN / kRPP;  // chunks per thread
   constexpr int LDR = DEPTH + 8;              // LDS row length (elements): 80 or 144 bytes
+  constexpr uint32_t kBeyond = 0x80000000u;   // byte offset past any buffer (tensors are < 2 GB)
   __shared__ __attribute__((aligned(16))) bf16_t lds_a[2][BM][LDR];
   __shared__ __attribute__((aligned(16))) bf16_t lds_b[2][BN][LDR];
   __shared__ int tdh[kMaxTaps], tdw[kMaxTaps], twoff[kMaxTaps];
@@ -145,40 +156,48 @@ __global__ __launch_bounds__(kThreads) void gather_bf16_kernel(const GatherH g,
     ows[i] = ow * g.isw;
     abase[i] = n * (uint32_t)g.Hs * g.Ws;
   }
-  // B loader: chunk `chunk` of weight rows n0 + arow + kRPP*i
-  uint32_t bbase[kBRows];
-  bool bok[kBRows];
+  // B loader: chunk `chunk` of weight rows n0 + arow + kRPP*i; byte offsets, fixed for the launch
+  uint32_t b_off[kBRows];
 #pragma unroll
   for (int i = 0; i < kBRows; ++i) {
     const int col = n0 + arow + kRPP * i;
-    bok[i] = col < g.Nout;
-    bbase[i] = (bok[i] ? (uint32_t)col : 0u) * g.wrow + chunk * 8;
+    b_off[i] = col < g.Nout ? ((uint32_t)col * g.wrow + chunk * 8) * 2u : kBeyond;
   }
   __syncthreads();
 
-  uint4_t ra[kARows], rb[kBRows];
-  bool ra_ok[kARows];
-  auto fetch = [&](int t, int c0) {  // t, c0 uniform
+  const __amdgpu_buffer_rsrc_t src_buf =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(src), 0, g.src_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t w_buf =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(w), 0, g.w_bytes, 0x00020000);
+  // per-tap state: byte offsets of this thread's rows of the source (or kBeyond), and the
+  // uniform byte offset of the tap inside a weight row
+  uint32_t a_off[kARows];
+  int w_tap = 0;
+  auto enter_tap = [&](int t) {  // t uniform
     const int dh = tdh[t], dw = tdw[t];
 #pragma unroll
     for (int i = 0; i < kARows; ++i) {
       const int hh = ohs[i] + dh, ww = ows[i] + dw;
-      ra_ok[i] = aok[i] && (unsigned)hh < (unsigned)g.Hs && (unsigned)ww < (unsigned)g.Ws;
-      const uint32_t e = ra_ok[i] ? (abase[i] + hh * g.Ws + ww) * (uint32_t)g.Cs + c0 + chunk * 8 : 0u;
-      ra[i] = *reinterpret_cast<const uint4_t*>(src + e);
+      const bool ok = aok[i] && (unsigned)hh < (unsigned)g.Hs && (unsigned)ww < (unsigned)g.Ws;
+      a_off[i] = ok ? ((abase[i] + hh * g.Ws + ww) * (uint32_t)g.Cs + chunk * 8) * 2u : kBeyond;
     }
-    const uint32_t wo = twoff[t] + c0;
-#pragma unroll
-    for (int i = 0; i < kBRows; ++i) rb[i] = *reinterpret_cast<const uint4_t*>(w + bbase[i] + wo);
+    w_tap = __builtin_amdgcn_readfirstlane(twoff[t]) * 2;
   };
-  auto stage = [&](int buf) {
-    const uint4_t z = {0u, 0u, 0u, 0u};
+  auto fetch = [&](uint4_t (&ra)[kARows], uint4_t (&rb)[kBRows], int c0) {  // c0 uniform
 #pragma unroll
     for (int i = 0; i < kARows; ++i)
-      *reinterpret_cast<uint4_t*>(&lds_a[buf][arow + kRPP * i][chunk * 8]) = ra_ok[i] ? ra[i] : z;
+      ra[i] = __builtin_amdgcn_raw_buffer_load_b128(src_buf, a_off[i], c0 * 2, 0);
 #pragma unroll
     for (int i = 0; i < kBRows; ++i)
-      *reinterpret_cast<uint4_t*>(&lds_b[buf][arow + kRPP * i][chunk * 8]) = bok[i] ? rb[i] : z;
+      rb[i] = __builtin_amdgcn_raw_buffer_load_b128(w_buf, b_off[i], w_tap + c0 * 2, 0);
+  };
+  auto stage = [&](int buf, const uint4_t (&ra)[kARows], const uint4_t (&rb)[kBRows]) {
+#pragma unroll
+    for (int i = 0; i < kARows; ++i)
+      *reinterpret_cast<uint4_t*>(&lds_a[buf][arow + kRPP * i][chunk * 8]) = ra[i];
+#pragma unroll
+    for (int i = 0; i < kBRows; ++i)
+      *reinterpret_cast<uint4_t*>(&lds_b[buf][arow + kRPP * i][chunk * 8]) = rb[i];
   };
 
   float16_t acc[2][TN];
@@ -192,25 +211,45 @@ __global__ __launch_bounds__(kThreads) void gather_bf16_kernel(const GatherH g,
   const int per_tap = g.Cs / DEPTH;
   const int ktiles = g.T * per_tap;
   if (ktiles > 0) {
-    int t = 0, c0 = 0;
-    auto fetch_next = [&]() {
-      fetch(t, c0);
+    uint4_t ra0[kARows], rb0[kBRows], ra1[kARows], rb1[kBRows];
+    int t = 0, c0 = 0;  // position of the next tile to fetch
+    enter_tap(0);
+    auto advance = [&]() {
       c0 += DEPTH;
       if (c0 == g.Cs) {
         c0 = 0;
         ++t;
+        if (t < g.T) enter_tap(t);
       }
     };
-    fetch_next();
-    stage(0);
+    fetch(ra0, rb0, c0);  // tile 0
+    advance();
+    if (ktiles > 1) {
+      fetch(ra1, rb1, c0);  // tile 1
+      advance();
+    }
+    stage(0, ra0, rb0);
     __syncthreads();
-    for (int kt = 0; kt < ktiles; ++kt) {
-      const int buf = kt & 1;
-      if (kt + 1 < ktiles) fetch_next();
-      mma_tile<2, TN, BM, BN, DEPTH>(lds_a[buf], lds_b[buf], wm, wn, lane, acc);
-      if (kt + 1 < ktiles) stage(buf ^ 1);
+    for (int kt = 0; kt + 1 < ktiles; kt += 2) {
+      // tile kt is in LDS buffer 0, tile kt+1 in flight in set 1
+      if (kt + 2 < ktiles) {
+        fetch(ra0, rb0, c0);
+        advance();
+      }
+      mma_tile<2, TN, BM, BN, DEPTH>(lds_a[0], lds_b[0], wm, wn, lane, acc);
+      stage(1, ra1, rb1);
+      __syncthreads();
+      // tile kt+1 is in LDS buffer 1, tile kt+2 in flight in set 0
+      if (kt + 3 < ktiles) {
+        fetch(ra1, rb1, c0);
+        advance();
+      }
+      mma_tile<2, TN, BM, BN, DEPTH>(lds_a[1], lds_b[1], wm, wn, lane, acc);
+      if (kt + 2 < ktiles) stage(0, ra0, rb0);
       __syncthreads();
     }
+    // an odd number of tiles: the last one was staged into buffer 0
+    if (ktiles & 1) mma_tile<2, TN, BM, BN, DEPTH>(lds_a[0], lds_b[0], wm, wn, lane, acc);
   }
 
   // epilogue: for a fixed register, lanes 0..31 hold 32 consecutive channels of one position
@@ -424,9 +463,16 @@ static int check16(const mn_conv2d* g) {
   return MN_OK;
 }
 
-static void launch_gather16(const GatherH& q, const bf16_t* src, const bf16_t* w, const bf16_t* bias,
-                            bf16_t* dst, hipStream_t s) {
-  if (q.npix == 0 || q.Nout == 0) return;
+static int launch_gather16(GatherH q, const bf16_t* src, const bf16_t* w, const bf16_t* bias,
+                           bf16_t* dst, hipStream_t s) {
+  if (q.npix == 0 || q.Nout == 0) return MN_OK;
+  // the kernel addresses its operands through buffer descriptors with byte offsets below 2^31
+  const unsigned long long n_img = q.npix / ((unsigned long long)q.OH * q.OW);
+  const unsigned long long src_bytes = n_img * q.Hs * q.Ws * q.Cs * 2ull;
+  const unsigned long long w_bytes = (unsigned long long)q.Nout * q.wrow * 2ull;
+  if (src_bytes >= (1ull << 31) || w_bytes >= (1ull << 31)) return MN_EUNSUPPORTED;
+  q.src_bytes = (uint32_t)src_bytes;
+  q.w_bytes = (uint32_t)w_bytes;
   // 32-deep staging: 64-deep tiles (half as many barriers) measured 10 % slower at the
   // ResNet-50 layer3 shape because their LDS footprint halves the resident workgroups
   if (q.Nout % 128 == 0) {
@@ -436,6 +482,7 @@ static void launch_gather16(const GatherH& q, const bf16_t* src, const bf16_t* w
     dim3 grid((q.npix + BM - 1) / BM, (q.Nout + 63) / 64);
     gather_bf16_kernel<64, 32><<<grid, kThreads, 0, s>>>(q, src, w, bias, dst);
   }
+  return MN_OK;
 }
 
 static void wgrad16_tiles(const mn_conv2d* g, int* bm, int* bn) {
@@ -509,7 +556,8 @@ int mn_conv16_fwd(const mn_conv2d* g, const void* x, const void* w, const void* 
       q.dw[t] = (int16_t)(sx * g->dW - g->pW);
       q.woff[t] = t * g->C;
     }
-  launch_gather16(q, (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias, (bf16_t*)y, s);
+  const int lst = launch_gather16(q, (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias, (bf16_t*)y, s);
+  if (lst != MN_OK) return lst;
   return mn_launch_status();
 }
 
@@ -571,7 +619,8 @@ int mn_conv16_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void* 
       q.osh = g->sH;
       q.osw = g->sW;
       q.wrow = (uint32_t)T * g->K;
-      launch_gather16(q, (const bf16_t*)dy, (const bf16_t*)ws, nullptr, (bf16_t*)dx, s);
+      const int lst = launch_gather16(q, (const bf16_t*)dy, (const bf16_t*)ws, nullptr, (bf16_t*)dx, s);
+      if (lst != MN_OK) return lst;
     }
   }
   return mn_launch_status();
