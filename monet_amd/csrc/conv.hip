@@ -118,6 +118,7 @@ struct Gather {
   int32_t aoff[kMaxTaps];
   int ksplit, tiles_per_split;  // split reduction (ksplit > 1): grid.z slices of k-tiles
   int accum;                    // add to what dst already holds instead of overwriting it
+  uint32_t src_bytes, a_bytes;  // sizes of the source tensor and of the repacked A (PACKED)
   FastDiv divOHW, divOW;        // column -> (image, row, column) by multiplication ...
   int exact_div;                // ... unless ncols * OH*OW is beyond FastDiv's exact range
 };
@@ -143,9 +144,14 @@ __device__ __forceinline__ void split_column(const Gather& g, uint32_t c, uint32
 // floats (a multiple of 128, zero padded), so a k-tile of A is BK contiguous
 // row pieces: one 16-byte load per lane and row piece, no masks, and 8 cache
 // lines per wavefront load instead of the ~20 a strided gather touches.
+// PACKED kernels fetch through raw buffer descriptors: a thread's byte offset is fixed for a
+// whole tap, an element outside the window or the tensor gets an offset beyond the buffer
+// and reads as zero (no masks when staging), and the per-tile part of an address is the
+// scalar offset of the load: no vector arithmetic per tile.  Both tensors must be < 2 GB.
 // POINT (with PACKED): a 1x1 filter, stride 1, no padding - the gather is the identity, a
 // k-tile of B is BK contiguous rows of pixels, loaded and staged as 16-byte vectors too.
 constexpr int kPadPacked = 4;  // keeps LDS rows 16-byte aligned for the 128-bit stores
+constexpr uint32_t kBeyond = 0x80000000u;  // a byte offset past the end of any buffer
 template <class TL, bool FAST, bool PACKED = false, bool POINT = false>
 __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
                                                                const float* __restrict__ a,
@@ -229,7 +235,7 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
       const bool ok = c4 < g.ncols;
       const uint32_t im = ok ? (g.exact_div ? c4 / PQ : g.divOHW.div(c4)) : 0u;
       const uint32_t px = ok ? c4 - im * PQ : 0u;
-      bp_b[i] = (im * (uint32_t)g.Cs + krow) * plane_b + px * 4u;
+      bp_b[i] = ok ? (im * (uint32_t)g.Cs + krow) * plane_b + px * 4u : kBeyond;
       bp_ok |= (ok ? 1u : 0u) << i;
     }
   }
@@ -246,11 +252,15 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
   uint32_t tap_b = 0, tap_a = 0;
   bool tap_in = false;
   bool b_in = false;  // tap_in at the time of the last fetch: what stage() masks with
+  const __amdgpu_buffer_rsrc_t src_buf = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float*>(src), 0, PACKED ? g.src_bytes : 0u, 0x00020000);
+  const __amdgpu_buffer_rsrc_t a_buf = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float*>(a), 0, PACKED ? g.a_bytes : 0u, 0x00020000);
   auto enter_tap = [&](int t) {  // t uniform
     const int dh = tdh[t], dw = tdw[t];
     const int hh = ohs + dh, ww = ows + dw;
     tap_in = col_ok && (unsigned)hh < (unsigned)g.Hs && (unsigned)ww < (unsigned)g.Ws;
-    tap_b = tap_in ? pix_b + (uint32_t)((dh * g.Ws + dw) * 4) : brow0 * plane_b;
+    tap_b = tap_in ? pix_b + (uint32_t)((dh * g.Ws + dw) * 4) : (PACKED ? kBeyond : brow0 * plane_b);
     const int ao = __builtin_amdgcn_readfirstlane(taoff[t]);  // uniform: keep it in a scalar register
     tap_a = PACKED ? (uint32_t)((long long)ao * g.Cs * g.lda * 4) : (uint32_t)(ao * 4);
   };
@@ -265,18 +275,25 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
   auto fetch_fast = [&](int c0) {  // c0 uniform
     b_in = tap_in;
     if (POINT) {
-      const char* spc = sp + (size_t)c0 * plane_b;
+      const uint32_t so = (uint32_t)c0 * plane_b;
 #pragma unroll
-      for (int i = 0; i < kB4; ++i) rb4[i] = *reinterpret_cast<const float4_t*>(spc + bp_b[i]);
+      for (int i = 0; i < kB4; ++i)
+        rb4[i] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(src_buf, bp_b[i], so, 0));
+    } else if (PACKED) {
+#pragma unroll
+      for (int i = 0; i < kBRows; ++i)
+        rb[i] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(
+            src_buf, tap_b, (uint32_t)(c0 + kBStep * i) * plane_b, 0));
     } else {
       const uint32_t off = tap_b + (uint32_t)c0 * plane_b;
 #pragma unroll
       for (int i = 0; i < kBRows; ++i) rb[i] = *reinterpret_cast<const float*>(b_rows[i] + off);
     }
     if (PACKED) {
-      const char* apc = ap + ((size_t)tap_a + (size_t)c0 * g.lda * 4);
+      const uint32_t so = tap_a + (uint32_t)c0 * (uint32_t)g.lda * 4u;
 #pragma unroll
-      for (int i = 0; i < kA4; ++i) ra4[i] = *reinterpret_cast<const float4_t*>(apc + ap_b[i]);
+      for (int i = 0; i < kA4; ++i)
+        ra4[i] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(a_buf, ap_b[i], so, 0));
     } else {
       const char* apc = ap + ((size_t)tap_a + (size_t)c0 * g.cha * 4);
 #pragma unroll
@@ -319,13 +336,14 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
 #pragma unroll
       for (int i = 0; i < kB4; ++i) {
         const int f = tid + kThreads * i;
-        *reinterpret_cast<float4_t*>(&lds_b[buf][f / (BN / 4)][4 * (f % (BN / 4))]) =
-            ((bp_ok >> i) & 1u) ? rb4[i] : z;
+        (void)z;
+        *reinterpret_cast<float4_t*>(&lds_b[buf][f / (BN / 4)][4 * (f % (BN / 4))]) = rb4[i];
       }
     } else {
 #pragma unroll
       for (int i = 0; i < kBRows; ++i) {
-        const bool in = FAST ? b_in : (((b_ok >> i) & 1u) != 0);
+        // PACKED: what lies outside the window was fetched as zero already
+        const bool in = PACKED ? true : (FAST ? b_in : (((b_ok >> i) & 1u) != 0));
         lds_b[buf][brow0 + kBStep * i][bcol] = in ? rb[i] : 0.f;
       }
     }
@@ -1087,6 +1105,11 @@ __global__ __launch_bounds__(kThreads) void pack_weights_kernel(const float* __r
 }
 
 static long long packed_rows(long long M) { return (M + 127) / 128 * 128; }
+// The repacked-weight kernels address both operands through buffer descriptors with byte
+// offsets below 2^31; larger tensors run variant 1 with the variant-0 kernel.
+static bool buffers_fit(size_t src_floats, size_t a_floats) {
+  return src_floats < (1ull << 29) && a_floats < (1ull << 29);
+}
 
 // ------------------------------------------------------------------ host --
 static int check(const mn_conv2d* g) {
@@ -1185,6 +1208,9 @@ static void launch_gather(Gather g, const float* a, const float* src, const floa
                           float* dst, hipStream_t s, bool packed = false, bool split_ok = false,
                           int tile = -1) {
   if (g.ncols == 0 || g.M == 0) return;
+  if (packed) {  // the callers have checked buffers_fit()
+    g.src_bytes = (uint32_t)((size_t)g.N * g.Cs * g.Hs * g.Ws * sizeof(float));
+  }
   g.divOHW = make_fastdiv((uint32_t)(g.OH * g.OW));
   g.divOW = make_fastdiv((uint32_t)g.OW);
   // multiplication by the reciprocal is exact while dividend * divisor < 2^32
@@ -1353,7 +1379,8 @@ int mn_conv_fwd(const mn_conv2d* g, const void* x, const void* w, const void* bi
   hipStream_t s = mn_stream(stream);
   const float* a = (const float*)w;
   // the repacked operand needs the tap-major path; other shapes run variant 1 like variant 0
-  const bool packed = variant == 1 && fast_path(q);
+  const bool packed = variant == 1 && fast_path(q) &&
+                      buffers_fit((size_t)g->N * g->C * g->H * g->W, (size_t)q.T * q.Cs * packed_rows(q.M));
   if (packed) {
     const long long Mp = packed_rows(q.M);
     const size_t n = (size_t)q.T * q.Cs * Mp;
@@ -1362,6 +1389,7 @@ int mn_conv_fwd(const mn_conv2d* g, const void* x, const void* w, const void* bi
         a, (float*)ws, q.M, (int)Mp, q.Cs, q.T, q.lda, q.cha);
     a = (const float*)ws;
     q.lda = Mp;
+    q.a_bytes = (uint32_t)(n * sizeof(float));
   }
   launch_gather(q, a, (const float*)x, (const float*)bias, (float*)y, s, packed, packed);
   return mn_launch_status();
@@ -1381,8 +1409,10 @@ static int conv_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void
   if (dtype != MN_F32) return MN_EUNSUPPORTED;
   const int RS = g->R * g->S;
   const float* a = (const float*)w;
+  uint32_t a_bytes = 0;  // size of the repacked operand
   long long lda = RS, cha = (long long)g->C * RS;  // read w[k][c][r][s] as A(c, k, rs)
-  const bool packed = variant == 1 && g->K % BK == 0;
+  const bool packed = variant == 1 && g->K % BK == 0 &&
+                      buffers_fit((size_t)g->N * g->K * g->P * g->Q, (size_t)RS * g->K * packed_rows(g->C));
   if (packed) {  // A'[rs][k][c], rows of Cp floats
     const long long Cp = packed_rows(g->C);
     const size_t n = (size_t)RS * g->K * Cp;
@@ -1391,6 +1421,7 @@ static int conv_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void
         a, (float*)ws, g->C, (int)Cp, g->K, RS, lda, cha);
     a = (const float*)ws;
     lda = Cp;
+    a_bytes = (uint32_t)(n * sizeof(float));
   }
   // Classes no tap can reach (e.g. 1x1 filters with stride 2) are plain zeros: clear dx once
   // with full-width stores instead of scattering zeros class by class.
@@ -1444,6 +1475,7 @@ static int conv_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void
       q.osh = g->sH;
       q.osw = g->sW;
       q.lda = lda;
+      q.a_bytes = a_bytes;
       q.cha = cha;
       q.accum = accum ? 1 : 0;
       launch_gather(q, a, (const float*)dy, nullptr, (float*)dx, s, packed,
