@@ -499,6 +499,7 @@ struct WGrad {
   uint32_t ncols;       // C*R*S
   FastDiv divRS, divS, divQ;
   int exact_div;             // P*Q or Q beyond FastDiv's range: divide the slow way
+  uint32_t dy_bytes, x_bytes;  // tensor sizes, for the kernels that read through buffer descriptors
   uint32_t tiles_per_split;  // k-tiles handled by one blockIdx.z
   int mode;             // 0: store, 1: atomicAdd into dw, 2: store partial [z][K][ncols]
 };
@@ -814,7 +815,8 @@ __global__ __launch_bounds__(kThreads) void wgrad_tap_kernel(const WGrad g,
 //  * dy (and x for a 1x1, stride-1, unpadded filter: VECB) is contiguous along the depth, so
 //    it is fetched as float4 and staged with one 128-bit write per fetch; byte offsets are
 //    carried from tile to tile by addition (image wrap: one compare), the row part of an
-//    address sits in a uniform base pointer, and only the last tile masks its tail.
+//    address is the scalar offset of a buffer load, and what lies beyond the reduction or
+//    outside the window is fetched as zero (an offset past the buffer): no staging masks.
 //  * the gathered x of a windowed filter keeps one (p, q) position per thread, also carried
 //    by addition.
 // Without VECA (P*Q not a multiple of 4, or unaligned tensors) dy is fetched lane by lane
@@ -887,49 +889,47 @@ __global__ __launch_bounds__(kThreads) void wgrad_rows_kernel(const WGrad g,
 
   const char* dyp = reinterpret_cast<const char*>(dy);
   const char* xp = reinterpret_cast<const char*>(x);
-  // uniform row bases of the loads (the per-thread part of an address is one 32-bit offset)
-  const char* a_rows[VECA ? kA4 : kRowsA];
-#pragma unroll
-  for (int i = 0; i < (VECA ? kA4 : kRowsA); ++i)
-    a_rows[i] = dyp + (VECA ? (size_t)i * kRowsPass * PQ4 : (size_t)i * kStep * PQ4);
-  const char* b_rows[VECB ? kB4 : kRowsB];
-#pragma unroll
-  for (int i = 0; i < (VECB ? kB4 : kRowsB); ++i)
-    b_rows[i] = xp + (VECB ? (size_t)i * kRowsPass * PQ4 : (size_t)i * b_step);
+  // Both tensors are read through buffer descriptors: the per-thread part of an address is one
+  // 32-bit byte offset, the row part the load's scalar offset, and an element that is not to
+  // be read (beyond the reduction, outside the window) gets an offset past the buffer and
+  // arrives as zero, so staging has no masks.
+  const __amdgpu_buffer_rsrc_t dy_buf =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(dy), 0, g.dy_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t x_buf =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(x), 0, g.x_bytes, 0x00020000);
+  const uint32_t a_row_step = (VECA ? kRowsPass : kStep) * PQ4;
+  const uint32_t b_row_step = VECB ? kRowsPass * PQ4 : b_step;
   float4_t ra4[VECA ? kA4 : 1], rb4[VECB ? kB4 : 1];
   float ra[VECA ? 1 : kRowsA], rb[VECB ? 1 : kRowsB];
   float row_sum[DB ? (VECA ? kA4 : kRowsA) : 1] = {};
   const bool sums_rows = DB && blockIdx.x == 0;
   bool a_ok = false, b_ok = false;
-  uint32_t tile_d0 = t_begin * DEPTH;  // uniform: first depth of the tile being fetched
-  bool tail = false;                   // uniform: that tile reaches past the reduction
   auto fetch = [&]() {
-    tail = tile_d0 + DEPTH > g.depth;
-    tile_d0 += DEPTH;
     if (VECA) {
       a_ok = vd < g.depth;
-      const uint32_t ao = a_ok ? a_off : a_safe;
+      const uint32_t ao = a_ok ? a_off : kBeyond;
 #pragma unroll
-      for (int i = 0; i < kA4; ++i) ra4[i] = *reinterpret_cast<const float4_t*>(a_rows[i] + ao);
+      for (int i = 0; i < kA4; ++i)
+        ra4[i] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(dy_buf, ao, i * a_row_step, 0));
     } else {
       a_ok = bd < g.depth;
-      const uint32_t ao = a_ok ? as_off : as_safe;
+      const uint32_t ao = a_ok ? as_off : kBeyond;
 #pragma unroll
-      for (int i = 0; i < kRowsA; ++i) ra[i] = *reinterpret_cast<const float*>(a_rows[i] + ao);
+      for (int i = 0; i < kRowsA; ++i)
+        ra[i] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(dy_buf, ao, i * a_row_step, 0));
     }
     if (VECB) {
-      const uint32_t bo = a_ok ? bv_off : bv_safe;
+      const uint32_t bo = a_ok ? bv_off : kBeyond;
 #pragma unroll
       for (int i = 0; i < kB4; ++i)
-        rb4[i] = *reinterpret_cast<const float4_t*>(b_rows[i] + bo);
+        rb4[i] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(x_buf, bo, i * b_row_step, 0));
     } else {
       const int h0 = (int)__umul24(bp, (uint32_t)g.sH), w0 = (int)__umul24(bq, (uint32_t)g.sW);
       b_ok = bd < g.depth && (unsigned)(h0 + dh) < (unsigned)g.H && (unsigned)(w0 + dw) < (unsigned)g.W;
-      // an element outside the window is staged as zero; its load reads the row's first element
-      const uint32_t bbase = b_ok ? img_off + (uint32_t)(h0 * g.W + w0) * 4u + b_row0 : (c0 + row0) * HW4;
+      const uint32_t bbase = b_ok ? img_off + (uint32_t)(h0 * g.W + w0) * 4u + b_row0 : kBeyond;
 #pragma unroll
       for (int i = 0; i < kRowsB; ++i)
-        rb[i] = *reinterpret_cast<const float*>(b_rows[i] + bbase);
+        rb[i] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(x_buf, bbase, i * b_row_step, 0));
       // next tile
       bd += DEPTH;
       bq += rq;
@@ -961,21 +961,6 @@ __global__ __launch_bounds__(kThreads) void wgrad_rows_kernel(const WGrad g,
   const uint32_t va_w = (uint32_t)(vrow0 * DEPTH + ((chunk ^ swz(vrow0)) << 2));
   const uint32_t sb_w = (uint32_t)(row0 * DEPTH + ((((kdl >> 2) ^ swz(row0)) << 2) | (kdl & 3)));
   auto stage = [&](int buf) {
-    const float4_t z = {0.f, 0.f, 0.f, 0.f};
-    if (tail) {  // only the last tile of the reduction; kept a branch (the asm is a barrier to if-conversion)
-      asm volatile("" ::: "memory");
-      if (VECA) {
-#pragma unroll
-        for (int i = 0; i < kA4; ++i) ra4[i] = a_ok ? ra4[i] : z;
-      } else {
-#pragma unroll
-        for (int i = 0; i < kRowsA; ++i) ra[i] = a_ok ? ra[i] : 0.f;
-      }
-      if (VECB) {
-#pragma unroll
-        for (int i = 0; i < kB4; ++i) rb4[i] = a_ok ? rb4[i] : z;
-      }
-    }
     if constexpr (VECA) {
 #pragma unroll
       for (int i = 0; i < kA4; ++i) {
@@ -1000,7 +985,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_rows_kernel(const WGrad g,
         *reinterpret_cast<float4_t*>(&lds_b[buf][va_w + i * kRowsPass * DEPTH]) = rb4[i];
     } else {
 #pragma unroll
-      for (int i = 0; i < kRowsB; ++i) lds_b[buf][sb_w + i * kStep * DEPTH] = b_ok ? rb[i] : 0.f;
+      for (int i = 0; i < kRowsB; ++i) lds_b[buf][sb_w + i * kStep * DEPTH] = rb[i];
     }
   };
 
@@ -1543,6 +1528,10 @@ static int conv_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, vo
   q.divRS = make_fastdiv(g->R * g->S);
   q.divS = make_fastdiv(g->S);
   q.divQ = make_fastdiv(g->Q);
+  const unsigned long long dy_bytes = (unsigned long long)g->N * g->K * g->P * g->Q * sizeof(float);
+  const unsigned long long x_bytes = (unsigned long long)g->N * g->C * g->H * g->W * sizeof(float);
+  q.dy_bytes = (uint32_t)dy_bytes;
+  q.x_bytes = (uint32_t)x_bytes;
   q.exact_div = ((long long)g->P * g->Q > (1ll << 20) || g->Q >= 4096) ? 1 : 0;
   int splits, tps;
   wgrad_split(g, variant, &splits, &tps);
@@ -1572,7 +1561,8 @@ static int conv_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, vo
     // aligned tensors, of x too where the filter is a plain 1x1
     const bool vecb = g->R * g->S == 1 && g->sH == 1 && g->sW == 1 && g->pH == 0 && g->pW == 0;
     const bool veca = ((long long)g->P * g->Q) % 4 == 0 && mn_aligned(dy, 16) && (!vecb || mn_aligned(x, 16));
-    bool rows = (long long)g->P * g->Q >= 32 && 32 / g->Q + 1 <= g->P;
+    bool rows = (long long)g->P * g->Q >= 32 && 32 / g->Q + 1 <= g->P &&
+                dy_bytes < (1ull << 31) && x_bytes < (1ull << 31);  // buffer offsets below 2^31
 #ifdef MN_TUNING
     if (const char* e = getenv("MN_WGRAD_ROWS")) rows = rows && atoi(e) != 0;
 #endif
