@@ -16,11 +16,30 @@ class AdaptiveAvgPool2D(OP):
     def forward(self, x, output_size):
         with torch.no_grad():
             self.params = x.shape, x.device, x.dtype
+            if self._replicates(x.shape, output_size):
+                # an output that is a whole multiple of the input averages windows of one
+                # element (the reference's UNet upsamples this way, unet_parts.py:45-56):
+                # nearest-neighbour replication, the same values from a plain copy kernel
+                return torch.ops.aten.upsample_nearest2d(x, [int(output_size[0]), int(output_size[1])])
             return torch._C._nn.adaptive_avg_pool2d(x, output_size)
 
     @staticmethod
     def _is_global(grad_shape):
         return len(grad_shape) == 4 and grad_shape[2] == 1 and grad_shape[3] == 1
+
+    @staticmethod
+    def _replicates(in_shape, out_size):
+        if len(in_shape) != 4 or out_size is None or len(out_size) != 2:
+            return False
+        if out_size[0] is None or out_size[1] is None:
+            return False
+        h, w, oh, ow = int(in_shape[2]), int(in_shape[3]), int(out_size[0]), int(out_size[1])
+        if h <= 0 or w <= 0 or oh % h or ow % w or (oh == h and ow == w):
+            return False
+        # powers of two only: the copy kernel finds its source as floor(i * (h / oh)) in
+        # single precision, which is exact for these factors
+        fh, fw = oh // h, ow // w
+        return fh & (fh - 1) == 0 and fw & (fw - 1) == 0
 
     def backward(self, grad_output, stored, nodel=False):
         assert len(stored) == 0
@@ -30,6 +49,12 @@ class AdaptiveAvgPool2D(OP):
                 # global average: every position of a plane gets grad / (H*W); one streaming
                 # write instead of the atomic scatter of the generic backward
                 return (grad_output * (1.0 / (shape[2] * shape[3]))).expand(shape).contiguous()
+            if len(shape) == 4 and self._replicates(shape, grad_output.shape[2:]):
+                # replication forward: every input element collects its fh x fw copies, a
+                # gather without the atomic scatter of the generic backward
+                return torch.ops.aten.upsample_nearest2d_backward(
+                    grad_output.contiguous(), [int(grad_output.shape[2]), int(grad_output.shape[3])],
+                    [int(d) for d in shape])
             # the aten backward only reads the shape of its second argument
             like = torch.empty(1, dtype=dtype, device=device).expand(list(shape))
             return torch.ops.aten._adaptive_avg_pool2d_backward(grad_output.contiguous(), like)

@@ -445,6 +445,19 @@ def test_glue_ops_backward_matches_autograd(cuda):
     torch.nn.functional.adaptive_avg_pool2d(xr, [1, 1]).backward(g)
     torch.testing.assert_close(op.backward(g, []), xr.grad)
 
+    # an output that is a whole (power of two) multiple of the input: replication, taken by a
+    # copy kernel / gather instead of the generic pooling kernels; also a size that is not
+    for in_hw, out_hw in (((5, 7), (10, 14)), ((3, 4), (12, 4)), ((5, 7), (15, 21)), ((6, 6), (4, 9))):
+        xu = torch.randn(2, 3, *in_hw, device=cuda)
+        up = lm_ops.funcs.AdaptiveAvgPool2D()
+        yu = up.forward(xu, list(out_hw))
+        xur = xu.clone().requires_grad_(True)
+        ref = torch.nn.functional.adaptive_avg_pool2d(xur, list(out_hw))
+        assert torch.equal(yu, ref.detach())
+        gu = torch.randn_like(yu)
+        ref.backward(gu)
+        torch.testing.assert_close(up.backward(gu, []), xur.grad)
+
     lin = lm_ops.linear.LowMemLinear()
     inp = torch.randn(5, 8, device=cuda, requires_grad=True)
     w = torch.randn(3, 8, device=cuda, requires_grad=True)
