@@ -68,3 +68,24 @@ def test_ops_refuse_cpu_tensors():
         lm_ops.pool.IndicesActMaxPool2D().forward(torch.zeros(1, 1, 4, 4), 2, 2, 0, 1, False)
     with pytest.raises(RuntimeError, match="GPU tensor"):
         lm_ops.bn.bn_forward_train(torch.zeros(2, 2, 2, 2), None, None, None, None, 0.1, 1e-5)
+
+
+def test_adaptive_avg_pool_replication_path_equals_the_pooling_operator():
+    """Outputs that are a power-of-two multiple of the input (the reference UNet's upsampling,
+    unet_parts.py:45-56) take a copy / gather path; values and gradients must equal those of
+    aten's adaptive pooling, and other sizes must keep using it."""
+    torch.manual_seed(0)
+    rep = lm_ops.funcs.AdaptiveAvgPool2D._replicates
+    assert rep((1, 2, 26, 38), (52, 76)) and rep((1, 2, 3, 4), (12, 4))
+    assert not rep((1, 2, 5, 7), (15, 21))      # factor 3: not exact in single precision
+    assert not rep((1, 2, 6, 6), (4, 9)) and not rep((1, 2, 6, 6), (6, 6)) and not rep((1, 2, 6, 6), (1, 1))
+    for in_hw, out_hw in (((5, 7), (10, 14)), ((3, 4), (12, 4)), ((5, 7), (15, 21)), ((6, 6), (4, 9))):
+        x = torch.randn(2, 3, *in_hw, dtype=torch.float64)
+        op = lm_ops.funcs.AdaptiveAvgPool2D()
+        y = op.forward(x, list(out_hw))
+        xr = x.clone().requires_grad_(True)
+        ref = torch.nn.functional.adaptive_avg_pool2d(xr, list(out_hw))
+        assert torch.equal(y, ref.detach())
+        g = torch.randn_like(y)
+        ref.backward(g)
+        torch.testing.assert_close(op.backward(g, []), xr.grad, rtol=1e-12, atol=1e-12)
