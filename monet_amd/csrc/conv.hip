@@ -225,7 +225,6 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
   constexpr int kB4 = BN * BK / 4 / kThreads;
   float4_t rb4[kB4 > 0 ? kB4 : 1];
   uint32_t bp_b[kB4 > 0 ? kB4 : 1];
-  uint32_t bp_ok = 0;
   if (POINT) {
     const uint32_t PQ = (uint32_t)g.OH * g.OW;  // a multiple of 4: a float4 stays inside an image
 #pragma unroll
@@ -235,8 +234,8 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
       const bool ok = c4 < g.ncols;
       const uint32_t im = ok ? (g.exact_div ? c4 / PQ : g.divOHW.div(c4)) : 0u;
       const uint32_t px = ok ? c4 - im * PQ : 0u;
+      // columns past the end read as zero (an offset beyond the buffer)
       bp_b[i] = ok ? (im * (uint32_t)g.Cs + krow) * plane_b + px * 4u : kBeyond;
-      bp_ok |= (ok ? 1u : 0u) << i;
     }
   }
 
@@ -332,11 +331,9 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
   };
   auto stage = [&](int buf) {
     if (POINT) {
-      const float4_t z = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int i = 0; i < kB4; ++i) {
         const int f = tid + kThreads * i;
-        (void)z;
         *reinterpret_cast<float4_t*>(&lds_b[buf][f / (BN / 4)][4 * (f % (BN / 4))]) = rb4[i];
       }
     } else {
