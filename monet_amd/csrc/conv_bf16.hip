@@ -295,9 +295,23 @@ struct WGradH {
   uint32_t depth;            // N*P*Q
   uint32_t tiles_per_split;  // 32-position tiles per blockIdx.z
   int partial;               // 1: fp32 partial[z][K][T][C]; 0: bf16 dw[K][T][C] (single split)
+  uint32_t dy_bytes, x_bytes;  // tensor sizes for the buffer descriptors
 };
 
 // rows = BMW output channels (k), columns = BNW input channels of ONE tap.
+// Both operands hold 8 channels of one position per 16-byte chunk while LDS wants positions
+// innermost, so chunks are transposed on their way in.  As in the gather kernel everything
+// else a wavefront issues per tile is kept small, because a tile is only 8 matrix
+// instructions per wavefront:
+//  * chunk e = tid + kThreads*i of a tile is (position e % BK, channel group e / BK): all
+//    chunks of a thread share ONE position, so one (image, p, q) tracker per thread, moved by
+//    additions, serves them all, and consecutive lanes hold consecutive positions;
+//  * dy is [position][K]: its byte offset is fixed for the whole kernel, the tile offset is the
+//    load's scalar offset, and positions beyond the reduction lie beyond the buffer (read as
+//    zero).  x gets one offset per tile (or one beyond the buffer outside the window);
+//  * transposing store: a lane pair swaps halves (DPP) and one byte-permute builds the dword
+//    of (channel, two positions): 2 vector instructions per 4-byte LDS store, no masks;
+//  * two register sets keep the loads of tile t+2 in flight while tile t is multiplied.
 template <int BMW, int BNW>
 __global__ __launch_bounds__(kThreads) void wgrad_bf16_kernel(const WGradH g,
                                                               const bf16_t* __restrict__ dy,
@@ -306,6 +320,8 @@ __global__ __launch_bounds__(kThreads) void wgrad_bf16_kernel(const WGradH g,
   constexpr int TM = BMW / 64, TN = BNW / 64;
   constexpr int kAChunks = BMW * BK / 8 / kThreads;  // 16-byte chunks per thread and tile
   constexpr int kBChunks = BNW * BK / 8 / kThreads;
+  constexpr int kGroupStep = kThreads / BK;          // channel groups between a thread's chunks
+  constexpr uint32_t kBeyond = 0x80000000u;          // byte offset past any buffer (tensors < 2 GB)
   __shared__ __attribute__((aligned(16))) bf16_t lds_a[2][BMW][LDK];
   __shared__ __attribute__((aligned(16))) bf16_t lds_b[2][BNW][LDK];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -322,84 +338,72 @@ __global__ __launch_bounds__(kThreads) void wgrad_bf16_kernel(const WGradH g,
   const uint32_t t_begin = blockIdx.z * g.tiles_per_split;
   const uint32_t t_end = min(t_begin + g.tiles_per_split, total_tiles);
 
-  // chunk e = tid + kThreads*i of a tile: position e % BK, channel group e / BK.  Consecutive
-  // lanes take consecutive positions so that their two-byte LDS stores fall into different
-  // banks (8 rows apart is a multiple of all 32 banks); the loads of a channel group's
-  // neighbours come from the same cache lines a moment later.
-  uint32_t a_pos[kAChunks], b_pos[kBChunks];  // position inside the tile
-  uint32_t an[kAChunks], ap[kAChunks], aq[kAChunks];  // (n, p, q) of that position
-  uint32_t bn[kBChunks], bp[kBChunks], bq[kBChunks];
-  auto split = [&](uint32_t d, uint32_t& n, uint32_t& p, uint32_t& q) {
-    n = d / PQ;
-    const uint32_t pq = d - n * PQ;
-    p = pq / g.Q;
-    q = pq - p * g.Q;
-  };
-#pragma unroll
-  for (int i = 0; i < kAChunks; ++i) {
-    a_pos[i] = (tid + kThreads * i) % BK;
-    split(t_begin * BK + a_pos[i], an[i], ap[i], aq[i]);
+  const __amdgpu_buffer_rsrc_t dy_buf =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(dy), 0, g.dy_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t x_buf =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(x), 0, g.x_bytes, 0x00020000);
+  const uint32_t pos = tid % BK, group = tid / BK;
+  // dy: element (d, m0 + 8*group) of [depth][K]; chunk i lies 8*kGroupStep channels further
+  const uint32_t a_off = (pos * (uint32_t)g.K + m0 + group * 8) * 2u;
+  const uint32_t a_tile = BK * (uint32_t)g.K * 2u;  // bytes per tile
+  // x: this thread's position d = (image, p, q), carried from tile to tile
+  uint32_t d = t_begin * BK + pos, bp, bq, img_off;
+  {
+    const uint32_t n = d / PQ, pq = d - n * PQ;
+    bp = pq / g.Q;
+    bq = pq - bp * g.Q;
+    img_off = n * (uint32_t)g.H * g.W * (uint32_t)g.C * 2u;
   }
-#pragma unroll
-  for (int i = 0; i < kBChunks; ++i) {
-    b_pos[i] = (tid + kThreads * i) % BK;
-    split(t_begin * BK + b_pos[i], bn[i], bp[i], bq[i]);
-  }
-  auto advance = [&](uint32_t& n, uint32_t& p, uint32_t& q) {  // position += BK
-    q += BK;
-    while (q >= (uint32_t)g.Q) {
-      q -= g.Q;
-      ++p;
-    }
-    while (p >= (uint32_t)g.P) {
-      p -= g.P;
-      ++n;
-    }
-  };
+  const uint32_t kq = BK / (uint32_t)g.Q, rq = BK - kq * g.Q;
+  const uint32_t img_bytes = (uint32_t)g.H * g.W * (uint32_t)g.C * 2u;
+  const uint32_t b_chan = (c0 + group * 8) * 2u;
 
-  uint4_t ra[kAChunks], rb[kBChunks];
-  bool ra_ok[kAChunks], rb_ok[kBChunks];
-  auto fetch = [&](uint32_t d0) {
-#pragma unroll
-    for (int i = 0; i < kAChunks; ++i) {
-      const int kc = (tid + kThreads * i) / BK;
-      ra_ok[i] = d0 + a_pos[i] < g.depth;
-      const uint32_t e = ra_ok[i] ? ((an[i] * g.P + ap[i]) * (uint32_t)g.Q + aq[i]) * (uint32_t)g.K + m0 + kc * 8 : 0u;
-      ra[i] = *reinterpret_cast<const uint4_t*>(dy + e);
-      advance(an[i], ap[i], aq[i]);
-    }
-#pragma unroll
-    for (int i = 0; i < kBChunks; ++i) {
-      const int cc = (tid + kThreads * i) / BK;
-      const int hh = (int)bp[i] * g.sH + dh, ww = (int)bq[i] * g.sW + dw;
-      rb_ok[i] = d0 + b_pos[i] < g.depth && (unsigned)hh < (unsigned)g.H && (unsigned)ww < (unsigned)g.W;
-      const uint32_t e = rb_ok[i] ? ((bn[i] * g.H + hh) * (uint32_t)g.W + ww) * (uint32_t)g.C + c0 + cc * 8 : 0u;
-      rb[i] = *reinterpret_cast<const uint4_t*>(x + e);
-      advance(bn[i], bp[i], bq[i]);
-    }
-  };
-  // Transposing store: a chunk holds 8 channels of one position, LDS wants positions
-  // innermost.  Neighbouring lanes hold neighbouring positions, so a lane pair first swaps
-  // halves (DPP): the even lane ends up with channel 2j of both positions, the odd lane with
-  // channel 2j+1, and each writes 4 full dwords instead of 8 two-byte pieces.
-  const bool odd = tid & 1;
-  auto scatter = [&](bf16_t (*dstp)[LDK], int group, uint32_t pos, const uint4_t& v, bool ok) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const uint32_t own = ok ? v[j] : 0u;
-      const uint32_t other = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)own, 0xB1, 0xF, 0xF, true);
-      const uint32_t word = odd ? ((other >> 16) | (own & 0xFFFF0000u))
-                                : ((own & 0xFFFFu) | (other << 16));
-      *reinterpret_cast<uint32_t*>(&dstp[group * 8 + 2 * j + (odd ? 1 : 0)][pos & ~1u]) = word;
-    }
-  };
-  auto stage = [&](int buf) {
+  uint32_t tile = t_begin;  // next tile to fetch (uniform)
+  auto fetch = [&](uint4_t (&ra)[kAChunks], uint4_t (&rb)[kBChunks]) {
+    const uint32_t a_so = tile * a_tile;
 #pragma unroll
     for (int i = 0; i < kAChunks; ++i)
-      scatter(lds_a[buf], (tid + kThreads * i) / BK, a_pos[i], ra[i], ra_ok[i]);
+      ra[i] = __builtin_amdgcn_raw_buffer_load_b128(dy_buf, a_off + i * (8 * kGroupStep * 2), a_so, 0);
+    const int hh = (int)__umul24(bp, (uint32_t)g.sH) + dh, ww = (int)__umul24(bq, (uint32_t)g.sW) + dw;
+    const bool ok = d < g.depth && (unsigned)hh < (unsigned)g.H && (unsigned)ww < (unsigned)g.W;
+    const uint32_t pix = __umul24((uint32_t)hh, (uint32_t)g.W) + (uint32_t)ww;
+    const uint32_t b_off = ok ? img_off + pix * (uint32_t)g.C * 2u + b_chan : kBeyond;
 #pragma unroll
     for (int i = 0; i < kBChunks; ++i)
-      scatter(lds_b[buf], (tid + kThreads * i) / BK, b_pos[i], rb[i], rb_ok[i]);
+      rb[i] = __builtin_amdgcn_raw_buffer_load_b128(x_buf, b_off + i * (8 * kGroupStep * 2), 0, 0);
+    // next tile: position += BK
+    ++tile;
+    d += BK;
+    bq += rq;
+    bp += kq;
+    if (bq >= (uint32_t)g.Q) {
+      bq -= g.Q;
+      ++bp;
+    }
+    while (bp >= (uint32_t)g.P) {
+      bp -= g.P;
+      img_off += img_bytes;
+    }
+  };
+  // Transposing store of one chunk (8 channels of position `pos`): lane pairs hold positions
+  // 2j and 2j+1; after the swap the even lane owns the even channels of both positions, the
+  // odd lane the odd channels, each as whole dwords [channel][pos & ~1].
+  const bool odd = tid & 1;
+  const uint32_t sel = odd ? 0x03020706u : 0x05040100u;  // byte picks of (neighbour, own)
+  auto scatter = [&](bf16_t (*dstp)[LDK], int grp, const uint4_t& v) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t own = v[j];
+      const uint32_t other = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)own, 0xB1, 0xF, 0xF, true);
+      const uint32_t word = __builtin_amdgcn_perm(other, own, sel);
+      *reinterpret_cast<uint32_t*>(&dstp[grp * 8 + 2 * j + (odd ? 1 : 0)][pos & ~1u]) = word;
+    }
+  };
+  auto stage = [&](int buf, const uint4_t (&ra)[kAChunks], const uint4_t (&rb)[kBChunks]) {
+#pragma unroll
+    for (int i = 0; i < kAChunks; ++i) scatter(lds_a[buf], (int)group + kGroupStep * i, ra[i]);
+#pragma unroll
+    for (int i = 0; i < kBChunks; ++i) scatter(lds_b[buf], (int)group + kGroupStep * i, rb[i]);
   };
 
   float16_t acc[TM][TN];
@@ -411,16 +415,26 @@ __global__ __launch_bounds__(kThreads) void wgrad_bf16_kernel(const WGradH g,
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
   if (t_begin < t_end) {
-    fetch(t_begin * BK);
-    stage(0);
+    const uint32_t ntiles = t_end - t_begin;
+    uint4_t ra0[kAChunks], rb0[kBChunks], ra1[kAChunks], rb1[kBChunks];
+    fetch(ra0, rb0);
+    if (ntiles > 1) fetch(ra1, rb1);
+    stage(0, ra0, rb0);
     __syncthreads();
-    for (uint32_t kt = t_begin; kt < t_end; ++kt) {
-      const int buf = (kt - t_begin) & 1;
-      if (kt + 1 < t_end) fetch((kt + 1) * BK);
-      mma_tile<TM, TN, BMW, BNW>(lds_a[buf], lds_b[buf], wm, wn, lane, acc);
-      if (kt + 1 < t_end) stage(buf ^ 1);
+    for (uint32_t kt = 0; kt + 1 < ntiles; kt += 2) {
+      // tile kt is in LDS buffer 0, tile kt+1 in flight in set 1
+      if (kt + 2 < ntiles) fetch(ra0, rb0);
+      mma_tile<TM, TN, BMW, BNW>(lds_a[0], lds_b[0], wm, wn, lane, acc);
+      stage(1, ra1, rb1);
+      __syncthreads();
+      // tile kt+1 is in LDS buffer 1, tile kt+2 in flight in set 0
+      if (kt + 3 < ntiles) fetch(ra1, rb1);
+      mma_tile<TM, TN, BMW, BNW>(lds_a[1], lds_b[1], wm, wn, lane, acc);
+      if (kt + 2 < ntiles) stage(0, ra0, rb0);
       __syncthreads();
     }
+    // an odd number of tiles: the last one was staged into buffer 0
+    if (ntiles & 1) mma_tile<TM, TN, BMW, BNW>(lds_a[0], lds_b[0], wm, wn, lane, acc);
   }
 
   const size_t row_len = (size_t)g.T * g.C;
@@ -649,6 +663,12 @@ int mn_conv16_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, void
   q.dH = g->dH;
   q.dW = g->dW;
   q.depth = (uint32_t)((long long)g->N * g->P * g->Q);
+  // the kernel addresses both tensors through buffer descriptors with byte offsets below 2^31
+  const unsigned long long dy_bytes = (unsigned long long)q.depth * g->K * 2ull;
+  const unsigned long long x_bytes = (unsigned long long)g->N * g->H * g->W * g->C * 2ull;
+  if (dy_bytes >= (1ull << 31) || x_bytes >= (1ull << 31)) return MN_EUNSUPPORTED;
+  q.dy_bytes = (uint32_t)dy_bytes;
+  q.x_bytes = (uint32_t)x_bytes;
   int splits, tps, bm, bn;
   wgrad16_split(g, &splits, &tps);
   wgrad16_tiles(g, &bm, &bn);
