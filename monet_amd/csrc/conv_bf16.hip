@@ -312,8 +312,11 @@ struct WGradH {
 //  * transposing store: a lane pair swaps halves (DPP) and one byte-permute builds the dword
 //    of (channel, two positions): 2 vector instructions per 4-byte LDS store, no masks;
 //  * two register sets keep the loads of tile t+2 in flight while tile t is multiplied.
+// (3 waves per SIMD: the register allocator then keeps the accumulators in the unified file
+// instead of 166 + 64 registers, which would leave room for two)
 template <int BMW, int BNW>
-__global__ __launch_bounds__(kThreads) void wgrad_bf16_kernel(const WGradH g,
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))) void wgrad_bf16_kernel(
+    const WGradH g,
                                                               const bf16_t* __restrict__ dy,
                                                               const bf16_t* __restrict__ x,
                                                               void* __restrict__ out) {
