@@ -859,12 +859,11 @@ __global__ __launch_bounds__(kThreads) void wgrad_rows_kernel(const WGrad g,
   // depth position of this thread's float4 and the byte offsets that follow it
   uint32_t vd = t_begin * DEPTH + 4 * chunk;
   uint32_t vpq, a_off, bv_off = 0;
-  const uint32_t a_safe = (uint32_t)(m0 + vrow0) * PQ4, bv_safe = (c0 + vrow0) * PQ4;
   {
     const uint32_t n = vd / PQ;
     vpq = vd - n * PQ;
-    a_off = (n * (uint32_t)g.K * PQ + vpq) * 4u + a_safe;
-    if (VECB) bv_off = (n * (uint32_t)g.C * PQ + vpq) * 4u + bv_safe;
+    a_off = (n * (uint32_t)g.K * PQ + vpq) * 4u + (uint32_t)(m0 + vrow0) * PQ4;
+    if (VECB) bv_off = (n * (uint32_t)g.C * PQ + vpq) * 4u + (c0 + vrow0) * PQ4;
   }
   const uint32_t a_wrap = (uint32_t)(g.K - 1) * PQ4, bv_wrap = (uint32_t)(g.C - 1) * PQ4;
   // (p, q) of this thread's gathered element, and the byte offset of its image
@@ -875,17 +874,14 @@ __global__ __launch_bounds__(kThreads) void wgrad_rows_kernel(const WGrad g,
   const uint32_t chw4 = (uint32_t)g.C * HW4;
   const uint32_t b_row0 = (c0 + row0) * HW4 + (uint32_t)((dh * g.W + dw) * 4), b_step = kStep * HW4;
   uint32_t as_off = 0;  // scalar dy loader (!VECA): byte offset of (image, pixel, row m0 + row0)
-  const uint32_t as_safe = (uint32_t)(m0 + row0) * PQ4;
   if (!VECB) {
     const uint32_t n = bd / PQ, pq = bd - n * PQ;
     bp = pq / g.Q;
     bq = pq - bp * g.Q;
     img_off = n * chw4;
-    as_off = (n * (uint32_t)g.K * PQ + pq) * 4u + as_safe;
+    as_off = (n * (uint32_t)g.K * PQ + pq) * 4u + (uint32_t)(m0 + row0) * PQ4;
   }
 
-  const char* dyp = reinterpret_cast<const char*>(dy);
-  const char* xp = reinterpret_cast<const char*>(x);
   // Both tensors are read through buffer descriptors: the per-thread part of an address is one
   // 32-bit byte offset, the row part the load's scalar offset, and an element that is not to
   // be read (beyond the reduction, outside the window) gets an offset past the buffer and
