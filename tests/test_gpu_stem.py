@@ -39,7 +39,8 @@ def test_stem_block(cuda, combo):
     g64 = torch.ones(64, dtype=torch.float64, requires_grad=True)
     b64 = torch.zeros(64, dtype=torch.float64, requires_grad=True)
     rm64, rv64 = torch.zeros(64, dtype=torch.float64), torch.ones(64, dtype=torch.float64)
-    y64 = F.batch_norm(F.conv2d(x64, w64, None, 2, 3), rm64, rv64, g64, b64, True, 0.1, 1e-5)
+    c64 = F.conv2d(x64, w64, None, 2, 3)
+    y64 = F.batch_norm(c64, rm64, rv64, g64, b64, True, 0.1, 1e-5)
     z64, zi64 = F.max_pool2d(F.relu(y64), 3, 2, 1, return_indices=True)
 
     # ---- GPU forward through the operator classes
@@ -80,7 +81,11 @@ def test_stem_block(cuda, combo):
 
     # ---- forward values and decisions
     assert rel(z, z64.detach()) < 1e-5
-    assert rel(rm, rm64) < 1e-5 and rel(rv, rv64) < 1e-5
+    # the batch means are ~0.003 standard deviations of the data (100k samples per channel), so the
+    # running mean is held to 1e-6 of what it is a mean OF (momentum * the data's spread) rather
+    # than to 1e-5 of its own near-zero value
+    spread = 0.1 * float(c64.detach().std())
+    assert float((rm.double().cpu() - rm64).abs().max()) < 1e-6 * spread and rel(rv, rv64) < 1e-5
     assert float((sign != (y64.detach() > 0)).double().mean()) < 1e-5
     idx_gpu = O.unpack_nibbles(idx_packed, z64.numel()).reshape(z64.shape)
     h, wc = zi64.numpy() // 112, zi64.numpy() % 112
