@@ -1,0 +1,153 @@
+"""GPU checks at the full benchmark sizes (ResNet-50 shapes at batch 184), where the CPU
+oracle would take minutes: size-independent properties of each operator, with float64
+accumulation on the GPU (plain torch reductions) as the only arithmetic besides the kernels
+under test.
+
+* BatchNorm backward: sum(dx) = 0 and sum(dx * xhat) = 0 per channel (the gradient is
+  orthogonal to the two statistics it was centred by), dbeta = sum(dy), dgamma = sum(dy * xhat),
+  and the from-output form equals the from-input form.
+* ReLU mask: the packed mask unpacks to x > 0, backward is dy where the bit is set and 0
+  elsewhere, bit for bit.
+* Max pool: gathering x at the stored window indices gives y back; backward conserves the sum
+  of every plane and puts gradient only where an index points.
+* Convolution (every variant, fp32 and bf16): the three directions are adjoint to each other,
+  <conv(x, w), dy> = <x, bwd_data(dy, w)> = <w, bwd_weight(dy, x)>, and the forward is linear.
+"""
+import pytest
+import torch
+
+from monet_amd.lm_ops import bn as bn_ops
+from monet_amd.lm_ops import conv as conv_ops
+from monet_amd.lm_ops import pack as pk
+from monet_amd.lm_ops import pool as pool_ops
+from monet_amd.lm_ops import relu as relu_ops
+
+pytestmark = pytest.mark.gpu
+
+BIG = (184, 256, 56, 56)       # BatchNorm / ReLU shape of the benchmark
+POOL_IN = (184, 64, 112, 112)  # max-pool input of the benchmark
+LAYER3 = ((184, 256, 14, 14), (256, 256, 3, 3))
+
+
+def _randn(shape, device, seed):
+    g = torch.Generator(device=device)
+    g.manual_seed(seed)
+    return torch.randn(shape, device=device, generator=g)
+
+
+def _dot(a, b):
+    return float((a.double() * b.double()).sum())
+
+
+def test_batch_norm_backward_invariants_at_full_size(cuda):
+    x = _randn(BIG, cuda, 1) * 1.5 + 0.3
+    dy = _randn(BIG, cuda, 2)
+    C = BIG[1]
+    gamma = torch.rand(C, device=cuda) + 0.5
+    beta = torch.randn(C, device=cuda) * 0.1
+    y, mean, invstd = bn_ops.bn_forward_train(x, gamma, beta, None, None, 0.1, 1e-5)
+    dx_y, dg_y, db_y = bn_ops.bn_backward_from_output(dy.clone(), y, gamma, beta, invstd)
+    dx_x, dg_x, db_x = bn_ops.bn_backward_from_input(dy.clone(), x, gamma, mean, invstd)
+
+    M = x.numel() // C
+    xhat = (x.double() - mean.double().view(1, C, 1, 1)) * invstd.double().view(1, C, 1, 1)
+    # the statistics the forward saved are those of x (float64 reductions of the same data)
+    assert float((xhat.sum((0, 2, 3)) / M).abs().max()) < 1e-5
+    assert float(((xhat * xhat).sum((0, 2, 3)) / M - 1).abs().max()) < 1e-4   # eps = 1e-5 inside
+    # sums of M = 577 024 terms that should cancel: held to 1e-5 of sqrt(M) * the largest term
+    xh_max = float(xhat.abs().max())
+    for name, dx in (("from output", dx_y), ("from input", dx_x)):
+        s0 = dx.double().sum((0, 2, 3))
+        s1 = (dx.double() * xhat).sum((0, 2, 3))
+        dx_max = float(dx.abs().max())
+        assert float(s0.abs().max()) < 1e-5 * M ** 0.5 * dx_max, name
+        assert float(s1.abs().max()) < 1e-5 * M ** 0.5 * dx_max * xh_max, name
+    exp_db = dy.double().sum((0, 2, 3))
+    exp_dg = (dy.double() * xhat).sum((0, 2, 3))
+    for db, dg in ((db_y, dg_y), (db_x, dg_x)):
+        assert float((db.double() - exp_db).abs().max()) < 3e-5 * M ** 0.5
+        assert float((dg.double() - exp_dg).abs().max()) < 3e-5 * M ** 0.5
+    # the two forms are the same function of (dy, x): 1e-5 of the gradient's scale (the
+    # from-output form recovers xhat from y, one rounding more)
+    tol = 1e-5 * float(dx_x.abs().max())
+    assert float((dx_y - dx_x).abs().max()) < 4 * tol
+
+
+def test_relu_mask_round_trip_at_full_size(cuda):
+    x = _randn(BIG, cuda, 3)
+    dy = _randn(BIG, cuda, 4)
+    y, mask = relu_ops.relu_forward_with_mask(x)
+    positive = x > 0
+    assert torch.equal(y, torch.where(positive, x, torch.zeros_like(x)))
+    assert mask.numel() == (x.numel() + 7) // 8
+    assert torch.equal(pk.unpack(mask, x.numel()).view(x.shape), positive)
+    dx = relu_ops.relu_backward_from_mask(dy.clone(), mask)
+    assert torch.equal(dx, torch.where(positive, dy, torch.zeros_like(dy)))
+    dx2 = relu_ops.relu_backward_from_ref(dy.clone(), y)
+    assert torch.equal(dx2, dx)
+
+
+def test_max_pool_indices_at_full_size(cuda):
+    x = _randn(POOL_IN, cuda, 5)
+    y, idx4, geo = pool_ops.max_pool2d_with_packed_indices(x, [3, 3], [2, 2], [1, 1], [1, 1], False)
+    N, C, H, W = POOL_IN
+    PH, PW = H // 2, W // 2
+    assert list(y.shape) == [N, C, PH, PW]
+    assert torch.equal(y, torch.max_pool2d(x, 3, 2, 1))
+    # window-relative index -> input coordinate -> the element there is the maximum
+    idx = pk.unpack_two(idx4, y.numel()).view(N, C, PH, PW).long()
+    ph = torch.arange(PH, device=cuda).view(1, 1, PH, 1)
+    pw = torch.arange(PW, device=cuda).view(1, 1, 1, PW)
+    h = 2 * ph - 1 + idx // 3
+    w = 2 * pw - 1 + idx % 3
+    assert bool(((h >= 0) & (h < H) & (w >= 0) & (w < W)).all())
+    picked = x.view(N, C, H * W).gather(2, (h * W + w).view(N, C, PH * PW)).view(N, C, PH, PW)
+    assert torch.equal(picked, y)
+    # backward: every plane keeps its sum, and gradient lands only on picked elements
+    dy = _randn((N, C, PH, PW), cuda, 6)
+    dx = pool_ops.max_pool2d_backward_from_packed_indices(dy, idx4, geo, POOL_IN)
+    sums_in, sums_out = dx.double().sum((2, 3)), dy.double().sum((2, 3))
+    assert float((sums_in - sums_out).abs().max()) < 1e-5 * (PH * PW) ** 0.5
+    hit = torch.zeros(N, C, H * W, device=cuda, dtype=torch.bool)
+    hit.scatter_(2, (h * W + w).view(N, C, PH * PW), True)
+    assert not bool((dx.view(N, C, H * W) != 0)[~hit].any())
+    ref = torch.zeros(N, C, H * W, device=cuda, dtype=torch.float64)
+    ref.scatter_add_(2, (h * W + w).view(N, C, PH * PW), dy.double().view(N, C, PH * PW))
+    assert float((dx.double().view(N, C, H * W) - ref).abs().max()) < 1e-5
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 1e-2)])
+def test_convolution_directions_are_adjoint_at_full_size(cuda, dtype, tol):
+    xs, ws = LAYER3
+    x = _randn(xs, cuda, 7)
+    w = _randn(ws, cuda, 8) * (2.0 / (ws[0] * 9)) ** 0.5
+    if dtype == torch.bfloat16:
+        x = x.to(dtype).contiguous(memory_format=torch.channels_last)
+        w = w.to(dtype).contiguous(memory_format=torch.channels_last)
+    dy = None
+    for v in range(conv_ops.n_fwd_algos()):
+        y = conv_ops.conv_forward(x, w, None, 1, 1, 1, 1, v)
+        if dy is None:
+            dy = _randn(tuple(y.shape), cuda, 9)
+            if dtype == torch.bfloat16:
+                dy = dy.to(dtype).contiguous(memory_format=torch.channels_last)
+        lhs = _dot(y, dy)
+        # <conv(x, w), dy> is a sum of 9e6 products of independent values: its natural size is
+        # sqrt(n) * rms(y) * rms(dy) (a wrong operand, e.g. transposed weights, is off by ~0.2 of it)
+        scale = (y.numel() ** 0.5) * float(y.float().pow(2).mean().sqrt()) * float(dy.float().pow(2).mean().sqrt())
+        for vd in range(conv_ops.n_bwd_ip_algos()):
+            dx = conv_ops.conv_backward_input(list(xs), dy, w, 1, 1, 1, 1, vd)
+            assert abs(lhs - _dot(dx, x)) < tol * scale, (v, vd)
+        for vw in range(conv_ops.n_bwd_wt_algos()):
+            dw = conv_ops.conv_backward_weight(list(ws), dy, x, 1, 1, 1, 1, vw)
+            assert abs(lhs - _dot(dw, w)) < tol * scale, (v, vw)
+        # linearity of the forward in x (exact up to rounding of the two results)
+        x2 = _randn(xs, cuda, 10)
+        if dtype == torch.bfloat16:
+            x2 = x2.to(dtype).contiguous(memory_format=torch.channels_last)
+        y2 = conv_ops.conv_forward(x2, w, None, 1, 1, 1, 1, v)
+        ys = conv_ops.conv_forward((x.float() + x2.float()).to(dtype).contiguous(
+            memory_format=torch.channels_last if dtype == torch.bfloat16 else torch.contiguous_format),
+            w, None, 1, 1, 1, 1, v)
+        lin_tol = (4 if dtype == torch.float32 else 3) * tol * float(ys.float().abs().max())
+        assert float((ys.float() - (y.float() + y2.float())).abs().max()) < lin_tol, v
