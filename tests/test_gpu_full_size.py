@@ -151,3 +151,48 @@ def test_convolution_directions_are_adjoint_at_full_size(cuda, dtype, tol):
             w, None, 1, 1, 1, 1, v)
         lin_tol = (4 if dtype == torch.float32 else 3) * tol * float(ys.float().abs().max())
         assert float((ys.float() - (y.float() + y2.float())).abs().max()) < lin_tol, v
+
+
+@pytest.mark.parametrize("mode", ["inplace_conv_multiway_newnode", "fused_inplace_conv_multiway_newnode"])
+def test_resnet50_batch_184_under_the_committed_10gb_schedule(cuda, mode):
+    """The headline configuration end to end: `MONeTWrapper` with the schedule in data/ against
+    stock autograd on the same weights and batch.  Losses agree to 1e-5; the peak stays within
+    the budget plus allocator rounding; the classifier's gradients (what every earlier layer's
+    gradient flows from, and well conditioned) agree to 1e-3 of their scale - deep-layer
+    gradients of a random-init ResNet-50 differ by percents between ANY two fp32 summation
+    orders, which the float64-referenced schedule test covers on a smaller network."""
+    import os
+    from monet_amd.models import build_model
+    from monet_amd.monet_wrapper import MONeTWrapper
+    sol = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "data",
+                       "solution_resnet50_184_%s_10.00.pkl" % mode)
+    torch.manual_seed(0)
+    model = build_model("resnet50")[0]
+    x = _randn((184, 3, 224, 224), cuda, 11)
+    labels = torch.randint(0, 1000, (184,), device=cuda, generator=torch.Generator(device=cuda).manual_seed(12))
+    wrapped = MONeTWrapper(model, sol, (3, 224, 224)).to(cuda)
+    wrapped.train()
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    base = torch.cuda.memory_allocated()
+    loss = torch.nn.functional.cross_entropy(wrapped(x), labels)
+    loss.backward()
+    torch.cuda.synchronize()
+    peak_mb = (torch.cuda.max_memory_allocated() - base) / 2 ** 20
+    got = {k: p.grad.detach().clone() for k, p in wrapped.model.named_parameters()}
+    assert all(g is not None and bool(torch.isfinite(g).all()) for g in got.values())
+    # activations + workspaces of the step above what was resident before it (weights, batch)
+    assert peak_mb < 10 * 1024 * 1.02, peak_mb
+
+    ref = build_model("resnet50")[0]
+    ref.load_state_dict({k: v for k, v in wrapped.model.state_dict().items()})
+    ref = ref.to(cuda).train()
+    # the wrapped step has already moved the BatchNorm running statistics of ITS copy; the
+    # loss and gradients do not depend on them in training mode
+    ref_loss = torch.nn.functional.cross_entropy(ref(x), labels)
+    ref_loss.backward()
+    la, lb = float(loss.detach()), float(ref_loss.detach())
+    assert abs(la - lb) < 1e-5 * max(1.0, abs(lb))
+    for name in ("fc.weight", "fc.bias"):
+        r = dict(ref.named_parameters())[name].grad
+        assert float((got[name] - r).abs().max()) < 1e-3 * float(r.abs().max()), name
