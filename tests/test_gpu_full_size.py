@@ -196,3 +196,4 @@ def test_resnet50_batch_184_under_the_committed_10gb_schedule(cuda, mode):
     for name in ("fc.weight", "fc.bias"):
         r = dict(ref.named_parameters())[name].grad
         assert float((got[name] - r).abs().max()) < 1e-3 * float(r.abs().max()), name
+
