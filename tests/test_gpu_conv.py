@@ -33,6 +33,9 @@ CASES = [
     ((5, 128, 7, 7), (128, 128, 3, 3), 1, 1, 1),       # 49-pixel images: no 16-byte alignment along the depth
     ((5, 128, 7, 7), (256, 128, 1, 1), 1, 0, 1),       # the same, 1x1
     ((3, 64, 9, 11), (64, 64, 3, 3), 1, 1, 1),         # 99 pixels, 64-channel tiles
+    ((2, 32, 13, 17), (48, 32, 3, 3), 2, (2, 1), 2),   # tap-major path with stride, dilation, uneven padding
+    ((2, 64, 12, 12), (64, 64, 5, 5), 1, 2, 1),        # 25 taps, windows hanging over every border
+    ((1, 128, 6, 10), (128, 128, 3, 3), (1, 2), (1, 0), (1, 1)),  # stride on one axis only
 ]
 
 
