@@ -144,7 +144,7 @@ __device__ __forceinline__ void split_column(const Gather& g, uint32_t c, uint32
 // floats (a multiple of 128, zero padded), so a k-tile of A is BK contiguous
 // row pieces: one 16-byte load per lane and row piece, no masks, and 8 cache
 // lines per wavefront load instead of the ~20 a strided gather touches.
-// PACKED kernels fetch through raw buffer descriptors: a thread's byte offset is fixed for a
+// FAST kernels fetch through raw buffer descriptors: a thread's byte offset is fixed for a
 // whole tap, an element outside the window or the tensor gets an offset beyond the buffer
 // and reads as zero (no masks when staging), and the per-tile part of an address is the
 // scalar offset of the load: no vector arithmetic per tile.  Both tensors must be < 2 GB.
@@ -205,7 +205,9 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
     for (int i = 0; i < kARows; ++i) {
       const int m = m0 + arow0 + kAStep * i;
       const bool ok = m < g.M;
-      am_b[i] = ok ? (uint32_t)(((long long)m * g.lda + (FAST ? (long long)ak * g.cha : 0)) * 4) : 0u;
+      // tap-major path: rows past M get an offset beyond the buffer and read as zero
+      am_b[i] = ok ? (uint32_t)(((long long)m * g.lda + (FAST ? (long long)ak * g.cha : 0)) * 4)
+                   : (FAST ? kBeyond : 0u);
       am_ok |= (ok ? 1u : 0u) << i;
     }
   }
@@ -252,25 +254,20 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
   bool tap_in = false;
   bool b_in = false;  // tap_in at the time of the last fetch: what stage() masks with
   const __amdgpu_buffer_rsrc_t src_buf = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<float*>(src), 0, PACKED ? g.src_bytes : 0u, 0x00020000);
+      const_cast<float*>(src), 0, FAST ? g.src_bytes : 0u, 0x00020000);
   const __amdgpu_buffer_rsrc_t a_buf = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<float*>(a), 0, PACKED ? g.a_bytes : 0u, 0x00020000);
+      const_cast<float*>(a), 0, FAST ? g.a_bytes : 0u, 0x00020000);
   auto enter_tap = [&](int t) {  // t uniform
     const int dh = tdh[t], dw = tdw[t];
     const int hh = ohs + dh, ww = ows + dw;
     tap_in = col_ok && (unsigned)hh < (unsigned)g.Hs && (unsigned)ww < (unsigned)g.Ws;
-    tap_b = tap_in ? pix_b + (uint32_t)((dh * g.Ws + dw) * 4) : (PACKED ? kBeyond : brow0 * plane_b);
+    tap_b = tap_in ? pix_b + (uint32_t)((dh * g.Ws + dw) * 4) : kBeyond;
     const int ao = __builtin_amdgcn_readfirstlane(taoff[t]);  // uniform: keep it in a scalar register
     tap_a = PACKED ? (uint32_t)((long long)ao * g.Cs * g.lda * 4) : (uint32_t)(ao * 4);
   };
-  // Only issues loads: masking happens in stage(), after the multiply of the current
-  // tile, so the loads stay in flight behind the matrix instructions.  The per-tile part of
-  // every address is uniform (c0), so it goes into the base pointer and the per-thread
-  // offsets stay put for a whole tap.
-  // uniform bases of the rows one thread gathers (row i is channel brow0 + kBStep*i of the tile)
-  const char* b_rows[kBRows];
-#pragma unroll
-  for (int i = 0; i < kBRows; ++i) b_rows[i] = sp + (size_t)(kBStep * i) * plane_b;
+  // Only issues loads, so they stay in flight behind the matrix instructions of the current
+  // tile.  The per-tile part of every address is uniform (c0) and goes into the scalar offset
+  // of the load; the per-thread offsets stay put for a whole tap.
   auto fetch_fast = [&](int c0) {  // c0 uniform
     b_in = tap_in;
     if (POINT) {
@@ -278,15 +275,11 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
 #pragma unroll
       for (int i = 0; i < kB4; ++i)
         rb4[i] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(src_buf, bp_b[i], so, 0));
-    } else if (PACKED) {
+    } else {
 #pragma unroll
       for (int i = 0; i < kBRows; ++i)
         rb[i] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(
             src_buf, tap_b, (uint32_t)(c0 + kBStep * i) * plane_b, 0));
-    } else {
-      const uint32_t off = tap_b + (uint32_t)c0 * plane_b;
-#pragma unroll
-      for (int i = 0; i < kBRows; ++i) rb[i] = *reinterpret_cast<const float*>(b_rows[i] + off);
     }
     if (PACKED) {
       const uint32_t so = tap_a + (uint32_t)c0 * (uint32_t)g.lda * 4u;
@@ -294,9 +287,10 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
       for (int i = 0; i < kA4; ++i)
         ra4[i] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(a_buf, ap_b[i], so, 0));
     } else {
-      const char* apc = ap + ((size_t)tap_a + (size_t)c0 * g.cha * 4);
+      const uint32_t so = tap_a + (uint32_t)c0 * (uint32_t)g.cha * 4u;
 #pragma unroll
-      for (int i = 0; i < kARows; ++i) ra[i] = *reinterpret_cast<const float*>(apc + am_b[i]);
+      for (int i = 0; i < kARows; ++i)
+        ra[i] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(a_buf, am_b[i], so, 0));
     }
   };
   auto fetch_any = [&](int k0) {
@@ -339,8 +333,8 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
     } else {
 #pragma unroll
       for (int i = 0; i < kBRows; ++i) {
-        // PACKED: what lies outside the window was fetched as zero already
-        const bool in = PACKED ? true : (FAST ? b_in : (((b_ok >> i) & 1u) != 0));
+        // tap-major: what lies outside the window was fetched as zero already
+        const bool in = FAST ? true : (((b_ok >> i) & 1u) != 0);
         lds_b[buf][brow0 + kBStep * i][bcol] = in ? rb[i] : 0.f;
       }
     }
@@ -353,7 +347,7 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
     } else {
 #pragma unroll
       for (int i = 0; i < kARows; ++i)
-        lds_a[buf][ak][arow0 + kAStep * i] = (a_ok && ((am_ok >> i) & 1u)) ? ra[i] : 0.f;
+        lds_a[buf][ak][arow0 + kAStep * i] = (FAST || (a_ok && ((am_ok >> i) & 1u))) ? ra[i] : 0.f;
     }
   };
 
@@ -1085,6 +1079,11 @@ __global__ __launch_bounds__(kThreads) void pack_weights_kernel(const float* __r
 static long long packed_rows(long long M) { return (M + 127) / 128 * 128; }
 // The repacked-weight kernels address both operands through buffer descriptors with byte
 // offsets below 2^31; larger tensors run variant 1 with the variant-0 kernel.
+// Bytes of the weight tensor, or 0 if it cannot be addressed with 31-bit byte offsets.
+static uint32_t weight_bytes(const mn_conv2d* g) {
+  const unsigned long long b = (unsigned long long)g->K * g->C * g->R * g->S * sizeof(float);
+  return b < (1ull << 31) ? (uint32_t)b : 0u;
+}
 static bool buffers_fit(size_t src_floats, size_t a_floats) {
   return src_floats < (1ull << 29) && a_floats < (1ull << 29);
 }
@@ -1129,7 +1128,12 @@ static int pick_tile(long long M, long long ncols, bool fast, bool packed) {
   return M <= 64 ? 1 : 2;
 }
 
-static bool fast_path(const Gather& g) { return g.T > 0 && g.Cs % BK == 0; }
+// The tap-major kernels address both operands through buffer descriptors with byte offsets
+// below 2^31 (g.a_bytes is set by the callers, 0 if the operand is too large).
+static bool fast_path(const Gather& g) {
+  const unsigned long long src_bytes = (unsigned long long)g.N * g.Cs * g.Hs * g.Ws * sizeof(float);
+  return g.T > 0 && g.Cs % BK == 0 && src_bytes < (1ull << 31) && g.a_bytes > 0 && g.a_bytes < (1u << 31);
+}
 
 template <class TL>
 static void launch_gather_t(const Gather& g, const float* a, const float* src, const float* bias,
@@ -1186,9 +1190,7 @@ static void launch_gather(Gather g, const float* a, const float* src, const floa
                           float* dst, hipStream_t s, bool packed = false, bool split_ok = false,
                           int tile = -1) {
   if (g.ncols == 0 || g.M == 0) return;
-  if (packed) {  // the callers have checked buffers_fit()
-    g.src_bytes = (uint32_t)((size_t)g.N * g.Cs * g.Hs * g.Ws * sizeof(float));
-  }
+  if (fast_path(g)) g.src_bytes = (uint32_t)((size_t)g.N * g.Cs * g.Hs * g.Ws * sizeof(float));
   g.divOHW = make_fastdiv((uint32_t)(g.OH * g.OW));
   g.divOW = make_fastdiv((uint32_t)g.OW);
   // multiplication by the reciprocal is exact while dividend * divisor < 2^32
@@ -1356,6 +1358,7 @@ int mn_conv_fwd(const mn_conv2d* g, const void* x, const void* w, const void* bi
     }
   hipStream_t s = mn_stream(stream);
   const float* a = (const float*)w;
+  q.a_bytes = weight_bytes(g);  // weights read in place
   // the repacked operand needs the tap-major path; other shapes run variant 1 like variant 0
   const bool packed = variant == 1 && fast_path(q) &&
                       buffers_fit((size_t)g->N * g->C * g->H * g->W, (size_t)q.T * q.Cs * packed_rows(q.M));
@@ -1387,7 +1390,7 @@ static int conv_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void
   if (dtype != MN_F32) return MN_EUNSUPPORTED;
   const int RS = g->R * g->S;
   const float* a = (const float*)w;
-  uint32_t a_bytes = 0;  // size of the repacked operand
+  uint32_t a_bytes = weight_bytes(g);  // size of the A operand: the weights, or their repacked copy
   long long lda = RS, cha = (long long)g->C * RS;  // read w[k][c][r][s] as A(c, k, rs)
   const bool packed = variant == 1 && g->K % BK == 0 &&
                       buffers_fit((size_t)g->N * g->K * g->P * g->Q, (size_t)RS * g->K * packed_rows(g->C));
