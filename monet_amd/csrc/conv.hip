@@ -117,6 +117,7 @@ struct Gather {
   int16_t dh[kMaxTaps], dw[kMaxTaps];
   int32_t aoff[kMaxTaps];
   int ksplit, tiles_per_split;  // split reduction (ksplit > 1): grid.z slices of k-tiles
+  int chunk;  // tap-major kernels: the reduction visits all taps of `chunk` channels, then the next block
   int accum;                    // add to what dst already holds instead of overwriting it
   uint32_t src_bytes, a_bytes;  // sizes of the source tensor and of the repacked A (PACKED)
   FastDiv divOHW, divOW;        // column -> (image, row, column) by multiplication ...
@@ -168,8 +169,24 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
   __shared__ int tdh[kMaxTaps], tdw[kMaxTaps], taoff[kMaxTaps];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / TL::WN, wn = wave % TL::WN;
-  const int m0 = blockIdx.y * BM;
-  const uint32_t n0 = blockIdx.x * BN;
+  uint32_t bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
+  {
+    // Workgroups are handed to the 8 XCDs round-robin in launch order.  The launch index is
+    // re-read so that each XCD works on a contiguous range of column tiles, with all row
+    // tiles of a column tile one after the other: the workgroups that gather the same pixels
+    // (other output channels, overlapping windows) then share one L2 instead of pulling them
+    // into several (strided 1x1, 256 -> 512 channels at batch 184: 0.71 -> 0.41 ms).
+    const uint32_t nxy = gridDim.x * gridDim.y, total = nxy * gridDim.z;
+    const uint32_t lin = bx + gridDim.x * (by + gridDim.y * bz);
+    const uint32_t xcd = lin & 7u, j = lin >> 3;
+    const uint32_t logical = xcd * (total >> 3) + min(xcd, total & 7u) + j;
+    bz = logical / nxy;
+    const uint32_t rem = logical - bz * nxy;
+    bx = rem / gridDim.y;
+    by = rem - bx * gridDim.y;
+  }
+  const int m0 = by * BM;
+  const uint32_t n0 = bx * BN;
   if (tid < g.T) {
     tdh[tid] = g.dh[tid];
     tdw[tid] = g.dw[tid];
@@ -362,24 +379,33 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
   // reduction range of this workgroup: all k-tiles, or slice blockIdx.z of them (split
   // reduction: the slices are added into a cleared output with atomics)
   const int all_tiles = (g.Kd + BK - 1) / BK;
-  const int kt_begin = g.ksplit > 1 ? (int)blockIdx.z * g.tiles_per_split : 0;
+  const int kt_begin = g.ksplit > 1 ? (int)bz * g.tiles_per_split : 0;
   const int ktiles = g.ksplit > 1 ? min(kt_begin + g.tiles_per_split, all_tiles) : all_tiles;
   if (kt_begin < ktiles) {
     int t = 0, c0 = 0;  // FAST: position of the tile being fetched
+    int c_lo = 0, c_hi = g.chunk;  // the block of channels the taps are cycled over
     if (FAST && kt_begin > 0) {
-      const int per_tap = g.Cs / BK;
-      t = kt_begin / per_tap;
-      c0 = (kt_begin - t * per_tap) * BK;
+      const int per_tap = g.chunk / BK, per_chunk = per_tap * g.T;
+      const int ch = kt_begin / per_chunk, r = kt_begin - ch * per_chunk;
+      c_lo = ch * g.chunk;
+      c_hi = c_lo + g.chunk;
+      t = r / per_tap;
+      c0 = c_lo + (r - t * per_tap) * BK;
     }
     if (FAST) enter_tap(t);
     auto fetch_next = [&](int kt) {
       if (FAST) {
         fetch_fast(c0);
         c0 += BK;
-        if (c0 == g.Cs) {
-          c0 = 0;
+        if (c0 == c_hi) {
           ++t;
-          if (t < g.T) enter_tap(t);
+          if (t == g.T) {
+            t = 0;
+            c_lo = c_hi;
+            c_hi += g.chunk;
+          }
+          c0 = c_lo;
+          if (c_lo < g.Cs) enter_tap(t);
         }
       } else {
         fetch_any(kt * BK);
@@ -403,7 +429,7 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
   // address is a per-thread byte offset plus a compile-time multiple of the plane size.
   const uint32_t plane4 = (uint32_t)g.DH * g.DW * 4u;
   char* dstb = reinterpret_cast<char*>(dst);
-  const bool add_bias = bias != nullptr && blockIdx.z == 0;
+  const bool add_bias = bias != nullptr && bz == 0;
   const int mbase = m0 + wm * (TL::TM * 32) + 4 * (lane >> 5);
   auto emit = [&](auto full_tag, auto how_tag) {
     constexpr bool kFull = decltype(full_tag)::value;
@@ -502,7 +528,7 @@ struct WGrad {
 template <int LANES, int ROWS>
 __device__ __forceinline__ void store_row_sums(float (&row_sum)[ROWS], float* __restrict__ db,
                                                const WGrad& g, int first_row, int row_step,
-                                               int depth_lane) {
+                                               int depth_lane, uint32_t split = blockIdx.z) {
 #pragma unroll
   for (int i = 0; i < ROWS; ++i) {
     float v = row_sum[i];
@@ -513,7 +539,7 @@ __device__ __forceinline__ void store_row_sums(float (&row_sum)[ROWS], float* __
       if (g.mode == 1)
         atomicAdd(db + m, v);
       else
-        db[(g.mode == 2 ? (size_t)blockIdx.z * g.K : 0) + m] = v;
+        db[(g.mode == 2 ? (size_t)split * g.K : 0) + m] = v;
     }
   }
 }
@@ -671,9 +697,10 @@ __global__ __launch_bounds__(kThreads) void wgrad_kernel(const WGrad g,
 template <class TL>
 __device__ __forceinline__ void store_tap_tile(const WGrad& g, float16_t (&acc)[TL::TM][TL::TN],
                                                float* __restrict__ out, int m0, uint32_t c0,
-                                               uint32_t tap, int wm, int wn, int lane) {
+                                               uint32_t tap, int wm, int wn, int lane,
+                                               uint32_t split = blockIdx.z) {
   float* base = out;
-  if (g.mode == 2) base += (size_t)blockIdx.z * g.K * g.ncols;
+  if (g.mode == 2) base += (size_t)split * g.K * g.ncols;
   const uint32_t RS = (uint32_t)g.R * g.S;
 #pragma unroll
   for (int nj = 0; nj < TL::TN; ++nj) {
@@ -829,17 +856,32 @@ __global__ __launch_bounds__(kThreads) void wgrad_rows_kernel(const WGrad g,
   auto swz = [](int row) { return (row / RP) & (CPR - 1); };  // chunk c of a row sits at c ^ swz(row)
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / TL::WN, wn = wave % TL::WN;
-  const int m0 = blockIdx.y * BM;
+  // Workgroups are handed to the 8 XCDs round-robin in launch order.  The launch index is
+  // re-read so that each XCD gets whole slices of the reduction: all the (tap, channel tile,
+  // row tile) workgroups that read the same positions of dy and x then share one L2 instead of
+  // pulling those positions into all eight (layer2 3x3 stride 2 at batch 184: 0.54 -> 0.41 ms).
+  uint32_t bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
+  {
+    const uint32_t nxy = gridDim.x * gridDim.y, total = nxy * gridDim.z;
+    const uint32_t lin = bx + gridDim.x * (by + gridDim.y * bz);
+    const uint32_t xcd = lin & 7u, j = lin >> 3;
+    const uint32_t logical = xcd * (total >> 3) + min(xcd, total & 7u) + j;
+    bz = logical / nxy;
+    const uint32_t rem = logical - bz * nxy;
+    by = rem / gridDim.x;
+    bx = rem - by * gridDim.x;
+  }
+  const int m0 = by * BM;
   const uint32_t ctiles = (uint32_t)g.C / BN;
-  const uint32_t tap = blockIdx.x / ctiles;
-  const uint32_t c0 = (blockIdx.x - tap * ctiles) * BN;
+  const uint32_t tap = bx / ctiles;
+  const uint32_t c0 = (bx - tap * ctiles) * BN;
   const uint32_t r_tap = g.divS.div(tap), s_tap = tap - r_tap * g.S;
   const int dh = (int)r_tap * g.dH - g.pH, dw = (int)s_tap * g.dW - g.pW;
   const uint32_t PQ = (uint32_t)g.P * g.Q, PQ4 = PQ * 4u;
   const uint32_t HW4 = (uint32_t)g.H * g.W * 4u;
 
   const uint32_t total_tiles = (g.depth + DEPTH - 1) / DEPTH;
-  const uint32_t t_begin = blockIdx.z * (g.tiles_per_split * (WBK / DEPTH));
+  const uint32_t t_begin = bz * (g.tiles_per_split * (WBK / DEPTH));
   const uint32_t t_end = min(t_begin + g.tiles_per_split * (WBK / DEPTH), total_tiles);
 
   // float4 loader: float4 number f = tid + kThreads*i of a tile is (row f / CPR, chunk f % CPR)
@@ -889,7 +931,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_rows_kernel(const WGrad g,
   float4_t ra4[VECA ? kA4 : 1], rb4[VECB ? kB4 : 1];
   float ra[VECA ? 1 : kRowsA], rb[VECB ? 1 : kRowsB];
   float row_sum[DB ? (VECA ? kA4 : kRowsA) : 1] = {};
-  const bool sums_rows = DB && blockIdx.x == 0;
+  const bool sums_rows = DB && bx == 0;
   bool a_ok = false, b_ok = false;
   auto fetch = [&]() {
     if (VECA) {
@@ -1031,12 +1073,12 @@ __global__ __launch_bounds__(kThreads) void wgrad_rows_kernel(const WGrad g,
   if constexpr (DB) {
     if (sums_rows) {
       if constexpr (VECA)
-        store_row_sums<CPR, kA4>(row_sum, db, g, m0 + vrow0, kRowsPass, chunk);
+        store_row_sums<CPR, kA4>(row_sum, db, g, m0 + vrow0, kRowsPass, chunk, bz);
       else
-        store_row_sums<DEPTH, kRowsA>(row_sum, db, g, m0 + row0, kStep, kdl);
+        store_row_sums<DEPTH, kRowsA>(row_sum, db, g, m0 + row0, kStep, kdl, bz);
     }
   }
-  store_tap_tile<TL>(g, acc, out, m0, c0, tap, wm, wn, lane);
+  store_tap_tile<TL>(g, acc, out, m0, c0, tap, wm, wn, lane, bz);
 }
 
 // dw[i] = sum over splits of partial[z][i], fixed order.
@@ -1200,6 +1242,15 @@ static void launch_gather(Gather g, const float* a, const float* src, const floa
 #endif
   if (tile < 0) tile = pick_tile(g.M, g.ncols, fast_path(g), packed);
   plan_split(g, tile, split_ok && packed);
+  // Tap after tap over ALL channels re-reads each pixel once per tap with the whole channel
+  // range in between, far more than an L2 holds across the workgroups of an XCD.  Cycling the
+  // taps over a block of 2-4 k-tiles keeps the re-reads in cache; shorter blocks re-enter taps
+  // (a few vector instructions each) more often.
+  g.chunk = g.Cs;
+  if (g.T > 1 && fast_path(g)) {
+    const int want = g.Cs >= 256 ? 64 : 32;
+    if (g.Cs % want == 0) g.chunk = want;
+  }
   if (g.ksplit > 1 && !g.accum) {
     const size_t n = (size_t)g.N * g.M * g.DH * g.DW;
     fill_zero_kernel<<<(unsigned)((n / 4 + kThreads) / kThreads), kThreads, 0, s>>>(dst, n);
