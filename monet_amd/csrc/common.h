@@ -38,6 +38,18 @@ __device__ __forceinline__ float wave_sum(float v) {
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, MN_WAVE);
   return v;
 }
+// Workgroups are handed to the 8 XCDs (each with its own L2) round-robin in launch order.
+// xcd_slot() turns a workgroup's launch index into a position in a LOGICAL order in which each
+// XCD runs one contiguous range: a kernel that decodes its tile from the slot, neighbours
+// first, lets the workgroups that read the same data share one L2 instead of pulling it into
+// eight.  A bijection on [0, total) for any total.
+__device__ __forceinline__ uint32_t xcd_slot() {
+  const uint32_t total = gridDim.x * gridDim.y * gridDim.z;
+  const uint32_t lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+  const uint32_t xcd = lin & 7u, j = lin >> 3, rem = total & 7u;
+  return xcd * (total >> 3) + (xcd < rem ? xcd : rem) + j;
+}
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, MN_WAVE));

@@ -122,8 +122,12 @@ __global__ __launch_bounds__(kThreads) void gather_bf16_kernel(const GatherH g,
   __shared__ uint32_t row_dst[BM];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  const uint32_t p0 = blockIdx.x * BM;
-  const int n0 = blockIdx.y * BN;
+  // XCD-aware order: contiguous ranges of position tiles per XCD, the channel tiles of a
+  // position tile one after the other (they gather the same pixels)
+  const uint32_t slot = xcd_slot();
+  const uint32_t bx = slot / gridDim.y, by = slot - bx * gridDim.y;
+  const uint32_t p0 = bx * BM;
+  const int n0 = by * BN;
   const uint32_t plane = (uint32_t)g.OH * g.OW;
   if (tid < g.T) {
     tdh[tid] = g.dh[tid];
@@ -329,16 +333,22 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))
   __shared__ __attribute__((aligned(16))) bf16_t lds_b[2][BNW][LDK];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  const int m0 = blockIdx.y * BMW;
+  // XCD-aware order: whole slices of the reduction per XCD (their workgroups read the same
+  // positions of dy and x)
+  const uint32_t slot = xcd_slot();
+  const uint32_t bz = slot / (gridDim.x * gridDim.y);
+  const uint32_t in_z = slot - bz * (gridDim.x * gridDim.y);
+  const uint32_t by = in_z / gridDim.x, bx = in_z - by * gridDim.x;
+  const int m0 = by * BMW;
   const uint32_t ctiles = (uint32_t)g.C / BNW;
-  const uint32_t tap = blockIdx.x / ctiles;
-  const uint32_t c0 = (blockIdx.x - tap * ctiles) * BNW;
+  const uint32_t tap = bx / ctiles;
+  const uint32_t c0 = (bx - tap * ctiles) * BNW;
   const uint32_t r = tap / g.S, sx = tap - r * g.S;
   const int dh = (int)r * g.dH - g.pH, dw = (int)sx * g.dW - g.pW;
   const uint32_t PQ = (uint32_t)g.P * g.Q;
 
   const uint32_t total_tiles = (g.depth + BK - 1) / BK;
-  const uint32_t t_begin = blockIdx.z * g.tiles_per_split;
+  const uint32_t t_begin = bz * g.tiles_per_split;
   const uint32_t t_end = min(t_begin + g.tiles_per_split, total_tiles);
 
   const __amdgpu_buffer_rsrc_t dy_buf =
@@ -451,7 +461,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))
         const int m = m0 + wm * (BMW / 2) + 32 * i + acc_row(v, lane);
         const size_t o = (size_t)m * row_len + (size_t)tap * g.C + c;
         if (g.partial)
-          reinterpret_cast<float*>(out)[(size_t)blockIdx.z * g.K * row_len + o] = acc[i][j][v];
+          reinterpret_cast<float*>(out)[(size_t)bz * g.K * row_len + o] = acc[i][j][v];
         else
           reinterpret_cast<bf16_t*>(out)[o] = f2bf(acc[i][j][v]);
       }
