@@ -267,8 +267,10 @@ def end_to_end(iters=10, warmup=3):
     target = torch.randint(0, 1000, (E2E_BS,), device=dev)
     res = {"model": "resnet50", "batch": E2E_BS, "dtype": "f32", "unit": "images/s",
            "step": "forward + cross entropy + backward + SGD momentum update"}
-    # op set of the reference, then the same with BatchNorm+ReLU pairs fused into one operator
-    for suffix, mode in (("", E2E_MODE), ("_fused", "fused_" + E2E_MODE)):
+    # op set of the reference, then the same with BatchNorm+ReLU and add+ReLU pairs fused into
+    # one operator each, then also with BatchNorm+add+ReLU triples (the end of a residual block)
+    for suffix, mode in (("", E2E_MODE), ("_fused", "fused_" + E2E_MODE),
+                         ("_fused2", "fused2_" + E2E_MODE)):
         base = None
         for budget in (100, 10, 6):
             sol = ROOT / "data" / ("solution_resnet50_%d_%s_%.2f.pkl" % (E2E_BS, mode, budget))

@@ -187,6 +187,33 @@ int mn_bn_relu_bwd_from_x_f32(const float* dy, const float* x, const float* gamm
                               float* dgamma, float* dbeta, int64_t N, int64_t C, int64_t HW,
                               void* ws, size_t ws_bytes, mn_stream_t stream);
 
+/* The end of a residual block as ONE forward operator (no counterpart in the
+ * reference, which runs F.batch_norm, bn.py:12-54, then `out += identity`,
+ * funcs.py:34-59, then a ReLU, relu.py: five passes over the activation where
+ * this kernel makes three):
+ *   forward (training):    y = max(BN(x) + alpha * added, 0), statistics of x as
+ *                          mn_bn_fwd_train_f32
+ *   forward (saved stats): y = max((x-mean)*invstd*gamma + beta + alpha * added, 0)
+ * `added` has the shape of x.  y may alias `added` or x.
+ *   backward: g = dy where y > 0, else 0 (the ReLU backward from the stored
+ *             output, relu.py:31-52); dadded = alpha * g; (dx, dgamma, dbeta) as
+ *             mn_bn_bwd_from_x_f32 with g in place of dy.  One pass: reads dy,
+ *             x, y once, writes dx and dadded once (channels short enough for
+ *             one workgroup run as two launches instead).  dadded may alias dy. */
+int mn_bn_add_relu_fwd_train_f32(const float* x, const float* gamma, const float* beta,
+                                 float* running_mean, float* running_var, const float* added,
+                                 double alpha, float* y, float* save_mean, float* save_invstd,
+                                 int64_t N, int64_t C, int64_t HW, double momentum, double eps,
+                                 void* ws, size_t ws_bytes, mn_stream_t stream);
+int mn_bn_add_relu_bwd_f32(const float* dy, const float* x, const float* y, const float* gamma,
+                           const float* mean, const float* invstd, double alpha, float* dx,
+                           float* dadded, float* dgamma, float* dbeta, int64_t N, int64_t C,
+                           int64_t HW, void* ws, size_t ws_bytes, mn_stream_t stream);
+int mn_bn_add_relu_fwd_apply_f32(const float* x, const float* mean, const float* invstd,
+                                 const float* gamma, const float* beta, const float* added,
+                                 double alpha, float* y, int64_t N, int64_t C, int64_t HW,
+                                 mn_stream_t stream);
+
 /* ----------------------------------------------------------- convolution --
  * 2-D convolution over NCHW tensors, weights [K, C, R, S], groups == 1.
  * P/Q are the output sizes: floor((H + 2*pH - dH*(R-1) - 1) / sH) + 1. */

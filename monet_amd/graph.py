@@ -96,13 +96,20 @@ class ComputeNode(Node):
 
 FUSED_BN_RELU = "monet::batch_norm_relu"
 FUSED_ADD_RELU = "monet::add_relu"
+FUSED_BN_ADD_RELU = "monet::batch_norm_add_relu"
 _FUSABLE = {"aten::batch_norm": FUSED_BN_RELU, "aten::add_": FUSED_ADD_RELU, "aten::add": FUSED_ADD_RELU}
+
+
+def fusion_level(mode):
+    """Fusion level named by a mode string: "fused2_..." = 2 (pairs and BatchNorm + add + ReLU
+    triples), "fused_..." = 1 (pairs), anything else 0."""
+    return 2 if "fused2_" in mode else (1 if "fused" in mode else 0)
 
 
 def is_batch_norm(op_name):
     """BatchNorm, alone or fused with the ReLU behind it: operators whose first forward of a
     step computes statistics that recomputations and the backward must reuse."""
-    return op_name in ("aten::batch_norm", FUSED_BN_RELU)
+    return op_name in ("aten::batch_norm", FUSED_BN_RELU, FUSED_BN_ADD_RELU)
 
 
 def two_step_backward(node):
@@ -165,6 +172,58 @@ class Graph:
         g._outputs = [new_index[o] for o in self._outputs]
         return g
 
+    def fuse_batch_norm_add_relu(self):
+        """Second fusion level, on a graph that went through `fuse_batch_norm_relu`: a fused
+        add + ReLU whose FIRST operand is a plain BatchNorm that nothing else reads (the end of
+        a residual block) becomes one `monet::batch_norm_add_relu` node with the BatchNorm's
+        arguments followed by the add's other operand and factor.  The node takes the add's
+        place in the order (the other operand may be computed after the BatchNorm's input)."""
+        nodes = self._nodes
+        readers = [0] * len(nodes)
+        for n in nodes:
+            if isinstance(n, ComputeNode):
+                for a in n.args:
+                    if isinstance(a, ComputeNode.D):
+                        readers[a.index] += 1
+        for o in self._outputs:
+            readers[o] += 1
+        absorbed = {}  # index of the add+ReLU node -> index of the BatchNorm it absorbs
+        for j, n in enumerate(nodes):
+            if not (isinstance(n, ComputeNode) and n.op == FUSED_ADD_RELU):
+                continue
+            first = n.args[0]
+            if not isinstance(first, ComputeNode.D) or readers[first.index] != 1:
+                continue
+            bn = nodes[first.index]
+            if isinstance(bn, ComputeNode) and bn.op == "aten::batch_norm" and \
+                    list(bn.shape) == list(n.shape) and len(n.args) == 3 and \
+                    isinstance(n.args[2], ComputeNode.V):
+                absorbed[j] = first.index
+        gone = set(absorbed.values())
+        g = Graph()
+        new_index = {}
+
+        def moved(a):
+            return ComputeNode.D(new_index[a.index], a.requires_grad) \
+                if isinstance(a, ComputeNode.D) else a
+
+        for k, n in enumerate(nodes):
+            if k in gone:
+                continue
+            if k in absorbed:
+                bn = nodes[absorbed[k]]
+                args = [moved(a) for a in bn.args] + [moved(a) for a in n.args[1:]]
+                new_index[k] = g._add(ComputeNode(n.shape, len(g._nodes), FUSED_BN_ADD_RELU, args,
+                                                  n.has_backward))
+            elif isinstance(n, ComputeNode):
+                new_index[k] = g._add(ComputeNode(n.shape, len(g._nodes), n.op,
+                                                  [moved(a) for a in n.args], n.has_backward,
+                                                  n.is_depthwise))
+            else:
+                new_index[k] = g._add(n)
+        g._outputs = [new_index[o] for o in self._outputs]
+        return g
+
     def _add_is_fusable(self, n):
         """An add fuses only if both operands are activations of the output's shape (no
         broadcasting, no parameter operand)."""
@@ -176,8 +235,14 @@ class Graph:
 
     @classmethod
     def create(cls, model, input_shape=(3, 224, 224), fuse_bn_relu=False):
+        """`fuse_bn_relu`: 0 / False = the operators as traced; 1 / True = BatchNorm + ReLU and
+        add + ReLU pairs as single nodes; 2 = also BatchNorm + add + ReLU triples."""
         g = cls._trace(model, input_shape)
-        return g.fuse_batch_norm_relu() if fuse_bn_relu else g
+        if fuse_bn_relu:
+            g = g.fuse_batch_norm_relu()
+            if int(fuse_bn_relu) >= 2:
+                g = g.fuse_batch_norm_add_relu()
+        return g
 
     @classmethod
     def _trace(cls, model, input_shape):

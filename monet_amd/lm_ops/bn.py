@@ -190,3 +190,109 @@ class InputActBatchNormReLU(_BatchNormForward):
             if not nodel:
                 del stored[4], stored[3], stored[2], stored[1], stored[0]
             return di, dw, db, None, None
+
+
+FUSED_BN_ADD_RELU = 'monet::batch_norm_add_relu'
+
+
+def bn_add_relu_forward_train(x, weight, bias, running_mean, running_var, added, alpha, momentum,
+                              eps):
+    """Training forward of max(BN(x) + alpha*added, 0) -> (y, save_mean, save_invstd)."""
+    xc, N, C, HW = _as_nchw(x, "input")
+    ac, _, _, _ = _as_nchw(added, "added activation")
+    if ac.shape != xc.shape:
+        raise RuntimeError("the added activation must have the shape of the BatchNorm input")
+    y = torch.empty_like(xc)
+    save_mean = torch.empty(C, dtype=torch.float32, device=x.device)
+    save_invstd = torch.empty(C, dtype=torch.float32, device=x.device)
+    ws, nbytes = _workspace(N, C, HW, x.device)
+    _lib.call("mn_bn_add_relu_fwd_train_f32", _lib.ptr(xc), _lib.ptr(weight), _lib.ptr(bias),
+              _lib.ptr(running_mean), _lib.ptr(running_var), _lib.ptr(ac), float(alpha), _lib.ptr(y),
+              _lib.ptr(save_mean), _lib.ptr(save_invstd), N, C, HW, float(momentum), float(eps),
+              _lib.ptr(ws), nbytes, _lib.stream_ptr(x.device))
+    return y, save_mean, save_invstd
+
+
+def bn_add_relu_forward_apply(x, mean, invstd, weight, bias, added, alpha):
+    """max((x - mean) * invstd * weight + bias + alpha*added, 0) with given per-channel vectors."""
+    xc, N, C, HW = _as_nchw(x, "input")
+    ac, _, _, _ = _as_nchw(added, "added activation")
+    if ac.shape != xc.shape:
+        raise RuntimeError("the added activation must have the shape of the BatchNorm input")
+    y = torch.empty_like(xc)
+    _lib.call("mn_bn_add_relu_fwd_apply_f32", _lib.ptr(xc), _lib.ptr(mean), _lib.ptr(invstd),
+              _lib.ptr(weight), _lib.ptr(bias), _lib.ptr(ac), float(alpha), _lib.ptr(y), N, C, HW,
+              _lib.stream_ptr(x.device))
+    return y
+
+
+def bn_add_relu_backward(grad, x, y, weight, save_mean, save_invstd, alpha):
+    """Backward of y = relu(BN(x) + alpha*added) from x and y in one pass ->
+    (dx, dweight, dbias, dadded).  `grad` is overwritten: dadded lives in its storage."""
+    tc, N, C, HW = _as_nchw(x, "stored input")
+    yc, _, _, _ = _as_nchw(y, "stored output")
+    g = grad if grad.is_contiguous() else grad.contiguous()
+    _lib.require_gpu_tensor(g, "grad_output", torch.float32)
+    if g.shape != tc.shape or yc.shape != tc.shape:
+        raise RuntimeError("grad_output and the stored activations differ in shape")
+    dx = torch.empty_like(tc)
+    dw = torch.empty(C, dtype=torch.float32, device=x.device)
+    db = torch.empty(C, dtype=torch.float32, device=x.device)
+    ws, nbytes = _workspace(N, C, HW, x.device)
+    _lib.call("mn_bn_add_relu_bwd_f32", _lib.ptr(g), _lib.ptr(tc), _lib.ptr(yc), _lib.ptr(weight),
+              _lib.ptr(save_mean), _lib.ptr(save_invstd), float(alpha), _lib.ptr(dx), _lib.ptr(g),
+              _lib.ptr(dw), _lib.ptr(db), N, C, HW, _lib.ptr(ws), nbytes, _lib.stream_ptr(x.device))
+    return dx, dw, db, g
+
+
+@implements([FUSED_BN_ADD_RELU],
+            ['normal', 'multiway', 'newnode', 'multiway_newnode', 'conv_multiway_newnode',
+             'conv_normal'])
+class InputActBatchNormAddReLU(OP):
+    """The end of a residual block, relu(BN(x) + alpha*added), as ONE operator (the tracer's
+    second fusion level produces `monet::batch_norm_add_relu` nodes with the BatchNorm's
+    arguments followed by the add's second operand and factor; the reference runs the three
+    operators of bn.py:12-54, funcs.py:34-59 and relu.py one after the other).  The forward is
+    one pass (2 reads + 1 write instead of 3 + 2).  Keeps the BatchNorm input and the output:
+    the backward gates the gradient by the sign of the output (that is the gradient of `added`)
+    and continues as BatchNorm backward from the input, in one pass as well (3 reads + 2 writes
+    instead of 2 + 1 for the ReLU backward and 2 + 1 for the BatchNorm backward)."""
+    backward_storage = [InputStorage(0, 1, 2, 3, 4), OutputStorage()]
+    params = None   # (training, eps, save_mean, save_invstd, alpha)
+    running_mean = None
+    running_var = None
+
+    def forward(self, input_, weight, bias, running_mean, running_var, training, momentum, eps,
+                cudnn_enabled, added, alpha=1):
+        with torch.no_grad():
+            if self.running_mean is None and running_mean is not None:
+                self.running_mean = running_mean.requires_grad_(False)
+                self.running_var = running_var.requires_grad_(False)
+            if self.params is None:
+                if training:
+                    out, save_mean, save_invstd = bn_add_relu_forward_train(
+                        input_, weight, bias, self.running_mean, self.running_var, added, alpha,
+                        momentum, eps)
+                else:
+                    save_mean = self.running_mean
+                    save_invstd = torch.rsqrt(self.running_var + eps)
+                    out = bn_add_relu_forward_apply(input_, save_mean, save_invstd, weight, bias,
+                                                    added, alpha)
+                self.params = bool(training), eps, save_mean, save_invstd, alpha
+            else:
+                _, _, save_mean, save_invstd, _ = self.params
+                out = bn_add_relu_forward_apply(input_, save_mean, save_invstd, weight, bias, added,
+                                                alpha)
+            return out
+
+    def backward(self, grad_output, stored, nodel=False):
+        with torch.no_grad():
+            input_, weight, bias, running_mean, running_var, output = stored
+            training, eps, save_mean, save_invstd, alpha = self.params
+            if not training:
+                raise NotImplementedError
+            di, dw, db, da = bn_add_relu_backward(grad_output, input_, output, weight, save_mean,
+                                                  save_invstd, alpha)
+            if not nodel:
+                del stored[5], stored[4], stored[3], stored[2], stored[1], stored[0]
+            return di, dw, db, None, None, da

@@ -499,7 +499,7 @@ def main(argv=None):
 
     import torch
 
-    from .graph import Graph
+    from .graph import Graph, fusion_level
     from .models import build_model
 
     parser = argparse.ArgumentParser()
@@ -531,7 +531,7 @@ def main(argv=None):
         model_name = si.model_name
     else:
         model, input_shape, model_name = build_model(args.model)
-        graph = Graph.create(model, input_shape=input_shape, fuse_bn_relu="fused" in args.mode)
+        graph = Graph.create(model, input_shape=input_shape, fuse_bn_relu=fusion_level(args.mode))
         model.cuda()
         input_ = torch.randn([args.bs, *input_shape]).cuda()
         si = SolverInfo(args.bs, model_name=model_name, mode=args.mode, data_dir=args.data_dir)

@@ -27,7 +27,7 @@ from pathlib import Path
 import numpy as np
 
 from . import lm_ops
-from .graph import ComputeNode, Graph, Input, Param, is_batch_norm, two_step_backward
+from .graph import ComputeNode, Graph, Input, Param, fusion_level, is_batch_norm, two_step_backward
 
 MEMORY_MULTIPLIER = 4  # bytes per element: the path is fp32 (solver_info.py:10)
 
@@ -127,9 +127,10 @@ class SolverInfo:
         self.do_inplace = "inplace" in mode
         self.compute_newnode = "newnode" in mode
         # "fused_": the graph was traced with BatchNorm+ReLU pairs as single operators
-        self.fuse_bn_relu = "fused" in mode
+        # "fused2_": also BatchNorm + add + ReLU triples (the end of a residual block)
+        self.fuse_bn_relu = fusion_level(mode)
         # the registry knows nothing of these prefixes
-        self.mode = mode.replace("fused_", "").replace("inplace_", "")
+        self.mode = mode.replace("fused2_", "").replace("fused_", "").replace("inplace_", "")
 
     # ------------------------------------------------------------------ build
     def extract(self, graph: Graph, *args, cost_fn=None):

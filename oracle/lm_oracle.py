@@ -295,6 +295,27 @@ def bn_relu_bwd_from_x(dy, x, gamma, beta, mean, invstd, positive=None, dtype=np
     return bn_bwd_from_x(np.where(positive, dy, 0).astype(dy.dtype), x, gamma, mean, invstd, dtype)
 
 
+def bn_add_relu_fwd_train(x, gamma, beta, added, alpha, running_mean, running_var, momentum, eps,
+                          dtype=np.float64):
+    """The end of a residual block as one operator: relu(BN(x) + alpha * added), the
+    composition of bn_fwd_train, the residual add (monet/lm_ops/funcs.py:34-59) and max(., 0).
+    Returns what bn_fwd_train returns with y replaced.
+    Pinned by: torch.relu(F.batch_norm(training=True) + alpha * added) on CPU in float64."""
+    out = list(bn_fwd_train(x, gamma, beta, running_mean, running_var, momentum, eps, dtype))
+    out[0] = np.maximum(out[0] + dtype(alpha) * np.asarray(added, dtype=dtype), 0)
+    return tuple(out)
+
+
+def bn_add_relu_bwd(dy, x, y, gamma, mean, invstd, alpha=1.0, dtype=np.float64):
+    """Backward of y = relu(BN(x) + alpha * added) from the stored x and y: the gradient only
+    passes where y > 0; that gated gradient times alpha is the gradient of `added`, and
+    bn_bwd_from_x turns it into (dx, dgamma, dbeta).  Returns (dx, dgamma, dbeta, dadded).
+    Pinned by: float64 autograd through the torch composition for x, gamma, beta and added."""
+    g = np.where(np.asarray(y) > 0, dy, 0).astype(np.asarray(dy).dtype)
+    dx, dgamma, dbeta = bn_bwd_from_x(g, x, gamma, mean, invstd, dtype)
+    return dx, dgamma, dbeta, g.astype(dtype) * dtype(alpha)
+
+
 def bn_bwd_from_x(dy, x, gamma, mean, invstd, dtype=np.float64):
     """(dx, dgamma, dbeta) from the input: the standard BatchNorm backward that
     cudnn_batch_norm_backward computes for do_cudnn_backward (lrbn.cpp:43-70).

@@ -153,7 +153,8 @@ def test_convolution_directions_are_adjoint_at_full_size(cuda, dtype, tol):
         assert float((ys.float() - (y.float() + y2.float())).abs().max()) < lin_tol, v
 
 
-@pytest.mark.parametrize("mode", ["inplace_conv_multiway_newnode", "fused_inplace_conv_multiway_newnode"])
+@pytest.mark.parametrize("mode", ["inplace_conv_multiway_newnode", "fused_inplace_conv_multiway_newnode",
+                                  "fused2_inplace_conv_multiway_newnode"])
 def test_resnet50_batch_184_under_the_committed_10gb_schedule(cuda, mode):
     """The headline configuration end to end: `MONeTWrapper` with the schedule in data/ against
     stock autograd on the same weights and batch.  Losses agree to 1e-5; the peak stays within

@@ -318,6 +318,50 @@ def test_bn_relu_fused_forward_backward_and_recompute(cuda, shape):
     assert_rel(host(db), odb, 3e-5, "dbeta")
 
 
+@pytest.mark.parametrize("alpha", [1, 0.5])
+@pytest.mark.parametrize("shape", BN_SHAPES)
+def test_bn_add_relu_fused_forward_backward_and_recompute(cuda, shape, alpha):
+    """relu(BN(x) + alpha*r) as one operator: forward against the oracle, recomputation from
+    the saved statistics, backward against the oracle fed the GPU's own output (an output
+    within rounding distance of zero may legitimately fall on either side)."""
+    x, gamma, beta, dy = bn_problem(shape, 8)
+    r = np.random.default_rng(9).standard_normal(shape).astype(np.float32)
+    oy, omean, oinv, _, _ = O.bn_add_relu_fwd_train(x, gamma, beta, r, alpha, None, None, 0.1, 1e-5)
+    op = lm_ops.bn.InputActBatchNormAddReLU()
+    tx, tw, tb, tg, tr = (dev(x, cuda), dev(gamma, cuda), dev(beta, cuda), dev(dy, cuda),
+                          dev(r, cuda))
+    C = shape[1]
+    rm, rv = torch.zeros(C, device=cuda), torch.ones(C, device=cuda)
+    y = op.forward(tx, tw, tb, rm, rv, True, 0.1, 1e-5, True, tr, alpha)
+    assert_rel(host(y), oy, 1e-5, "relu(bn(x) + r)")
+    assert float(y.min()) >= 0.0
+    assert np.array_equal(host(tx), x) and np.array_equal(host(tr), r)   # operands untouched
+    # the statistics are those of the plain forward
+    plain = lm_ops.bn.InputActBatchNorm()
+    rm2, rv2 = torch.zeros(C, device=cuda), torch.ones(C, device=cuda)
+    plain.forward(tx, tw, tb, rm2, rv2, True, 0.1, 1e-5)
+    # (another piece length, hence another summation order: equal to rounding, not bit for bit)
+    assert_rel(host(op.params[2]), host(plain.params[2]), 1e-6, "save_mean")
+    assert_rel(host(op.params[3]), host(plain.params[3]), 1e-6, "save_invstd")
+    assert_rel(host(rm), host(rm2), 1e-6, "running_mean")
+    assert_rel(host(rv), host(rv2), 1e-6, "running_var")
+    rm_after_first = rm.clone()
+    pre = O.bn_fwd_train(x, gamma, beta, None, None, 0.1, 1e-5)[0] + alpha * r.astype(np.float64)
+    clear = np.abs(pre) > 1e-4
+    assert np.array_equal((host(y) > 0)[clear], (oy > 0)[clear])
+    y2 = op.forward(tx, tw, tb, rm, rv, True, 0.1, 1e-5, True, tr, alpha)   # recomputation
+    assert_rel(host(y2), host(y), 2e-7, "recomputed relu(bn(x) + r)")
+    assert torch.equal(rm, rm_after_first)                                 # no second update
+    odx, odg, odb, odr = O.bn_add_relu_bwd(dy, x, host(y), gamma, omean, oinv, alpha)
+    stored = [tx, tw, tb, rm, rv, y]
+    dx, dg, db, n1, n2, dr = op.backward(tg.clone(), stored)
+    assert stored == [] and n1 is None and n2 is None
+    assert_rel(host(dx), odx, 1e-5, "dx")
+    assert_rel(host(dg), odg, 3e-5, "dgamma")
+    assert_rel(host(db), odb, 3e-5, "dbeta")
+    assert np.array_equal(host(dr), odr.astype(np.float32))               # a gated copy: exact
+
+
 @pytest.mark.parametrize("shape", BN_SHAPES)
 def test_bn_backward_from_input_and_from_output(cuda, shape):
     x, gamma, beta, dy = bn_problem(shape, 1)

@@ -35,10 +35,10 @@ class SmallNet(nn.Module):
 
 
 def _solve(model, shape, bs, mode, budget_gb, cuda):
-    from monet_amd.graph import Graph
+    from monet_amd.graph import Graph, fusion_level
     from monet_amd.solver import Model
     from monet_amd.solver_info import SolverInfo
-    graph = Graph.create(copy.deepcopy(model).cpu(), shape, fuse_bn_relu="fused" in mode)
+    graph = Graph.create(copy.deepcopy(model).cpu(), shape, fuse_bn_relu=fusion_level(mode))
     x = torch.randn((bs,) + shape, device=cuda)
     si = SolverInfo(bs, "test", mode)
     si.extract(graph, x, *list(model.state_dict(keep_vars=True).values()))
@@ -59,7 +59,8 @@ def _rel(a, b, floor=1e-30):
 
 @pytest.mark.parametrize("mode", ["normal", "multiway_newnode", "conv_multiway_newnode",
                                   "inplace_conv_multiway_newnode",
-                                  "fused_inplace_conv_multiway_newnode"])
+                                  "fused_inplace_conv_multiway_newnode",
+                                  "fused2_inplace_conv_multiway_newnode"])
 def test_schedule_matches_autograd(cuda, mode):
     from monet_amd.schedule import Schedule
     torch.manual_seed(0)

@@ -274,6 +274,26 @@ def test_bn_relu_fused_matches_autograd_of_the_composition(shape):
     np.testing.assert_allclose(dx2, dx, rtol=1e-12)
 
 
+@pytest.mark.parametrize("shape,alpha", [((4, 3, 5, 5), 1.0), ((2, 8, 7, 3), 0.5), ((16, 4, 6, 6), 1.0)])
+def test_bn_add_relu_fused_matches_autograd_of_the_composition(shape, alpha):
+    x, gamma, beta, dy = _bn_problem(shape, 6)
+    r = np.random.default_rng(7).standard_normal(shape)
+    tx = torch.from_numpy(x).requires_grad_(True)
+    tw = torch.from_numpy(gamma).requires_grad_(True)
+    tb = torch.from_numpy(beta).requires_grad_(True)
+    tr = torch.from_numpy(r).requires_grad_(True)
+    ty = torch.relu(F.batch_norm(tx, None, None, tw, tb, True, 0.1, 1e-5) + alpha * tr)
+    ty.backward(torch.from_numpy(dy))
+    y, mean, invstd, _, _ = O.bn_add_relu_fwd_train(x, gamma, beta, r, alpha, None, None, 0.1, 1e-5)
+    np.testing.assert_allclose(y, ty.detach().numpy(), rtol=1e-12, atol=1e-14)
+    assert (y >= 0).all() and (y == 0).any() and (y > 0).any()
+    dx, dg, db, dr = O.bn_add_relu_bwd(dy, x, y, gamma, mean, invstd, alpha)
+    np.testing.assert_allclose(dx, tx.grad.numpy(), rtol=1e-9, atol=1e-10)
+    np.testing.assert_allclose(dg, tw.grad.numpy(), rtol=1e-9, atol=1e-10)
+    np.testing.assert_allclose(db, tb.grad.numpy(), rtol=1e-9, atol=1e-10)
+    np.testing.assert_allclose(dr, tr.grad.numpy(), rtol=1e-12, atol=1e-14)
+
+
 # ------------------------------------------------------------------- softmax
 @pytest.mark.parametrize("shape,dim", [((7, 10), 1), ((3, 2, 5, 4), 1), ((4, 6, 3), 2), ((5,), 0)])
 def test_softmax_matches_torch(shape, dim):

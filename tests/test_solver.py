@@ -42,7 +42,7 @@ def synthetic_cost(si):
                    ([mb] * nf, [mb * (1.0 - 0.1 * c) for c in range(nb)], [])
         if si.do_inplace and hasattr(op, 'inplace'):
             return ([0.0, 0.0], [0.0], []), ([0.1 * mb, 0.1 * mb], [0.1 * mb], [])
-        if n.op in ("aten::batch_norm", "monet::batch_norm_relu"):
+        if n.op in ("aten::batch_norm", "monet::batch_norm_relu", "monet::batch_norm_add_relu"):
             return ([0.0], [0.0], [0.0]), ([0.2 * mb], [0.3 * mb], [0.1 * mb])
         # implementations that keep an intermediate are a bit slower
         extra = 0.02 * mb if "Binary" in type(op).__name__ or "Indices" in type(op).__name__ else 0
@@ -241,6 +241,7 @@ def test_model_definitions_trace_to_the_expected_operators():
     assert name == "resnet50" and shape == (3, 224, 224)
     assert sum(p.numel() for p in model.parameters()) == 25557032
     g = Graph.create(model, shape)
+    from collections import Counter
     ops = Counter(n.op for n in g.nodes if isinstance(n, ComputeNode))
     assert ops == {"aten::_convolution": 53, "aten::batch_norm": 53, "aten::relu_": 49,
                    "aten::add_": 16, "aten::max_pool2d": 1, "aten::adaptive_avg_pool2d": 1,
@@ -277,3 +278,36 @@ def test_batch_norm_relu_fusion_pass():
     assert si.fuse_bn_relu and si.mode == "conv_multiway_newnode"
     sol = Model(si, budget=1.0, time_limit=60, mip_rel_gap=0.0).solve()
     Schedule(f, si).init_schedule(sol, si.mode)
+
+
+def test_batch_norm_add_relu_fusion_pass():
+    """Second fusion level: the BatchNorm in front of a residual add + ReLU joins them."""
+    f1 = Graph.create(SmallNet(), (3, 16, 16), fuse_bn_relu=1)
+    f2 = Graph.create(SmallNet(), (3, 16, 16), fuse_bn_relu=2)
+    kinds = [n.op for n in f2.nodes if isinstance(n, ComputeNode)]
+    assert kinds == ["aten::_convolution", "monet::batch_norm_relu", "aten::max_pool2d",
+                     "aten::_convolution", "monet::batch_norm_add_relu",
+                     "aten::adaptive_avg_pool2d", "aten::flatten", "aten::linear"]
+    assert len(f2.nodes) == len(f1.nodes) - 1 and f2._outputs == [len(f2.nodes) - 1]
+    triple = next(n for n in f2.nodes if isinstance(n, ComputeNode) and
+                  n.op == "monet::batch_norm_add_relu")
+    # the BatchNorm's nine arguments, then the add's second operand and factor
+    assert len(triple.args) == 11
+    assert f2.nodes[triple.args[0].index].op == "aten::_convolution"
+    assert f2.nodes[triple.args[9].index].op == "aten::max_pool2d"
+    assert isinstance(triple.args[10], ComputeNode.V) and triple.args[10].value == 1
+    assert [d for d, _ in triple.dependencies][:5] == [a.index for a in triple.args[:5]]
+    si = SolverInfo(16, "small", "fused2_inplace_conv_multiway_newnode")
+    si.extract(f2, cost_fn=synthetic_cost(si))
+    assert si.fuse_bn_relu == 2 and si.mode == "conv_multiway_newnode"
+    sol = Model(si, budget=1.0, time_limit=60, mip_rel_gap=0.0).solve()
+    Schedule(f2, si).init_schedule(sol, si.mode)
+    # ResNet-50: every block's last BatchNorm joins its add + ReLU (16), the downsample
+    # BatchNorms (second operand of the add) stay
+    from monet_amd.models import build_model
+    model, shape, _ = build_model("resnet50")
+    g = Graph.create(model, shape, fuse_bn_relu=2)
+    from collections import Counter
+    ops = Counter(n.op for n in g.nodes if isinstance(n, ComputeNode))
+    assert ops["monet::batch_norm_add_relu"] == 16 and ops["monet::add_relu"] == 0
+    assert ops["aten::batch_norm"] == 4 and ops["monet::batch_norm_relu"] == 33
