@@ -51,6 +51,7 @@ struct Vec<1> {
 struct Shape {
   int C;
   int S;         // pieces per channel
+  int G;         // resident launch: channels whose pieces are handed out interleaved
   uint32_t HWV;  // vectors per (n, c) slab
   uint32_t HW;   // elements per slab
   uint64_t L;    // vectors per piece
@@ -449,8 +450,20 @@ __device__ __forceinline__ void hold_piece(const Args& A, uint32_t item, Held<VE
   typedef CursorT<THREADS> Cursor;
   const Shape& sh = A.sh;
   const int S = sh.S;
-  h.c = item / S;
-  h.piece = item - h.c * S;
+  if (SOLO || sh.G <= 1) {
+    h.c = item / S;
+    h.piece = item - h.c * S;
+  } else {
+    // tickets run over groups of G neighbouring channels, inside a group piece by piece with
+    // the channels of a piece next to each other: workgroups that run at the same time read
+    // neighbouring planes of the same images
+    const uint32_t per_group = (uint32_t)sh.G * S;
+    const uint32_t grp = item / per_group, within = item - grp * per_group;
+    const uint32_t c0 = grp * sh.G;
+    const uint32_t gc = min((uint32_t)sh.G, (uint32_t)sh.C - c0);
+    h.piece = within / gc;
+    h.c = c0 + (within - h.piece * gc);
+  }
   h.sft = reduce_shift<MODE>(A, h.c);  // forward: the pivot, read before any store to the channel
   {
     Cursor cur(sh, h.piece);
@@ -648,6 +661,7 @@ static void fill_shape(int64_t N, int64_t C, int64_t HW, int vec, int64_t S, uin
   sh.HW = (uint32_t)HW;
   sh.tot = (uint64_t)N * sh.HWV;
   sh.L = L;
+  sh.G = 1;
 }
 
 template <int MODE>
@@ -692,6 +706,15 @@ static int run(Args& A, int64_t N, int64_t C, int64_t HW, bool aligned16, void* 
   if (t.resident && rp <= kMaxResident) {
     fill_shape(N, C, HW, vec, rp, vec == 4 ? (uint64_t)threads * keep : (uint64_t)kThreads * 16, A.sh);
     const unsigned blocks = (unsigned)(C * rp);
+    // Interleave the pieces of up to 8 neighbouring channels (the workgroups of the moment then
+    // read neighbouring planes of the same images: 1-2 % at [184,256,56,56]).  A workgroup only
+    // waits while it holds two published pieces, both inside the lowest unfinished group or
+    // later, so with at least kMaxResident workgroups running nobody can be left waiting as
+    // long as a group has fewer than 2 * kMaxResident pieces.
+    A.sh.G = (int)(448 / rp < 1 ? 1 : (448 / rp > 8 ? 8 : 448 / rp));
+#ifdef MN_TUNING
+    if (const char* e = getenv("MN_BN_GROUP")) A.sh.G = atoi(e);
+#endif
     bn_prepare_kernel<<<(blocks + 255) / 256, 256, 0, s>>>(
           reinterpret_cast<uint64_t*>(A.partial), blocks, A.ticket);
     // persistent grid: enough workgroups to fill 256 CUs at this register footprint
