@@ -690,7 +690,11 @@ static int run(Args& A, int64_t N, int64_t C, int64_t HW, bool aligned16, void* 
   }
   // whole channels in one workgroup's registers
   const uint64_t chan = (uint64_t)N * (HW / vec);
-  if (t.resident && t.keep == 8 && t.threads == kThreads) {
+  bool solo = t.resident && t.keep == 8 && t.threads == kThreads;
+#ifdef MN_TUNING
+  if (const char* e = getenv("MN_BN_SOLO")) solo = solo && atoi(e) != 0;
+#endif
+  if (solo) {
     const unsigned grid = (unsigned)(C < 65535 ? C : 65535);
 #define MN_BN_SOLO(V, K, T)                                              \
   do {                                                                   \
