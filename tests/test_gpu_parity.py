@@ -427,6 +427,38 @@ def test_bn_channel_too_large_to_keep_on_chip(cuda):
     assert_rel(host(db), odb, 1e-4, "dbeta")
 
 
+def test_bn_add_relu_channel_too_large_to_keep_on_chip(cuda):
+    # the fused end of a residual block on the two-launch (reduce, apply) formulation
+    shape = (1, 2, 2100, 2048)
+    x, gamma, beta, dy = bn_problem(shape, 6)
+    r = np.random.default_rng(10).standard_normal(shape).astype(np.float32)
+    oy, omean, oinv, _, _ = O.bn_add_relu_fwd_train(x, gamma, beta, r, 1.0, None, None, 0.1, 1e-5)
+    tx, tw, tb, tr = dev(x, cuda), dev(gamma, cuda), dev(beta, cuda), dev(r, cuda)
+    y, mean, invstd = bn_ops.bn_add_relu_forward_train(tx, tw, tb, None, None, tr, 1, 0.1, 1e-5)
+    assert_rel(host(y), oy, 1e-5, "y")
+    y2 = bn_ops.bn_add_relu_forward_apply(tx, mean, invstd, tw, tb, tr, 1)
+    assert_rel(host(y2), host(y), 2e-7, "recomputed y")
+    odx, odg, odb, odr = O.bn_add_relu_bwd(dy, x, host(y), gamma, omean, oinv, 1.0)
+    dx, dg, db, dr = bn_ops.bn_add_relu_backward(dev(dy, cuda), tx, y, tw, mean, invstd, 1)
+    assert_rel(host(dx), odx, 2e-5, "dx")
+    assert_rel(host(dg), odg, 1e-4, "dgamma")
+    assert_rel(host(db), odb, 1e-4, "dbeta")
+    assert np.array_equal(host(dr), odr.astype(np.float32))
+
+
+def test_bn_add_relu_eval_mode_uses_running_statistics(cuda):
+    op = lm_ops.bn.InputActBatchNormAddReLU()
+    x = torch.randn(2, 3, 4, 4, device=cuda)
+    r = torch.randn(2, 3, 4, 4, device=cuda)
+    w, b = torch.rand(3, device=cuda) + 0.5, torch.randn(3, device=cuda)
+    rm, rv = torch.randn(3, device=cuda), torch.rand(3, device=cuda) + 0.5
+    y = op.forward(x, w, b, rm, rv, False, 0.1, 1e-5, True, r, 1)
+    ref = torch.relu(torch.nn.functional.batch_norm(x, rm, rv, w, b, False, 0.1, 1e-5) + r)
+    torch.testing.assert_close(y, ref, rtol=1e-5, atol=1e-6)
+    with pytest.raises(NotImplementedError):
+        op.backward(torch.ones_like(y), [x, w, b, rm, rv, y])
+
+
 def test_bn_non_affine_and_inplace_output(cuda):
     shape = (4, 3, 8, 8)
     x, _, _, dy = bn_problem(shape, 3)
