@@ -4,7 +4,12 @@
   OutputActBatchNorm   backward from the stored OUTPUT  (bn.py:96-140), so an
                        in-place consumer chain can drop the input.
 
-Both share the forward: the first forward of an iteration computes batch
+  InputActBatchNormReLU     relu(BN(x)) as one operator, from the stored input
+  InputActBatchNormAddReLU  relu(BN(x) + alpha*r) as one operator (the end of a residual
+                            block), from the stored input and output
+(the last two only exist in graphs that went through the tracer's fusion passes).
+
+The first three share the forward: the first forward of an iteration computes batch
 statistics, updates the running statistics and records
 `params = (training, eps, save_mean, save_invstd, reserve)`; a forward on an
 instance whose `params` are already set is a RECOMPUTATION and re-applies the
