@@ -606,7 +606,10 @@ template <int VEC, int MODE, int KEEP, int THREADS>
 __global__ __launch_bounds__(THREADS) void bn_solo_kernel(const Args A) {
   __shared__ float lds[2 * (THREADS / MN_WAVE)];
   Held<VEC, KEEP> h;
-  for (uint32_t c = blockIdx.x; c < (uint32_t)A.sh.C; c += gridDim.x) {
+  // Planes this short do not end on cache-line boundaries: neighbouring channels share their
+  // first and last lines.  Each XCD takes a contiguous range of channels, so the shared lines
+  // meet in one L2 instead of being fetched (and written back in parts) by two.
+  for (uint32_t c = xcd_slot(); c < (uint32_t)A.sh.C; c += gridDim.x) {
     hold_piece<VEC, MODE, KEEP, THREADS, true>(A, c, h, lds);
     finish_piece<VEC, MODE, KEEP, THREADS, true>(A, h, lds);
   }
