@@ -32,7 +32,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth, GB/s
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `--only lm_ops`, scaled by
 # what the same counters read for a plain copy of known size (FETCH_SIZE x2.000, WRITE_SIZE x1.000);
 # the counter run cannot happen inside this program, so the figures are recorded here
-TRAFFIC = {"bn_bwd_from_output": 1775456256, "relu_bwd_mask": 1200261120, "maxpool_bwd_idx": 778724352}
+TRAFFIC = {"bn_bwd_from_output": 1775575040, "relu_bwd_mask": 1200261120, "maxpool_bwd_idx": 778724352}
 
 N, C, H, W = 184, 256, 56, 56          # BN / ReLU tensor
 PN, PC, PH_IN, PW_IN = 184, 64, 112, 112  # max-pool input
