@@ -209,6 +209,27 @@ int mn_bn_add_relu_bwd_f32(const float* dy, const float* x, const float* y, cons
                            const float* mean, const float* invstd, double alpha, float* dx,
                            float* dadded, float* dgamma, float* dbeta, int64_t N, int64_t C,
                            int64_t HW, void* ws, size_t ws_bytes, mn_stream_t stream);
+/* The same operator keeping a 1-bit mask of y > 0 (format of mn_pack_bits_u8 /
+ * mn_relu_fwd_mask_f32: (N*C*HW + 7) / 8 bytes over the flat tensor, first
+ * element in bit 7) instead of relying on y in the backward: the forward writes
+ * the mask from the registers that hold y (planes of a multiple of 8 elements;
+ * other shapes pack y in a second launch), the backward reads dy, x and the
+ * mask and writes dx and dadded: 4 + 1/32 passes instead of 5. */
+int mn_bn_add_relu_mask_fwd_train_f32(const float* x, const float* gamma, const float* beta,
+                                      float* running_mean, float* running_var, const float* added,
+                                      double alpha, float* y, uint8_t* mask, float* save_mean,
+                                      float* save_invstd, int64_t N, int64_t C, int64_t HW,
+                                      double momentum, double eps, void* ws, size_t ws_bytes,
+                                      mn_stream_t stream);
+int mn_bn_add_relu_mask_fwd_apply_f32(const float* x, const float* mean, const float* invstd,
+                                      const float* gamma, const float* beta, const float* added,
+                                      double alpha, float* y, uint8_t* mask, int64_t N, int64_t C,
+                                      int64_t HW, mn_stream_t stream);
+int mn_bn_add_relu_mask_bwd_f32(const float* dy, const float* x, const uint8_t* mask,
+                                const float* gamma, const float* mean, const float* invstd,
+                                double alpha, float* dx, float* dadded, float* dgamma,
+                                float* dbeta, int64_t N, int64_t C, int64_t HW, void* ws,
+                                size_t ws_bytes, mn_stream_t stream);
 int mn_bn_add_relu_fwd_apply_f32(const float* x, const float* mean, const float* invstd,
                                  const float* gamma, const float* beta, const float* added,
                                  double alpha, float* y, int64_t N, int64_t C, int64_t HW,

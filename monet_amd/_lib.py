@@ -81,6 +81,13 @@ _SIGNATURES = {
                                              c_int64, _P]),
     "mn_bn_add_relu_bwd_f32": (c_int, [_P, _P, _P, _P, _P, _P, c_double, _P, _P, _P, _P, c_int64,
                                        c_int64, c_int64, _P, c_size_t, _P]),
+    "mn_bn_add_relu_mask_fwd_train_f32": (c_int, [_P, _P, _P, _P, _P, _P, c_double, _P, _P, _P, _P,
+                                                  c_int64, c_int64, c_int64, c_double, c_double, _P,
+                                                  c_size_t, _P]),
+    "mn_bn_add_relu_mask_fwd_apply_f32": (c_int, [_P, _P, _P, _P, _P, _P, c_double, _P, _P, c_int64,
+                                                  c_int64, c_int64, _P]),
+    "mn_bn_add_relu_mask_bwd_f32": (c_int, [_P, _P, _P, _P, _P, _P, c_double, _P, _P, _P, _P, c_int64,
+                                            c_int64, c_int64, _P, c_size_t, _P]),
     "mn_softmax_fwd_f32": (c_int, [_P, _P, c_int64, c_int64, c_int64, _P]),
     "mn_softmax_bwd_f32": (c_int, [_P, _P, _P, c_int64, c_int64, c_int64, _P]),
     "mn_xent_bwd_f32": (c_int, [_P, _P, _P, c_int64, c_int64, c_int64, c_float, _P]),

@@ -111,7 +111,15 @@ __device__ __forceinline__ void setc(float& v, int, float a) { v = a; }
 // BWD_FROM_X_GATED: its backward from x and the output y: the incoming gradient only counts
 // where y > 0; the gated gradient (times ralpha) is also written out, as the gradient of the
 // added tensor.
-enum Mode { BWD_FROM_X = 0, BWD_FROM_Y = 1, FWD_TRAIN = 2, FWD_TRAIN_ADD = 3, BWD_FROM_X_GATED = 4 };
+// BWD_FROM_X_MASKED: the same with the gate read from a 1-bit mask (bit 7 of a byte = first
+// element) that the forward wrote.
+enum Mode {
+  BWD_FROM_X = 0, BWD_FROM_Y = 1, FWD_TRAIN = 2, FWD_TRAIN_ADD = 3, BWD_FROM_X_GATED = 4,
+  BWD_FROM_X_MASKED = 5
+};
+constexpr bool hands_on_gradient(int mode) {
+  return mode == BWD_FROM_X_GATED || mode == BWD_FROM_X_MASKED;
+}
 constexpr bool is_fwd(int mode) { return mode == FWD_TRAIN || mode == FWD_TRAIN_ADD; }
 
 // Everything a statistics-then-apply operator needs.
@@ -140,7 +148,10 @@ struct Args {
   const float* rbeta;
   float ralpha;         // FWD_TRAIN_ADD: factor of the added tensor; BWD_FROM_X_GATED: of gated_out
   const float* gate_ref;  // BWD_FROM_X_GATED: y
-  float* gated_out;       // BWD_FROM_X_GATED: ralpha * (y > 0 ? dy : 0); may alias a
+  float* gated_out;       // BWD_FROM_X_GATED / _MASKED: ralpha * (gate ? dy : 0); may alias a
+  const uint8_t* mask_in; // BWD_FROM_X_MASKED: packed sign bits of y over the flat tensor
+  uint8_t* mask_out;      // FWD_TRAIN_ADD, optional: packed y > 0 (vector kernels whose lane pairs
+                          // hold the two halves of a byte: HW % 8 == 0, even piece lengths)
 };
 
 // g where ref > 0, else 0 (a NaN reference passes nothing, like the ReLU backward from a
@@ -152,6 +163,27 @@ __device__ __forceinline__ float4_t gate_by(float4_t g, float4_t ref) {
   return r;
 }
 __device__ __forceinline__ float gate_by(float g, float ref) { return ref > 0.f ? g : 0.f; }
+// The same from the packed mask; `o` = flat element offset of the vector / element.
+__device__ __forceinline__ float4_t gate_by_mask(float4_t g, const uint8_t* mask, size_t o) {
+  const uint32_t byte = mask[o >> 3];
+  const uint32_t nib = (o & 4) ? (byte & 15u) : (byte >> 4);
+  float4_t r;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) r[k] = (nib & (8u >> k)) ? g[k] : 0.f;
+  return r;
+}
+__device__ __forceinline__ float gate_by_mask(float g, const uint8_t* mask, size_t o) {
+  return ((mask[o >> 3] >> (7 - (o & 7))) & 1u) ? g : 0.f;
+}
+// Forward: the four sign bits of a result vector, joined with the neighbouring lane's into one
+// mask byte (the even lane of a pair holds the even vector, i.e. the high nibble, and stores).
+__device__ __forceinline__ void put_mask(uint8_t* mask, size_t o, float4_t y) {
+  const uint32_t nib = (y[0] > 0.f ? 8u : 0u) | (y[1] > 0.f ? 4u : 0u) | (y[2] > 0.f ? 2u : 0u) |
+                       (y[3] > 0.f ? 1u : 0u);
+  const uint32_t other = __shfl_xor(nib, 1, MN_WAVE);
+  if (!(threadIdx.x & 1u)) mask[o >> 3] = (uint8_t)((nib << 4) | other);
+}
+__device__ __forceinline__ void put_mask(uint8_t*, size_t, float) {}
 
 // The ReLU gate of the fused backward, per channel.
 struct Gate {
@@ -193,6 +225,7 @@ __device__ __forceinline__ void reduce_piece(const Args& A, int c, int piece, fl
         vb[u] = ldv<VEC>(A.b + o);
         if (!is_fwd(MODE)) va[u] = ldv<VEC>(A.a + o);
         if (MODE == BWD_FROM_X_GATED) va[u] = gate_by(va[u], ldv<VEC>(A.gate_ref + o));
+        if (MODE == BWD_FROM_X_MASKED) va[u] = gate_by_mask(va[u], A.mask_in, o);
       }
       cur.next();
     }
@@ -245,6 +278,7 @@ __device__ __forceinline__ void apply_piece(const Args& A, int c, int piece, flo
         vb[u] = ldv<VEC>(A.b + o[u]);
         if (MODE != FWD_TRAIN) va[u] = ldv<VEC>(A.a + o[u]);
         if (MODE == BWD_FROM_X_GATED) va[u] = gate_by(va[u], ldv<VEC>(A.gate_ref + o[u]));
+        if (MODE == BWD_FROM_X_MASKED) va[u] = gate_by_mask(va[u], A.mask_in, o[u]);
       }
       cur.next();
     }
@@ -264,7 +298,8 @@ __device__ __forceinline__ void apply_piece(const Args& A, int c, int piece, flo
           }
         }
         stv<VEC>(A.out + o[u], r);
-        if (MODE == BWD_FROM_X_GATED) stv<VEC>(A.gated_out + o[u], va[u] * A.ralpha);
+        if (hands_on_gradient(MODE)) stv<VEC>(A.gated_out + o[u], va[u] * A.ralpha);
+        if (MODE == FWD_TRAIN_ADD && VEC == 4 && A.mask_out) put_mask(A.mask_out, o[u], r);
       }
     }
   }
@@ -496,6 +531,18 @@ __device__ __forceinline__ void hold_piece(const Args& A, uint32_t item, Held<VE
       cur2.next();
     }
   }
+  if (MODE == BWD_FROM_X_MASKED) {
+    Cursor cur(sh, h.piece);
+#pragma unroll
+    for (int k = 0; k < KEEP; ++k) {
+      if (cur.valid()) {
+        const size_t o = cur.template off<VEC>(sh.C, h.c, sh.HW);
+        h.a[k] = gate_by_mask(h.a[k], A.mask_in, o);
+        stv<VEC>(A.gated_out + o, h.a[k] * A.ralpha);
+      }
+      cur.next();
+    }
+  }
   float s0 = 0.f, s1 = 0.f;
   {
     const Gate gate = make_gate<MODE>(A, h.c);
@@ -560,7 +607,9 @@ __device__ __forceinline__ void finish_piece(const Args& A, const Held<VEC, KEEP
           setc(r, e, (gate(comp(h.a[k], e), d) - d * proj - gmean) * gscale);
         }
       }
-      stv<VEC>(A.out + cur.template off<VEC>(sh.C, h.c, sh.HW), r);
+      const size_t o = cur.template off<VEC>(sh.C, h.c, sh.HW);
+      stv<VEC>(A.out + o, r);
+      if (MODE == FWD_TRAIN_ADD && VEC == 4 && A.mask_out) put_mask(A.mask_out, o, r);
     }
     cur.next();
   }
@@ -663,7 +712,7 @@ static void fill_shape(int64_t N, int64_t C, int64_t HW, int vec, int64_t S, uin
   sh.HWV = (uint32_t)(HW / vec);
   sh.HW = (uint32_t)HW;
   sh.tot = (uint64_t)N * sh.HWV;
-  sh.L = L;
+  sh.L = L + (L & 1);  // even: a lane pair never straddles two pieces (put_mask)
   sh.G = 1;
 }
 
@@ -768,18 +817,21 @@ int bwd_launch(bool from_y, const float* dy, const float* t, const float* gamma,
                const float* invstd, float* dx, float* dgamma, float* dbeta, int64_t N, int64_t C,
                int64_t HW, void* ws, size_t ws_bytes, hipStream_t s, const Tuning& tune,
                bool relu = false, const float* relu_beta = nullptr,
-               const float* gate_ref = nullptr, float* gated_out = nullptr, float alpha = 1.f) {
+               const float* gate_ref = nullptr, float* gated_out = nullptr, float alpha = 1.f,
+               const uint8_t* mask_in = nullptr) {
   if (N < 0 || C < 0 || HW < 0) return MN_EINVAL;
   if (N == 0 || C == 0 || HW == 0) return MN_OK;
   if (!dy || !t || !invstd || !ws) return MN_EINVAL;
-  if ((gate_ref != nullptr) != (gated_out != nullptr)) return MN_EINVAL;
-  if (gate_ref && (from_y || relu || !dx)) return MN_EUNSUPPORTED;
+  if (gate_ref && mask_in) return MN_EINVAL;
+  if ((gate_ref != nullptr || mask_in != nullptr) != (gated_out != nullptr)) return MN_EINVAL;
+  if (gated_out && (from_y || relu || !dx)) return MN_EUNSUPPORTED;
   if (!shape_limits(N, C, HW)) return MN_EUNSUPPORTED;
   if (ws_bytes < ws_bytes_for(N, C, HW) || !mn_aligned(ws, 8)) return MN_EINVAL;
   Args A = {};
   const bool al = mn_aligned(dy, 16) && mn_aligned(t, 16) && (!dx || mn_aligned(dx, 16)) &&
                   mn_aligned(gate_ref, 16) && mn_aligned(gated_out, 16);
   A.gate_ref = gate_ref;
+  A.mask_in = mask_in;
   A.gated_out = gated_out;
   A.ralpha = alpha;
   A.a = dy;
@@ -795,6 +847,7 @@ int bwd_launch(bool from_y, const float* dy, const float* t, const float* gamma,
   A.rbeta = relu_beta;
   if (relu && from_y) return MN_EUNSUPPORTED;
   if (gate_ref) return run<BWD_FROM_X_GATED>(A, N, C, HW, al, ws, tune, s);
+  if (mask_in) return run<BWD_FROM_X_MASKED>(A, N, C, HW, al, ws, tune, s);
   return from_y ? run<BWD_FROM_Y>(A, N, C, HW, al, ws, tune, s)
                 : run<BWD_FROM_X>(A, N, C, HW, al, ws, tune, s);
 }
@@ -803,7 +856,7 @@ int fwd_train_launch(const float* x, const float* gamma, const float* beta, floa
                      float* running_var, float* y, float* save_mean, float* save_invstd, int64_t N,
                      int64_t C, int64_t HW, double momentum, double eps, void* ws, size_t ws_bytes,
                      hipStream_t s, const Tuning& tune, bool relu = false,
-                     const float* added = nullptr, float alpha = 1.f) {
+                     const float* added = nullptr, float alpha = 1.f, uint8_t* mask = nullptr) {
   if (N < 0 || C < 0 || HW < 0) return MN_EINVAL;
   if (N == 0 || C == 0 || HW == 0) return MN_OK;
   if (!x || !y || !save_mean || !save_invstd || !ws) return MN_EINVAL;
@@ -814,6 +867,7 @@ int fwd_train_launch(const float* x, const float* gamma, const float* beta, floa
   const double M = (double)N * (double)HW;
   A.a = added;
   A.ralpha = alpha;
+  A.mask_out = (al && HW % 8 == 0) ? mask : nullptr;  // else the caller packs y afterwards
   A.b = x;
   A.gamma = gamma;
   A.shift = beta;
@@ -851,7 +905,7 @@ int mn_bn_fwd_train_f32(const float* x, const float* gamma, const float* beta, f
 static int bn_fwd_apply(const float* x, const float* mean, const float* invstd, const float* gamma,
                         const float* beta, float* y, int64_t N, int64_t C, int64_t HW,
                         mn_stream_t stream, bool relu, const float* added = nullptr,
-                        float alpha = 1.f) {
+                        float alpha = 1.f, uint8_t* mask = nullptr) {
   using namespace mn_bn;
   if (N < 0 || C < 0 || HW < 0) return MN_EINVAL;
   if (N == 0 || C == 0 || HW == 0) return MN_OK;
@@ -875,6 +929,7 @@ static int bn_fwd_apply(const float* x, const float* mean, const float* invstd, 
   A.relu = relu ? 1 : 0;
   A.a = added;
   A.ralpha = alpha;
+  A.mask_out = (vec == 4 && HW % 8 == 0) ? mask : nullptr;
   const unsigned blocks = (unsigned)C * A.sh.S;
   hipStream_t s = mn_stream(stream);
   if (added) {
@@ -950,6 +1005,50 @@ int mn_bn_add_relu_bwd_f32(const float* dy, const float* x, const float* y, cons
   return mn_bn::bwd_launch(false, dy, x, gamma, mean, invstd, dx, dgamma, dbeta, N, C, HW, ws,
                            ws_bytes, mn_stream(stream), mn_bn::Tuning(), false, nullptr, y, dadded,
                            (float)alpha);
+}
+
+// Whether the forward kernels write the mask themselves (else mn_relu_fwd_mask_f32 packs y).
+static bool mask_in_kernel(const float* x, const float* y, const float* added, int64_t HW) {
+  return HW % 8 == 0 && mn_aligned(x, 16) && mn_aligned(y, 16) && mn_aligned(added, 16);
+}
+
+int mn_bn_add_relu_mask_fwd_train_f32(const float* x, const float* gamma, const float* beta,
+                                      float* running_mean, float* running_var, const float* added,
+                                      double alpha, float* y, uint8_t* mask, float* save_mean,
+                                      float* save_invstd, int64_t N, int64_t C, int64_t HW,
+                                      double momentum, double eps, void* ws, size_t ws_bytes,
+                                      mn_stream_t stream) {
+  if (N <= 0 || C <= 0 || HW <= 0) return (N < 0 || C < 0 || HW < 0) ? MN_EINVAL : MN_OK;
+  if (!added || !mask) return MN_EINVAL;
+  const int st = mn_bn::fwd_train_launch(x, gamma, beta, running_mean, running_var, y, save_mean,
+                                         save_invstd, N, C, HW, momentum, eps, ws, ws_bytes,
+                                         mn_stream(stream), mn_bn::Tuning(), true, added,
+                                         (float)alpha, mask);
+  if (st != MN_OK || mask_in_kernel(x, y, added, HW)) return st;
+  return mn_relu_fwd_mask_f32(y, nullptr, mask, (size_t)N * C * HW, stream);
+}
+
+int mn_bn_add_relu_mask_fwd_apply_f32(const float* x, const float* mean, const float* invstd,
+                                      const float* gamma, const float* beta, const float* added,
+                                      double alpha, float* y, uint8_t* mask, int64_t N, int64_t C,
+                                      int64_t HW, mn_stream_t stream) {
+  if (N <= 0 || C <= 0 || HW <= 0) return (N < 0 || C < 0 || HW < 0) ? MN_EINVAL : MN_OK;
+  if (!added || !mask) return MN_EINVAL;
+  const int st = bn_fwd_apply(x, mean, invstd, gamma, beta, y, N, C, HW, stream, true, added,
+                              (float)alpha, mask);
+  if (st != MN_OK || mask_in_kernel(x, y, added, HW)) return st;
+  return mn_relu_fwd_mask_f32(y, nullptr, mask, (size_t)N * C * HW, stream);
+}
+
+int mn_bn_add_relu_mask_bwd_f32(const float* dy, const float* x, const uint8_t* mask,
+                                const float* gamma, const float* mean, const float* invstd,
+                                double alpha, float* dx, float* dadded, float* dgamma,
+                                float* dbeta, int64_t N, int64_t C, int64_t HW, void* ws,
+                                size_t ws_bytes, mn_stream_t stream) {
+  if (N > 0 && C > 0 && HW > 0 && (!mean || !mask || !dadded || !dx)) return MN_EINVAL;
+  return mn_bn::bwd_launch(false, dy, x, gamma, mean, invstd, dx, dgamma, dbeta, N, C, HW, ws,
+                           ws_bytes, mn_stream(stream), mn_bn::Tuning(), false, nullptr, nullptr,
+                           dadded, (float)alpha, mask);
 }
 
 int mn_bn_relu_bwd_from_x_f32(const float* dy, const float* x, const float* gamma,

@@ -20,7 +20,8 @@ the saved invstd as is, so it reproduces the first forward bit for bit
 import torch
 
 from .. import _lib
-from .base import OP, InputStorage, OutputStorage, implements
+from .base import OP, InputStorage, IntermediateStorage, OutputStorage, implements
+from .relu import _numel
 
 
 def _as_nchw(t, name):
@@ -200,9 +201,14 @@ class InputActBatchNormReLU(_BatchNormForward):
 FUSED_BN_ADD_RELU = 'monet::batch_norm_add_relu'
 
 
+def _mask_like(t):
+    return torch.empty((t.numel() + 7) // 8, dtype=torch.uint8, device=t.device)
+
+
 def bn_add_relu_forward_train(x, weight, bias, running_mean, running_var, added, alpha, momentum,
-                              eps):
-    """Training forward of max(BN(x) + alpha*added, 0) -> (y, save_mean, save_invstd)."""
+                              eps, want_mask=False):
+    """Training forward of max(BN(x) + alpha*added, 0) -> (y, save_mean, save_invstd), with
+    `want_mask` -> (y, mask of y > 0, save_mean, save_invstd)."""
     xc, N, C, HW = _as_nchw(x, "input")
     ac, _, _, _ = _as_nchw(added, "added activation")
     if ac.shape != xc.shape:
@@ -211,6 +217,14 @@ def bn_add_relu_forward_train(x, weight, bias, running_mean, running_var, added,
     save_mean = torch.empty(C, dtype=torch.float32, device=x.device)
     save_invstd = torch.empty(C, dtype=torch.float32, device=x.device)
     ws, nbytes = _workspace(N, C, HW, x.device)
+    if want_mask:
+        mask = _mask_like(y)
+        _lib.call("mn_bn_add_relu_mask_fwd_train_f32", _lib.ptr(xc), _lib.ptr(weight),
+                  _lib.ptr(bias), _lib.ptr(running_mean), _lib.ptr(running_var), _lib.ptr(ac),
+                  float(alpha), _lib.ptr(y), _lib.ptr(mask), _lib.ptr(save_mean),
+                  _lib.ptr(save_invstd), N, C, HW, float(momentum), float(eps), _lib.ptr(ws), nbytes,
+                  _lib.stream_ptr(x.device))
+        return y, mask, save_mean, save_invstd
     _lib.call("mn_bn_add_relu_fwd_train_f32", _lib.ptr(xc), _lib.ptr(weight), _lib.ptr(bias),
               _lib.ptr(running_mean), _lib.ptr(running_var), _lib.ptr(ac), float(alpha), _lib.ptr(y),
               _lib.ptr(save_mean), _lib.ptr(save_invstd), N, C, HW, float(momentum), float(eps),
@@ -218,27 +232,50 @@ def bn_add_relu_forward_train(x, weight, bias, running_mean, running_var, added,
     return y, save_mean, save_invstd
 
 
-def bn_add_relu_forward_apply(x, mean, invstd, weight, bias, added, alpha):
-    """max((x - mean) * invstd * weight + bias + alpha*added, 0) with given per-channel vectors."""
+def bn_add_relu_forward_apply(x, mean, invstd, weight, bias, added, alpha, want_mask=False):
+    """max((x - mean) * invstd * weight + bias + alpha*added, 0) with given per-channel vectors
+    (`want_mask`: also the packed mask of the result > 0)."""
     xc, N, C, HW = _as_nchw(x, "input")
     ac, _, _, _ = _as_nchw(added, "added activation")
     if ac.shape != xc.shape:
         raise RuntimeError("the added activation must have the shape of the BatchNorm input")
     y = torch.empty_like(xc)
+    if want_mask:
+        mask = _mask_like(y)
+        _lib.call("mn_bn_add_relu_mask_fwd_apply_f32", _lib.ptr(xc), _lib.ptr(mean),
+                  _lib.ptr(invstd), _lib.ptr(weight), _lib.ptr(bias), _lib.ptr(ac), float(alpha),
+                  _lib.ptr(y), _lib.ptr(mask), N, C, HW, _lib.stream_ptr(x.device))
+        return y, mask
     _lib.call("mn_bn_add_relu_fwd_apply_f32", _lib.ptr(xc), _lib.ptr(mean), _lib.ptr(invstd),
               _lib.ptr(weight), _lib.ptr(bias), _lib.ptr(ac), float(alpha), _lib.ptr(y), N, C, HW,
               _lib.stream_ptr(x.device))
     return y
 
 
-def bn_add_relu_backward(grad, x, y, weight, save_mean, save_invstd, alpha):
-    """Backward of y = relu(BN(x) + alpha*added) from x and y in one pass ->
-    (dx, dweight, dbias, dadded).  `grad` is overwritten: dadded lives in its storage."""
+def bn_add_relu_backward(grad, x, y, weight, save_mean, save_invstd, alpha, mask=None):
+    """Backward of y = relu(BN(x) + alpha*added) from x and y (or, with `mask`, from x and the
+    packed mask of y > 0) in one pass -> (dx, dweight, dbias, dadded).  `grad` is overwritten:
+    dadded lives in its storage."""
     tc, N, C, HW = _as_nchw(x, "stored input")
-    yc, _, _, _ = _as_nchw(y, "stored output")
     g = grad if grad.is_contiguous() else grad.contiguous()
     _lib.require_gpu_tensor(g, "grad_output", torch.float32)
-    if g.shape != tc.shape or yc.shape != tc.shape:
+    if g.shape != tc.shape:
+        raise RuntimeError("grad_output and the stored activations differ in shape")
+    if mask is not None:
+        _lib.require_gpu_tensor(mask, "mask", torch.uint8)
+        if mask.numel() != (tc.numel() + 7) // 8:
+            raise RuntimeError("the mask does not have one bit per element")
+        dx = torch.empty_like(tc)
+        dw = torch.empty(C, dtype=torch.float32, device=x.device)
+        db = torch.empty(C, dtype=torch.float32, device=x.device)
+        ws, nbytes = _workspace(N, C, HW, x.device)
+        _lib.call("mn_bn_add_relu_mask_bwd_f32", _lib.ptr(g), _lib.ptr(tc), _lib.ptr(mask),
+                  _lib.ptr(weight), _lib.ptr(save_mean), _lib.ptr(save_invstd), float(alpha),
+                  _lib.ptr(dx), _lib.ptr(g), _lib.ptr(dw), _lib.ptr(db), N, C, HW, _lib.ptr(ws),
+                  nbytes, _lib.stream_ptr(x.device))
+        return dx, dw, db, g
+    yc, _, _, _ = _as_nchw(y, "stored output")
+    if yc.shape != tc.shape:
         raise RuntimeError("grad_output and the stored activations differ in shape")
     dx = torch.empty_like(tc)
     dw = torch.empty(C, dtype=torch.float32, device=x.device)
@@ -266,6 +303,7 @@ class InputActBatchNormAddReLU(OP):
     params = None   # (training, eps, save_mean, save_invstd, alpha)
     running_mean = None
     running_var = None
+    keeps_mask = False
 
     def forward(self, input_, weight, bias, running_mean, running_var, training, momentum, eps,
                 cudnn_enabled, added, alpha=1):
@@ -273,22 +311,26 @@ class InputActBatchNormAddReLU(OP):
             if self.running_mean is None and running_mean is not None:
                 self.running_mean = running_mean.requires_grad_(False)
                 self.running_var = running_var.requires_grad_(False)
+            m = self.keeps_mask
             if self.params is None:
                 if training:
-                    out, save_mean, save_invstd = bn_add_relu_forward_train(
+                    res = bn_add_relu_forward_train(
                         input_, weight, bias, self.running_mean, self.running_var, added, alpha,
-                        momentum, eps)
+                        momentum, eps, want_mask=m)
+                    out, save_mean, save_invstd = res[:-2], res[-2], res[-1]
                 else:
                     save_mean = self.running_mean
                     save_invstd = torch.rsqrt(self.running_var + eps)
                     out = bn_add_relu_forward_apply(input_, save_mean, save_invstd, weight, bias,
-                                                    added, alpha)
+                                                    added, alpha, want_mask=m)
+                    out = out if m else (out,)
                 self.params = bool(training), eps, save_mean, save_invstd, alpha
             else:
                 _, _, save_mean, save_invstd, _ = self.params
                 out = bn_add_relu_forward_apply(input_, save_mean, save_invstd, weight, bias, added,
-                                                alpha)
-            return out
+                                                alpha, want_mask=m)
+                out = out if m else (out,)
+            return tuple(out) if m else out[0]
 
     def backward(self, grad_output, stored, nodel=False):
         with torch.no_grad():
@@ -298,6 +340,28 @@ class InputActBatchNormAddReLU(OP):
                 raise NotImplementedError
             di, dw, db, da = bn_add_relu_backward(grad_output, input_, output, weight, save_mean,
                                                   save_invstd, alpha)
+            if not nodel:
+                del stored[5], stored[4], stored[3], stored[2], stored[1], stored[0]
+            return di, dw, db, None, None, da
+
+
+@implements([FUSED_BN_ADD_RELU], ['newnode', 'multiway_newnode', 'conv_multiway_newnode'])
+class BinaryActBatchNormAddReLU(InputActBatchNormAddReLU):
+    """The same operator keeping the BatchNorm input and a 1-bit mask of the output's sign
+    instead of the output: the forward writes the mask along with the output, the backward
+    reads gradient, input and mask (4 + 1/32 passes instead of 5)."""
+    backward_storage = [InputStorage(0, 1, 2, 3, 4),
+                        IntermediateStorage(lambda shape: (_numel(shape) + 7) // 8)]
+    keeps_mask = True
+
+    def backward(self, grad_output, stored, nodel=False):
+        with torch.no_grad():
+            input_, weight, bias, running_mean, running_var, mask = stored
+            training, eps, save_mean, save_invstd, alpha = self.params
+            if not training:
+                raise NotImplementedError
+            di, dw, db, da = bn_add_relu_backward(grad_output, input_, None, weight, save_mean,
+                                                  save_invstd, alpha, mask=mask)
             if not nodel:
                 del stored[5], stored[4], stored[3], stored[2], stored[1], stored[0]
             return di, dw, db, None, None, da

@@ -427,6 +427,44 @@ def test_bn_channel_too_large_to_keep_on_chip(cuda):
     assert_rel(host(db), odb, 1e-4, "dbeta")
 
 
+@pytest.mark.parametrize("alpha", [1, 0.5])
+@pytest.mark.parametrize("shape", BN_SHAPES + [(8, 6, 8, 8), (1, 2, 2100, 2048)])
+def test_bn_add_relu_with_mask_forward_backward_and_recompute(cuda, shape, alpha):
+    """The mask-keeping variant: same output as the output-keeping one bit for bit, mask =
+    packed sign of the GPU's own output, recomputation reproduces both, backward against the
+    oracle fed that output.  Shapes with planes of a multiple of 8 elements write the mask in
+    the BatchNorm kernel, the others in a second launch; the last shape runs the two-launch
+    formulation."""
+    x, gamma, beta, dy = bn_problem(shape, 12)
+    r = np.random.default_rng(13).standard_normal(shape).astype(np.float32)
+    tx, tw, tb, tg, tr = (dev(x, cuda), dev(gamma, cuda), dev(beta, cuda), dev(dy, cuda),
+                          dev(r, cuda))
+    C = shape[1]
+    rm, rv = torch.zeros(C, device=cuda), torch.ones(C, device=cuda)
+    rm0, rv0 = rm.clone(), rv.clone()
+    plain = lm_ops.bn.InputActBatchNormAddReLU()
+    y0 = plain.forward(tx, tw, tb, rm0, rv0, True, 0.1, 1e-5, True, tr, alpha)
+    op = lm_ops.bn.BinaryActBatchNormAddReLU()
+    y, mask = op.forward(tx, tw, tb, rm, rv, True, 0.1, 1e-5, True, tr, alpha)
+    assert torch.equal(y, y0) and torch.equal(rm, rm0) and torch.equal(rv, rv0)
+    assert mask.dtype == torch.uint8 and mask.numel() == (y.numel() + 7) // 8
+    assert np.array_equal(host(mask), O.pack_bits(host(y).ravel() > 0))
+    y2, mask2 = op.forward(tx, tw, tb, rm, rv, True, 0.1, 1e-5, True, tr, alpha)   # recomputation
+    assert_rel(host(y2), host(y), 2e-7, "recomputed output")
+    assert np.array_equal(host(mask2), O.pack_bits(host(y2).ravel() > 0))
+    assert torch.equal(rm, rm0)
+    _, omean, oinv, _, _ = O.bn_fwd_train(x, gamma, beta, None, None, 0.1, 1e-5)
+    odx, odg, odb, odr = O.bn_add_relu_bwd(dy, x, host(y), gamma, omean, oinv, alpha)
+    stored = [tx, tw, tb, rm, rv, mask]
+    dx, dg, db, n1, n2, dr = op.backward(tg.clone(), stored)
+    assert stored == [] and n1 is None and n2 is None
+    big = shape[2] * shape[3] > 1000000
+    assert_rel(host(dx), odx, 2e-5 if big else 1e-5, "dx")
+    assert_rel(host(dg), odg, 1e-4 if big else 3e-5, "dgamma")
+    assert_rel(host(db), odb, 1e-4 if big else 3e-5, "dbeta")
+    assert np.array_equal(host(dr), odr.astype(np.float32))
+
+
 def test_bn_add_relu_channel_too_large_to_keep_on_chip(cuda):
     # the fused end of a residual block on the two-launch (reduce, apply) formulation
     shape = (1, 2, 2100, 2048)
