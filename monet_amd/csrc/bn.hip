@@ -767,7 +767,9 @@ static int run(Args& A, int64_t N, int64_t C, int64_t HW, bool aligned16, void* 
     // waits while it holds two published pieces, both inside the lowest unfinished group or
     // later, so with at least kMaxResident workgroups running nobody can be left waiting as
     // long as a group has fewer than 2 * kMaxResident pieces.
-    A.sh.G = (int)(448 / rp < 1 ? 1 : (448 / rp > 8 ? 8 : 448 / rp));
+    // Not with one workgroup per CU (`wide`): a channel then completes G times later and nothing
+    // else on the CU covers the wait (64 x 112 x 112 at batch 184: 0.377 -> 0.454 ms with G = 3).
+    A.sh.G = wide ? 1 : (int)(448 / rp < 1 ? 1 : (448 / rp > 8 ? 8 : 448 / rp));
 #ifdef MN_TUNING
     if (const char* e = getenv("MN_BN_GROUP")) A.sh.G = atoi(e);
 #endif
