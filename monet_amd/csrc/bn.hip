@@ -755,7 +755,7 @@ static int run(Args& A, int64_t N, int64_t C, int64_t HW, bool aligned16, void* 
     return mn_launch_status();                                           \
   } while (0)
     if (vec == 4 && chan <= 256u * 9u) MN_BN_SOLO(4, 9, 256);
-    if (vec == 4 && chan <= 1024u * 9u) MN_BN_SOLO(4, 9, 1024);
+    if (vec == 4 && chan <= 1024u * 9u) MN_BN_SOLO(4, 18, 512);
     if (vec == 1 && chan <= 256u * 36u) MN_BN_SOLO(1, 36, 256);
 #undef MN_BN_SOLO
   }
