@@ -139,6 +139,26 @@ int mn_bn_bwd_from_x_f32(const float* dy, const float* x, const float* gamma, co
 int mn_bn_bwd_from_y_f32(const float* dy, const float* y, const float* gamma, const float* beta,
                          const float* invstd, float* dx, float* dgamma, float* dbeta, int64_t N,
                          int64_t C, int64_t HW, void* ws, size_t ws_bytes, mn_stream_t stream);
+/* The statistics-then-apply entry points above may run as ONE launch in which a
+ * workgroup waits (bounded) for the other workgroups of its channel.  If such a
+ * wait ever gives up (the device ran fewer workgroups at once than the launch
+ * relies on), every result derived from the missing totals is NaN and an error
+ * word in the workspace is raised; each launch clears the word first.
+ * mn_bn_ws_status waits for `stream`, reads the word left by the LAST launch
+ * that used `ws` for a tensor of this shape and returns MN_ELAUNCH if it is
+ * raised.  The reference's kernel (one block per channel, lrbn.cu:212-235)
+ * has no cross-block wait and so no counterpart of this call. */
+int mn_bn_ws_status(const void* ws, size_t ws_bytes, int64_t N, int64_t C, int64_t HW,
+                    mn_stream_t stream);
+/* mn_bn_bwd_from_y_f32 with the two launch limits given explicitly (0 = the
+ * default): `spin_limit` polls before a wait gives up, at most
+ * `max_workgroups` persistent workgroups.  For diagnosis and for testing the
+ * error path above from the host; no counterpart in the reference. */
+int mn_bn_bwd_from_y_f32_limits(const float* dy, const float* y, const float* gamma,
+                                const float* beta, const float* invstd, float* dx, float* dgamma,
+                                float* dbeta, int64_t N, int64_t C, int64_t HW, void* ws,
+                                size_t ws_bytes, uint32_t spin_limit, uint32_t max_workgroups,
+                                mn_stream_t stream);
 
 /* --------------------------------------------------------------- softmax --
  * The tensor is viewed as [outer, dim, inner]; softmax runs over `dim`.
@@ -273,11 +293,16 @@ typedef struct mn_conv2d {
  *                      tiles load as full 16-byte vectors; channel counts
  *                      that are not a multiple of 16 run it like variant 0.
  *                      Launches with few, long workgroups split the reduction
- *                      and add the slices with atomics (sums may then differ in
- *                      the last bits from run to run; variant 0 never does)
+ *                      in TWO and add the slices with atomics into a cleared
+ *                      output: 0 + a + b and 0 + b + a round identically, so
+ *                      the forward gives the same bits on every run (a
+ *                      recomputed forward must reproduce masks and indices)
  *   backward-data    0 implicit GEMM reading the weights through strides
  *                    1 same with the weights repacked [tap][k][c] (c padded
- *                      to a multiple of 128) into the workspace
+ *                      to a multiple of 128) into the workspace; may split
+ *                      the reduction up to 8 ways and add the slices with
+ *                      atomics (last bits can differ from run to run; variant
+ *                      0 never does)
  *   backward-weight  0 split reduction combined with atomics into a cleared dw
  *                    1 split reduction through per-split partials in the
  *                      workspace, then a fixed-order sum (reproducible) */

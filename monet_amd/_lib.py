@@ -6,7 +6,7 @@ caller gets an exception, never a fallback.
 import ctypes
 import os
 from ctypes import (POINTER, Structure, c_char_p, c_double, c_float, c_int, c_int32, c_int64,
-                    c_size_t, c_void_p)
+                    c_size_t, c_uint32, c_void_p)
 from pathlib import Path
 
 import torch
@@ -70,6 +70,9 @@ _SIGNATURES = {
                                      _P, c_size_t, _P]),
     "mn_bn_bwd_from_y_f32": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64,
                                      _P, c_size_t, _P]),
+    "mn_bn_bwd_from_y_f32_limits": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int64,
+                                            c_int64, _P, c_size_t, c_uint32, c_uint32, _P]),
+    "mn_bn_ws_status": (c_int, [_P, c_size_t, c_int64, c_int64, c_int64, _P]),
     "mn_bn_relu_fwd_train_f32": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64,
                                          c_double, c_double, _P, c_size_t, _P]),
     "mn_bn_relu_fwd_apply_f32": (c_int, [_P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, _P]),

@@ -22,8 +22,12 @@
 // counter when they start, so the items of a channel are held by workgroups
 // that are all running or about to be started in ticket order; the lowest
 // unfinished channel can always complete because at most S <= 256 workgroups
-// are needed at once and the device holds more than that.  A spin bound turns
-// a broken launch into wrong numbers instead of a hang.
+// are needed at once and the device holds more than that.  If that guarantee
+// is lost (fewer workgroups resident than a channel has pieces: a partitioned
+// or CU-masked device, another stream's kernel beside this one) a bounded wait
+// gives up: the totals of that piece become NaN, so every result derived from
+// them is NaN, and an error word in the workspace is set, which
+// mn_bn_ws_status() reports as MN_ELAUNCH.  Every workgroup still exits.
 //
 // Channels too large for S <= 256 resident pieces fall back to two launches
 // (reduce, then apply) that read the operands twice.
@@ -140,6 +144,8 @@ struct Args {
   float* partial;       // [C][S][2]
   float* pivot;         // [C], forward only
   uint32_t* ticket;     // resident launch only
+  uint32_t* error;      // set to 1 by a wait that gave up; cleared by every launch
+  uint32_t spin_limit;  // polls of one slot before the wait gives up
   float inv_m, unbias, momentum, eps;
   // Fused ReLU.  Forward: out = max(out, 0).  Backward from the input: the incoming gradient
   // is that of the ReLU output, so it only counts where the recomputed pre-activation
@@ -381,6 +387,7 @@ __global__ __launch_bounds__(kThreads) void bn_reduce_kernel(const Args A) {
   const int piece = blockIdx.x - c * A.sh.S;
   const float sft = reduce_shift<MODE>(A, c);
   if (is_fwd(MODE) && piece == 0 && threadIdx.x == 0) A.pivot[c] = sft;
+  if (blockIdx.x == 0 && threadIdx.x == 0) *A.error = 0u;  // this formulation never waits
   float s0, s1;
   reduce_piece<VEC, MODE>(A, c, piece, sft, s0, s1);
   block_sum2<kWaves>(s0, s1, lds);
@@ -420,10 +427,14 @@ __global__ __launch_bounds__(kThreads) void bn_fwd_saved_kernel(const Args A, co
 // slots hold kEmptySlot, which publish() never writes.
 constexpr uint64_t kEmptySlot = 0xFFFFFFFFFFFFFFFFull;
 
-__global__ void bn_prepare_kernel(uint64_t* slots, uint32_t nslots, uint32_t* ticket) {
+__global__ void bn_prepare_kernel(uint64_t* slots, uint32_t nslots, uint32_t* ticket,
+                                  uint32_t* error) {
   const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < nslots) slots[i] = kEmptySlot;
-  if (i == 0) *ticket = 0u;
+  if (i == 0) {
+    *ticket = 0u;
+    *error = 0u;
+  }
 }
 
 __device__ __forceinline__ void publish(uint64_t* slot, float s0, float s1) {
@@ -438,7 +449,7 @@ constexpr int kMaxResident = 256;  // most pieces per channel in the resident fo
 // a fixed order (lane l takes slots l, l+64, ..; then a lane tree) and hands
 // the totals to the workgroup through `lds`.
 __device__ __forceinline__ void gather_totals(const uint64_t* slots, int S, float* lds, float& t0,
-                                              float& t1) {
+                                              float& t1, uint32_t spin_limit, uint32_t* error) {
   if (threadIdx.x < MN_WAVE) {
     const int lane = threadIdx.x;
     float p0 = 0.f, p1 = 0.f;
@@ -446,12 +457,17 @@ __device__ __forceinline__ void gather_totals(const uint64_t* slots, int S, floa
       uint64_t w;
       uint32_t spins = 0;
       // The pieces polled here are published or held by running workgroups that publish
-      // before they wait, so this ends; the bound only keeps a broken launch from hanging
-      // the device (the results are then wrong).
+      // before they wait, so this ends.  Should that guarantee ever be lost, the bound ends
+      // the wait anyway: the slot then counts as (NaN, NaN), which poisons everything computed
+      // from these totals, and the workspace's error word is raised.
       while ((w = __hip_atomic_load(slots + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) ==
                  kEmptySlot &&
-             ++spins < (1u << 22))
+             ++spins < spin_limit)
         __builtin_amdgcn_s_sleep(1);
+      if (w == kEmptySlot) {
+        w = 0x7FC000007FC00000ull;
+        __hip_atomic_store(error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
       p0 += __uint_as_float((uint32_t)w);
       p1 += __uint_as_float((uint32_t)(w >> 32));
     }
@@ -584,7 +600,8 @@ __device__ __forceinline__ void finish_piece(const Args& A, const Held<VEC, KEEP
   float t0 = h.t0, t1 = h.t1;
   if (!SOLO) {
     __syncthreads();  // lds is free again
-    gather_totals(reinterpret_cast<uint64_t*>(A.partial) + (size_t)h.c * sh.S, sh.S, lds, t0, t1);
+    gather_totals(reinterpret_cast<uint64_t*>(A.partial) + (size_t)h.c * sh.S, sh.S, lds, t0, t1,
+                  A.spin_limit, A.error);
   }
   float s_, proj, gmean, gscale;
   coefficients<MODE>(A, h.c, h.piece, t0, t1, h.sft, s_, proj, gmean, gscale);
@@ -655,6 +672,7 @@ template <int VEC, int MODE, int KEEP, int THREADS>
 __global__ __launch_bounds__(THREADS) void bn_solo_kernel(const Args A) {
   __shared__ float lds[2 * (THREADS / MN_WAVE)];
   Held<VEC, KEEP> h;
+  if (blockIdx.x == 0 && threadIdx.x == 0) *A.error = 0u;  // nothing here ever waits
   // Planes this short do not end on cache-line boundaries: neighbouring channels share their
   // first and last lines.  Each XCD takes a contiguous range of channels, so the shared lines
   // meet in one L2 instead of being fetched (and written back in parts) by two.
@@ -674,6 +692,7 @@ struct Tuning {
   int keep = 8;              // vectors kept per thread, tensor and piece (two pieces in flight)
   int threads = 256;         // workgroup size of the resident kernel
   int grid = 768;            // persistent workgroups of the resident kernel (3 per CU)
+  uint32_t spin_limit = 1u << 22;  // polls of one slot (seconds) before a wait gives up
 };
 
 static bool shape_limits(int64_t N, int64_t C, int64_t HW) {
@@ -724,6 +743,8 @@ static int run(Args& A, int64_t N, int64_t C, int64_t HW, bool aligned16, void* 
   uint32_t* counters = reinterpret_cast<uint32_t*>(A.partial + ws_floats(N, C, HW));
   A.pivot = reinterpret_cast<float*>(counters) - C;  // last C floats of the float area
   A.ticket = counters;
+  A.error = counters + 1;
+  A.spin_limit = t.spin_limit ? t.spin_limit : 1u;
   int keep = t.keep > 0 ? t.keep : 8, threads = t.threads > 0 ? t.threads : kThreads;
   // The forward holds one tensor per piece: 512-thread workgroups (pieces twice as long, half as
   // many partials to publish and poll) measured 7-20 % faster on every ResNet-50 shape at batch
@@ -743,9 +764,6 @@ static int run(Args& A, int64_t N, int64_t C, int64_t HW, bool aligned16, void* 
   // whole channels in one workgroup's registers
   const uint64_t chan = (uint64_t)N * (HW / vec);
   bool solo = t.resident && t.keep == 8 && t.threads == kThreads;
-#ifdef MN_TUNING
-  if (const char* e = getenv("MN_BN_SOLO")) solo = solo && atoi(e) != 0;
-#endif
   if (solo) {
     const unsigned grid = (unsigned)(C < 65535 ? C : 65535);
 #define MN_BN_SOLO(V, K, T)                                              \
@@ -770,26 +788,15 @@ static int run(Args& A, int64_t N, int64_t C, int64_t HW, bool aligned16, void* 
     // Not with one workgroup per CU (`wide`): a channel then completes G times later and nothing
     // else on the CU covers the wait (64 x 112 x 112 at batch 184: 0.377 -> 0.454 ms with G = 3).
     A.sh.G = wide ? 1 : (int)(448 / rp < 1 ? 1 : (448 / rp > 8 ? 8 : 448 / rp));
-#ifdef MN_TUNING
-    if (const char* e = getenv("MN_BN_GROUP")) A.sh.G = atoi(e);
-#endif
     bn_prepare_kernel<<<(blocks + 255) / 256, 256, 0, s>>>(
-          reinterpret_cast<uint64_t*>(A.partial), blocks, A.ticket);
+          reinterpret_cast<uint64_t*>(A.partial), blocks, A.ticket, A.error);
     // persistent grid: enough workgroups to fill 256 CUs at this register footprint
     // (512-thread workgroups: one per CU at this register footprint)
-    const unsigned want = wide ? 256u : (unsigned)t.grid;
+    const unsigned want = (wide && t.grid > 256) ? 256u : (unsigned)t.grid;
     const unsigned grid = blocks < want ? blocks : want;
 #define MN_BN_RES(V, K, T) bn_resident_kernel<V, MODE, K, T><<<grid, T, 0, s>>>(A, blocks)
     if (vec == 4) {
       if (wide || long_pieces) MN_BN_RES(4, 8, 512);
-#ifdef MN_TUNING
-      else if (keep == 8 && threads == 256) MN_BN_RES(4, 8, 256);
-      else if (keep == 4 && threads == 512) MN_BN_RES(4, 4, 512);
-      else if (keep == 8 && threads == 512) MN_BN_RES(4, 8, 512);
-      else if (keep == 4 && threads == 1024) MN_BN_RES(4, 4, 1024);
-      else if (keep == 16 && threads == 256) MN_BN_RES(4, 16, 256);
-      else if (keep == 12 && threads == 256) MN_BN_RES(4, 12, 256);
-#endif
       else MN_BN_RES(4, 8, 256);
     } else {
       MN_BN_RES(1, 16, 256);
@@ -1077,23 +1084,31 @@ int mn_bn_bwd_from_y_f32(const float* dy, const float* y, const float* gamma, co
                            ws_bytes, mn_stream(stream), mn_bn::Tuning());
 }
 
-}  // extern "C"
-
-#ifdef MN_TUNING
-// Only in tuning builds: the backward-from-output with explicit launch tunables.
-extern "C" int mn_tune_bn_bwd_from_y(const float* dy, const float* y, const float* gamma,
-                                     const float* beta, const float* invstd, float* dx,
-                                     float* dgamma, float* dbeta, int64_t N, int64_t C, int64_t HW,
-                                     void* ws, size_t ws_bytes, mn_stream_t stream,
-                                     int target_blocks, int resident, int keep, int threads,
-                                     int grid) {
+int mn_bn_bwd_from_y_f32_limits(const float* dy, const float* y, const float* gamma,
+                                const float* beta, const float* invstd, float* dx, float* dgamma,
+                                float* dbeta, int64_t N, int64_t C, int64_t HW, void* ws,
+                                size_t ws_bytes, uint32_t spin_limit, uint32_t max_workgroups,
+                                mn_stream_t stream) {
   mn_bn::Tuning t;
-  t.target_blocks = target_blocks;
-  t.resident = resident;
-  t.keep = keep;
-  t.threads = threads;
-  t.grid = grid;
+  if (spin_limit) t.spin_limit = spin_limit;
+  if (max_workgroups) t.grid = (int)(max_workgroups < 65535u ? max_workgroups : 65535u);
   return mn_bn::bwd_launch(true, dy, y, gamma, beta, invstd, dx, dgamma, dbeta, N, C, HW, ws,
                            ws_bytes, mn_stream(stream), t);
 }
-#endif
+
+int mn_bn_ws_status(const void* ws, size_t ws_bytes, int64_t N, int64_t C, int64_t HW,
+                    mn_stream_t stream) {
+  if (N <= 0 || C <= 0 || HW <= 0) return (N < 0 || C < 0 || HW < 0) ? MN_EINVAL : MN_OK;
+  if (!ws || !mn_bn::shape_limits(N, C, HW) || ws_bytes < mn_bn::ws_bytes_for(N, C, HW))
+    return MN_EINVAL;
+  const char* word = static_cast<const char*>(ws) + mn_bn::ws_floats(N, C, HW) * sizeof(float) +
+                     sizeof(uint32_t);
+  uint32_t raised = 0;
+  hipStream_t s = mn_stream(stream);
+  if (hipMemcpyAsync(&raised, word, sizeof(raised), hipMemcpyDeviceToHost, s) != hipSuccess ||
+      hipStreamSynchronize(s) != hipSuccess)
+    return MN_ELAUNCH;
+  return raised ? MN_ELAUNCH : MN_OK;
+}
+
+}  // extern "C"

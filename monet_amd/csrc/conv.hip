@@ -22,9 +22,6 @@
 // the global loads of tile t+1 are in flight while tile t is multiplied.
 #include "common.h"
 #include <type_traits>
-#ifdef MN_TUNING
-#include <cstdlib>
-#endif
 
 // bf16 / channels-last kernels (conv_bf16.hip)
 int mn_conv16_ws_bytes(const mn_conv2d* g, int direction, size_t* bytes);
@@ -1184,15 +1181,10 @@ static void tile_dims(int tile, int* bm, int* bn);
 // Few, long workgroups quantise badly over 256 CUs (2.2 per CU run as 3 rounds): when a
 // launch has fewer than ~6 workgroups per CU, a long reduction and a dense output, slice the
 // reduction so that there are ~8 per CU and add the slices into a cleared output.
-static void plan_split(Gather& g, int tile, bool allow) {
+static void plan_split(Gather& g, int tile, bool allow, int max_split) {
   g.ksplit = 1;
   g.tiles_per_split = 0;
   if (!allow || g.osh != 1 || g.osw != 1) return;
-#ifdef MN_TUNING
-  if (const char* e = getenv("MN_CONV_SPLIT")) {
-    if (atoi(e) <= 1) return;
-  }
-#endif
   int bm, bn;
   tile_dims(tile, &bm, &bn);
   const long long wgs = ((long long)(g.ncols + bn - 1) / bn) * ((g.M + bm - 1) / bm);
@@ -1200,10 +1192,7 @@ static void plan_split(Gather& g, int tile, bool allow) {
   if (wgs >= 6 * 256 || ktiles < 32) return;
   int want = (int)((8 * 256 + wgs - 1) / wgs);
   if (want > ktiles / 16) want = ktiles / 16;  // at least 16 k-tiles per slice
-  if (want > 8) want = 8;
-#ifdef MN_TUNING
-  if (const char* e = getenv("MN_CONV_SPLIT")) want = atoi(e);
-#endif
+  if (want > max_split) want = max_split;
   if (want <= 1) return;
   g.tiles_per_split = (ktiles + want - 1) / want;
   g.ksplit = (ktiles + g.tiles_per_split - 1) / g.tiles_per_split;
@@ -1214,18 +1203,15 @@ static void plan_split(Gather& g, int tile, bool allow) {
 // `split_ok`: the caller allows a split reduction (dst is then cleared here first).
 static void launch_gather(Gather g, const float* a, const float* src, const float* bias,
                           float* dst, hipStream_t s, bool packed = false, bool split_ok = false,
-                          int tile = -1) {
+                          int max_split = 8, int tile = -1) {
   if (g.ncols == 0 || g.M == 0) return;
   if (fast_path(g)) g.src_bytes = (uint32_t)((size_t)g.N * g.Cs * g.Hs * g.Ws * sizeof(float));
   g.divOHW = make_fastdiv((uint32_t)(g.OH * g.OW));
   g.divOW = make_fastdiv((uint32_t)g.OW);
   // multiplication by the reciprocal is exact while dividend * divisor < 2^32
   g.exact_div = ((unsigned long long)(g.ncols + 256) * (unsigned long long)(g.OH * g.OW) >= (1ull << 32)) ? 1 : 0;
-#ifdef MN_TUNING
-  if (const char* e = getenv("MN_CONV_TILE")) tile = atoi(e);
-#endif
   if (tile < 0) tile = pick_tile(g.M, g.ncols, fast_path(g), packed);
-  plan_split(g, tile, split_ok && packed);
+  plan_split(g, tile, split_ok && packed, max_split);
   // Tap after tap over ALL channels re-reads each pixel once per tap with the whole channel
   // range in between, far more than an L2 holds across the workgroups of an XCD.  Cycling the
   // taps over a block of 2-4 k-tiles keeps the re-reads in cache; shorter blocks re-enter taps
@@ -1250,9 +1236,6 @@ static void launch_gather(Gather g, const float* a, const float* src, const floa
 
 // Split of the (n, p, q) reduction: enough workgroups for ~2 per CU.
 static int wgrad_tile(const mn_conv2d* g, int variant) {
-#ifdef MN_TUNING
-  if (const char* e = getenv("MN_WGRAD_TILE")) return atoi(e);
-#endif
   // from the same sweeps: 128 x 128 for windows, 128 x 64 for 1x1 filters, 64 rows for K <= 64
   const long long ncols = (long long)g->C * g->R * g->S;
   int tile;
@@ -1271,9 +1254,6 @@ static int wgrad_tile(const mn_conv2d* g, int variant) {
   return tile;
 }
 static bool wgrad_tap_major(const mn_conv2d* g, int bm, int bn) {
-#ifdef MN_TUNING
-  if (const char* e = getenv("MN_WGRAD_TAP")) return atoi(e) != 0 && g->C % bn == 0 && g->K % bm == 0;
-#endif
   return g->C % bn == 0 && g->K % bm == 0;
 }
 static void tile_dims(int tile, int* bm, int* bn) {
@@ -1301,9 +1281,6 @@ static void wgrad_split(const mn_conv2d* g, int variant, int* splits, int* tiles
   const bool tap = wgrad_tap_major(g, bm, bn) && (variant == 1 || g->R * g->S == 1);
   const int per_cu = tile == 0 ? (tap ? 3 : 2) : (tile == 4 ? 4 : 3);
   long long slots = 256ll * per_cu;
-#ifdef MN_TUNING
-  if (const char* e = getenv("MN_WGRAD_SLOTS")) slots = atoll(e);
-#endif
   long long want = slots / out_tiles;  // rounded down: never a partial extra round
   if (want > total_tiles) want = total_tiles;
   if (want > 256) want = 256;
@@ -1407,7 +1384,11 @@ int mn_conv_fwd(const mn_conv2d* g, const void* x, const void* w, const void* bi
     q.lda = Mp;
     q.a_bytes = (uint32_t)(n * sizeof(float));
   }
-  launch_gather(q, a, (const float*)x, (const float*)bias, (float*)y, s, packed, packed);
+  // A forward may be run again by a schedule that recomputes it, and what follows (a ReLU mask,
+  // max-pool indices) must then come out bit for bit the same.  With two slices the atomic
+  // additions into the cleared output give the same bits in either order (0 + a + b and
+  // 0 + b + a round identically); with more they would not.
+  launch_gather(q, a, (const float*)x, (const float*)bias, (float*)y, s, packed, packed, 2);
   return mn_launch_status();
 }
 
@@ -1594,9 +1575,6 @@ static int conv_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, vo
     const bool veca = ((long long)g->P * g->Q) % 4 == 0 && mn_aligned(dy, 16) && (!vecb || mn_aligned(x, 16));
     bool rows = (long long)g->P * g->Q >= 32 && 32 / g->Q + 1 <= g->P &&
                 dy_bytes < (1ull << 31) && x_bytes < (1ull << 31);  // buffer offsets below 2^31
-#ifdef MN_TUNING
-    if (const char* e = getenv("MN_WGRAD_ROWS")) rows = rows && atoi(e) != 0;
-#endif
     if (rows) {
 #define MN_ROWS_V(TL, D, B, V)                                                                   \
   if (veca)                                                                                      \
@@ -1629,9 +1607,6 @@ static int conv_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, vo
 #undef MN_ROWS_V
     } else {
     int deep = tile == 0 ? 16 : 32;  // 128 x 128 at depth 32 leaves LDS for 2 workgroups per CU only
-#ifdef MN_TUNING
-    if (const char* e = getenv("MN_WGRAD_DEPTH")) deep = atoi(e);
-#endif
 #define MN_TAP_D(TL, D)                                                                           \
   if (db)                                                                                         \
     wgrad_tap_kernel<TL, D, true><<<grid, kThreads, 0, s>>>(q, (const float*)dy, (const float*)x, \

@@ -446,8 +446,9 @@ int mn_maxpool_bwd_idx_f32(const mn_pool2d* g, const float* dy, const uint8_t* i
   if ((size_t)g->N * g->C == 0) return MN_OK;
   if (!dy || !dx || !idx4) return MN_EINVAL;
   hipStream_t s = mn_stream(stream);
-  if (is_ct(g, 3, 2, 1) && g->H % 2 == 0 && g->W % 4 == 0 && mn_aligned(dx, 16) &&
-      mn_aligned(dy, 8) && g->W / 4 <= kThreads)
+  // the fast kernel assumes pooled planes of exactly H/2 x W/2 (ceil_mode can add a row)
+  if (is_ct(g, 3, 2, 1) && g->H % 2 == 0 && g->W % 4 == 0 && g->PH == g->H / 2 &&
+      g->PW == g->W / 2 && mn_aligned(dx, 16) && mn_aligned(dy, 8) && g->W / 4 <= kThreads)
     maxpool_bwd_k3s2p1_kernel<<<(unsigned)g->N * g->C, kThreads, 0, s>>>(dy, idx4, dx, g->H, g->W);
   else if (is_ct(g, 3, 2, 1))
     launch_bwd(CtGeo<3, 2, 1>{}, g, dy, idx4, dx, s);

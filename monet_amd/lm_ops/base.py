@@ -54,6 +54,10 @@ class OP:
     """
     names: List[str] = []
     backward_storage: Optional[Union[StorageInfo, List[StorageInfo]]] = None
+    # True: `backward` writes into the storage of the gradient it is given (the reference's
+    # ReLU backward does, lrrelu.cpp:14-15).  The executor hands such an operator a private
+    # copy when another pending gradient still shares that storage.
+    overwrites_grad = False
 
     def intermediate(self, *args, **kwargs):
         return None

@@ -17,6 +17,8 @@ saved statistics without touching the running ones.  The recomputation uses
 the saved invstd as is, so it reproduces the first forward bit for bit
 (the reference's F.batch_norm call at bn.py:32-34 adds eps a second time).
 """
+import os
+
 import torch
 
 from .. import _lib
@@ -39,6 +41,19 @@ def _workspace(N, C, HW, device):
     return torch.empty(max(nbytes, 4), dtype=torch.uint8, device=device), nbytes
 
 
+# True (or MONET_AMD_CHECK_BN_WAITS=1 in the environment): after every BatchNorm call that
+# used a workspace, wait for it and raise if one of its workgroups gave up waiting for the
+# others (the results are NaN then).  Costs a device synchronisation per call: for diagnosis.
+check_waits = os.environ.get("MONET_AMD_CHECK_BN_WAITS", "0") not in ("", "0")
+
+
+def _ws_call(ws_shape, name, *args):
+    _lib.call(name, *args)
+    if check_waits:
+        ws, nbytes, N, C, HW = ws_shape
+        _lib.call("mn_bn_ws_status", _lib.ptr(ws), nbytes, N, C, HW, args[-1])
+
+
 def bn_forward_train(x, weight, bias, running_mean, running_var, momentum, eps, out=None,
                      relu=False):
     """Training forward -> (y, save_mean, save_invstd); relu=True applies max(., 0) to y."""
@@ -47,7 +62,7 @@ def bn_forward_train(x, weight, bias, running_mean, running_var, momentum, eps, 
     save_mean = torch.empty(C, dtype=torch.float32, device=x.device)
     save_invstd = torch.empty(C, dtype=torch.float32, device=x.device)
     ws, nbytes = _workspace(N, C, HW, x.device)
-    _lib.call("mn_bn_relu_fwd_train_f32" if relu else "mn_bn_fwd_train_f32", _lib.ptr(xc), _lib.ptr(weight), _lib.ptr(bias),
+    _ws_call((ws, nbytes, N, C, HW), "mn_bn_relu_fwd_train_f32" if relu else "mn_bn_fwd_train_f32", _lib.ptr(xc), _lib.ptr(weight), _lib.ptr(bias),
               _lib.ptr(running_mean), _lib.ptr(running_var), _lib.ptr(y), _lib.ptr(save_mean),
               _lib.ptr(save_invstd), N, C, HW, float(momentum), float(eps), _lib.ptr(ws), nbytes,
               _lib.stream_ptr(x.device))
@@ -74,7 +89,7 @@ def _bn_backward(entry, grad, t, weight, shift, invstd):
     dw = torch.empty(C, dtype=torch.float32, device=t.device)
     db = torch.empty(C, dtype=torch.float32, device=t.device)
     ws, nbytes = _workspace(N, C, HW, t.device)
-    _lib.call(entry, _lib.ptr(g), _lib.ptr(tc), _lib.ptr(weight), _lib.ptr(shift),
+    _ws_call((ws, nbytes, N, C, HW), entry, _lib.ptr(g), _lib.ptr(tc), _lib.ptr(weight), _lib.ptr(shift),
               _lib.ptr(invstd), _lib.ptr(dx), _lib.ptr(dw), _lib.ptr(db), N, C, HW, _lib.ptr(ws),
               nbytes, _lib.stream_ptr(t.device))
     return dx, dw, db
@@ -92,7 +107,7 @@ def bn_relu_backward_from_input(grad, x, weight, bias, save_mean, save_invstd):
     dw = torch.empty(C, dtype=torch.float32, device=x.device)
     db = torch.empty(C, dtype=torch.float32, device=x.device)
     ws, nbytes = _workspace(N, C, HW, x.device)
-    _lib.call("mn_bn_relu_bwd_from_x_f32", _lib.ptr(g), _lib.ptr(tc), _lib.ptr(weight), _lib.ptr(bias),
+    _ws_call((ws, nbytes, N, C, HW), "mn_bn_relu_bwd_from_x_f32", _lib.ptr(g), _lib.ptr(tc), _lib.ptr(weight), _lib.ptr(bias),
               _lib.ptr(save_mean), _lib.ptr(save_invstd), _lib.ptr(dx), _lib.ptr(dw), _lib.ptr(db),
               N, C, HW, _lib.ptr(ws), nbytes, _lib.stream_ptr(x.device))
     return dx, dw, db
@@ -219,13 +234,13 @@ def bn_add_relu_forward_train(x, weight, bias, running_mean, running_var, added,
     ws, nbytes = _workspace(N, C, HW, x.device)
     if want_mask:
         mask = _mask_like(y)
-        _lib.call("mn_bn_add_relu_mask_fwd_train_f32", _lib.ptr(xc), _lib.ptr(weight),
+        _ws_call((ws, nbytes, N, C, HW), "mn_bn_add_relu_mask_fwd_train_f32", _lib.ptr(xc), _lib.ptr(weight),
                   _lib.ptr(bias), _lib.ptr(running_mean), _lib.ptr(running_var), _lib.ptr(ac),
                   float(alpha), _lib.ptr(y), _lib.ptr(mask), _lib.ptr(save_mean),
                   _lib.ptr(save_invstd), N, C, HW, float(momentum), float(eps), _lib.ptr(ws), nbytes,
                   _lib.stream_ptr(x.device))
         return y, mask, save_mean, save_invstd
-    _lib.call("mn_bn_add_relu_fwd_train_f32", _lib.ptr(xc), _lib.ptr(weight), _lib.ptr(bias),
+    _ws_call((ws, nbytes, N, C, HW), "mn_bn_add_relu_fwd_train_f32", _lib.ptr(xc), _lib.ptr(weight), _lib.ptr(bias),
               _lib.ptr(running_mean), _lib.ptr(running_var), _lib.ptr(ac), float(alpha), _lib.ptr(y),
               _lib.ptr(save_mean), _lib.ptr(save_invstd), N, C, HW, float(momentum), float(eps),
               _lib.ptr(ws), nbytes, _lib.stream_ptr(x.device))
@@ -269,7 +284,7 @@ def bn_add_relu_backward(grad, x, y, weight, save_mean, save_invstd, alpha, mask
         dw = torch.empty(C, dtype=torch.float32, device=x.device)
         db = torch.empty(C, dtype=torch.float32, device=x.device)
         ws, nbytes = _workspace(N, C, HW, x.device)
-        _lib.call("mn_bn_add_relu_mask_bwd_f32", _lib.ptr(g), _lib.ptr(tc), _lib.ptr(mask),
+        _ws_call((ws, nbytes, N, C, HW), "mn_bn_add_relu_mask_bwd_f32", _lib.ptr(g), _lib.ptr(tc), _lib.ptr(mask),
                   _lib.ptr(weight), _lib.ptr(save_mean), _lib.ptr(save_invstd), float(alpha),
                   _lib.ptr(dx), _lib.ptr(g), _lib.ptr(dw), _lib.ptr(db), N, C, HW, _lib.ptr(ws),
                   nbytes, _lib.stream_ptr(x.device))
@@ -281,7 +296,7 @@ def bn_add_relu_backward(grad, x, y, weight, save_mean, save_invstd, alpha, mask
     dw = torch.empty(C, dtype=torch.float32, device=x.device)
     db = torch.empty(C, dtype=torch.float32, device=x.device)
     ws, nbytes = _workspace(N, C, HW, x.device)
-    _lib.call("mn_bn_add_relu_bwd_f32", _lib.ptr(g), _lib.ptr(tc), _lib.ptr(yc), _lib.ptr(weight),
+    _ws_call((ws, nbytes, N, C, HW), "mn_bn_add_relu_bwd_f32", _lib.ptr(g), _lib.ptr(tc), _lib.ptr(yc), _lib.ptr(weight),
               _lib.ptr(save_mean), _lib.ptr(save_invstd), float(alpha), _lib.ptr(dx), _lib.ptr(g),
               _lib.ptr(dw), _lib.ptr(db), N, C, HW, _lib.ptr(ws), nbytes, _lib.stream_ptr(x.device))
     return dx, dw, db, g
@@ -304,6 +319,7 @@ class InputActBatchNormAddReLU(OP):
     running_mean = None
     running_var = None
     keeps_mask = False
+    overwrites_grad = True   # the gradient of `added` is written over the incoming gradient
 
     def forward(self, input_, weight, bias, running_mean, running_var, training, momentum, eps,
                 cudnn_enabled, added, alpha=1):

@@ -28,6 +28,14 @@ from .base import OP, InputStorage, implements
 DEFAULT_VARIANT = 0
 
 
+def _refused(exc):
+    """True when a kernel variant was refused before anything was launched (unknown index,
+    shape it does not cover): the only failures the operators answer by running variant 0.
+    Launch failures, host-side shape / dtype errors and allocator failures propagate."""
+    return isinstance(exc, _lib.MonetHipError) and exc.status in (_lib.MN_EUNSUPPORTED,
+                                                                  _lib.MN_EINVAL)
+
+
 def _pair(v):
     v = list(v) if isinstance(v, (list, tuple, torch.Size)) else [v]
     if len(v) == 1:
@@ -169,7 +177,15 @@ def _depthwise_forward(input_, weight, bias, stride, padding, dilation, groups):
                                       list(dilation), False, [0, 0], groups)
 
 
-def _depthwise_backward(grad, input_, weight, stride, padding, dilation, groups, mask):
+def _depthwise_backward(grad, input_, weight, stride, padding, dilation, groups, mask,
+                        input_shape=None):
+    """(di, dw) of a grouped convolution through aten.  `mask` says which of the two to
+    compute; an input the executor has already dropped (input-gradient step of a split
+    backward) is replaced by a shape-only stand-in, which is all aten reads of it then."""
+    if input_ is None:
+        assert not mask[1] and input_shape is not None
+        input_ = torch.empty(1, dtype=grad.dtype, device=grad.device).expand(
+            [int(d) for d in input_shape])
     di, dw, _ = torch.ops.aten.convolution_backward(
         grad, input_, weight, None, list(stride), list(padding), list(dilation), False, [0, 0],
         groups, [bool(mask[0]), bool(mask[1]), False])
@@ -222,9 +238,22 @@ class _ConvBase(OP):
                 del stored[1]
                 del stored[0]
             di = dw = db = None
-            if self.is_depthwise or groups != 1:
+            if self.is_depthwise:
+                # one backward step computes everything (conv.py:301-302 in the reference)
                 di, dw = _depthwise_backward(grad_output, input_, weight, stride, padding, dilation,
                                              groups, do_grad[:2])
+                if do_grad[2]:
+                    db = grad_output.sum([0, 2, 3])
+            elif groups != 1:
+                # grouped, not depthwise: split like every other convolution (kind 0: parameter
+                # gradients, 1: input gradient, 2: both), the arithmetic is aten's
+                want_di = kind in (1, 2) and do_grad[0] and weight is not None
+                want_dw = kind in (0, 2) and do_grad[1] and input_ is not None
+                if want_di or want_dw:
+                    di, dw = _depthwise_backward(grad_output, input_, weight, stride, padding,
+                                                 dilation, groups, [want_di, want_dw], input_shape)
+                if kind in (0, 2) and do_grad[2]:
+                    db = grad_output.sum([0, 2, 3])
             else:
                 if kind in (0, 2) and input_ is not None:
                     if do_grad[1] and do_grad[2]:
@@ -257,7 +286,9 @@ class SpecificAlgoConvolution(_ConvBase):
         try:
             return conv_forward(input_, weight, bias, padding, stride, dilation, groups,
                                 self.algorithm)
-        except Exception:
+        except _lib.MonetHipError as e:
+            if not _refused(e):
+                raise
             out = conv_forward(input_, weight, bias, padding, stride, dilation, groups,
                                DEFAULT_VARIANT)
             self.algorithm = DEFAULT_VARIANT
@@ -269,7 +300,9 @@ class SpecificAlgoConvolution(_ConvBase):
         try:
             return conv_backward_weight(weight_shape, grad, input_, padding, stride, dilation,
                                         groups, algo, with_bias_grad)
-        except Exception:
+        except _lib.MonetHipError as e:
+            if not _refused(e):
+                raise
             out = conv_backward_weight(weight_shape, grad, input_, padding, stride, dilation,
                                        groups, DEFAULT_VARIANT, with_bias_grad)
             self.algorithm = kind * 10 + DEFAULT_VARIANT
@@ -281,8 +314,10 @@ class SpecificAlgoConvolution(_ConvBase):
         try:
             return conv_backward_input(input_shape, grad, weight, padding, stride, dilation, groups,
                                        algo, acc)
-        except Exception:
-            # (a variant is refused before anything is launched, so nothing was added yet)
+        except _lib.MonetHipError as e:
+            if not _refused(e):
+                raise
+            # (a refused variant launched nothing, so nothing was added yet)
             out = conv_backward_input(input_shape, grad, weight, padding, stride, dilation, groups,
                                       DEFAULT_VARIANT, acc)
             self.algorithm = kind * 10 + DEFAULT_VARIANT
@@ -308,8 +343,11 @@ def _autotune(n_variants, run):
             fits = config.budget <= 0 or peak_gb < config.budget * 1.01
             if fits and (best_t is None or t < best_t):
                 best, best_t = alg, t
-        except Exception:
-            pass
+        except _lib.MonetHipError as e:
+            if not _refused(e):
+                raise
+        except torch.cuda.OutOfMemoryError:
+            pass  # a variant whose workspace does not fit is not a candidate
         torch.cuda.empty_cache()
         torch.cuda.reset_peak_memory_stats()
     if best == -1:
@@ -331,7 +369,9 @@ class GreedyAlgoConvolution(_ConvBase):
         try:
             return conv_forward(input_, weight, bias, padding, stride, dilation, groups,
                                 self.fwd_algo)
-        except Exception:
+        except _lib.MonetHipError as e:
+            if not _refused(e):
+                raise
             self.fwd_algo = DEFAULT_VARIANT
             return conv_forward(input_, weight, bias, padding, stride, dilation, groups,
                                 DEFAULT_VARIANT)
@@ -344,7 +384,9 @@ class GreedyAlgoConvolution(_ConvBase):
         try:
             return conv_backward_weight(weight_shape, grad, input_, padding, stride, dilation,
                                         groups, self.bwd_wt_algo, with_bias_grad)
-        except Exception:
+        except _lib.MonetHipError as e:
+            if not _refused(e):
+                raise
             self.bwd_wt_algo = DEFAULT_VARIANT
             return conv_backward_weight(weight_shape, grad, input_, padding, stride, dilation,
                                         groups, DEFAULT_VARIANT, with_bias_grad)
@@ -356,7 +398,9 @@ class GreedyAlgoConvolution(_ConvBase):
         try:
             return conv_backward_input(input_shape, grad, weight, padding, stride, dilation, groups,
                                        self.bwd_ip_algo)
-        except Exception:
+        except _lib.MonetHipError as e:
+            if not _refused(e):
+                raise
             self.bwd_ip_algo = DEFAULT_VARIANT
             return conv_backward_input(input_shape, grad, weight, padding, stride, dilation, groups,
                                        DEFAULT_VARIANT)

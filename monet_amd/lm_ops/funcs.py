@@ -117,6 +117,7 @@ class _AddReLUBase(OP):
     Both inputs receive the ReLU-masked gradient (b's scaled by alpha)."""
     params = None
     inplace = False
+    overwrites_grad = True
 
     def _split(self, g):
         s = self.params

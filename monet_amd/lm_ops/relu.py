@@ -71,6 +71,7 @@ def relu_backward_from_mask(grad, mask):
 @implements(['aten::relu', 'aten::relu_'],
             ['normal', 'multiway', 'newnode', 'multiway_newnode', 'conv_multiway_newnode'])
 class InputActReLU(OP):
+    overwrites_grad = True
     backward_storage = InputStorage(0)
     params = None
     inplace = False
@@ -90,6 +91,7 @@ class InputActReLU(OP):
 @implements(['aten::relu', 'aten::relu_'],
             ['multiway', 'multiway_newnode', 'conv_multiway_newnode', 'conv_normal'])
 class OutputActReLU(OP):
+    overwrites_grad = True
     backward_storage = OutputStorage()
     params = None
     inplace = False
@@ -108,6 +110,7 @@ class OutputActReLU(OP):
 
 @implements(['aten::relu', 'aten::relu_'], ['newnode', 'multiway_newnode', 'conv_multiway_newnode'])
 class BinaryActReLU(OP):
+    overwrites_grad = True
     # mask bytes for an output of `shape`
     backward_storage = IntermediateStorage(lambda shape: (_numel(shape) + 7) // 8)
     params = None

@@ -81,6 +81,8 @@ class Schedule(Graph):
         self._ints = [None] * self.lennodes
         self._state = [None] * self.lennodes
         self._bw = [None] * self.lennodes
+        # storage address -> number of pending gradients (entries of _bw) that live in it
+        self._shared = {}
         self._args = []
 
     # ------------------------------------------------------------ compile
@@ -301,26 +303,58 @@ class Schedule(Graph):
                 grad = bw[k]
                 assert grad is not None, "Backward input not computed for graph node %d (%s)" % (
                     k, self._nodes[k].op)
+                # Pending gradients may share storage (an add hands ONE tensor to both operands,
+                # a view operator hands on a view).  Whoever writes into such storage - an
+                # operator that overwrites its gradient, an accumulation - gets a private copy
+                # while another pending gradient still lives there.
+                shared = self._shared
                 if last:
                     bw[k] = None
-                target = bw[deps[0][0]] if acc else None
+                    key = grad.untyped_storage().data_ptr()
+                    others = shared.get(key, 1) - 1
+                    if others > 0:
+                        shared[key] = others
+                        if op.overwrites_grad:
+                            grad = grad.clone()
+                    else:
+                        shared.pop(key, None)
+                target = None
+                if acc:
+                    ti = deps[0][0]
+                    target = bw[ti]
+                    if target is not None:
+                        key = target.untyped_storage().data_ptr()
+                        if shared.get(key, 1) > 1:
+                            shared[key] -= 1
+                            target = bw[ti] = target.clone()
+                            shared[target.untyped_storage().data_ptr()] = 1
                 if target is not None:
                     outs = op.backward(grad, stored, accumulate_into=target)
                 else:
                     outs = op.backward(grad, stored)
-                del grad, stored, target
+                del grad, stored
                 if not isinstance(outs, (list, tuple)):
                     outs = (outs,)
                 assert len(outs) == len(deps), \
                     "Require the same number of grad outputs as forward inputs %s: %d vs %d" % (
                         self._nodes[k].op, len(outs), len(deps))
-                for (i, r), o in zip(deps, outs):
+                for pos, ((i, r), o) in enumerate(zip(deps, outs)):
                     if r and o is not None:
                         if bw[i] is None:
                             bw[i] = o
-                        elif o is not bw[i]:  # (else: the operator already added it in place)
-                            bw[i] += o
-                del outs
+                            key = o.untyped_storage().data_ptr()
+                            shared[key] = shared.get(key, 0) + 1
+                        elif pos == 0 and o is target:
+                            pass  # the operator has added it to the pending gradient itself
+                        else:
+                            key = bw[i].untyped_storage().data_ptr()
+                            if shared.get(key, 1) > 1:   # someone else still reads this storage
+                                shared[key] -= 1
+                                bw[i] = bw[i] + o
+                                shared[bw[i].untyped_storage().data_ptr()] = 1
+                            else:
+                                bw[i] += o
+                del outs, target
 
     def forward(self, *args):
         """Forward pass; `args` = (input, *parameters and buffers) in graph-node order."""
@@ -341,8 +375,11 @@ class Schedule(Graph):
 
     def backward(self, delta_x):
         bw = self._bw
+        self._shared.clear()
         for k in self._outputs:
             bw[k] = delta_x
+            # the caller's tensor: never written in place (counted as if someone else held it)
+            self._shared[delta_x.untyped_storage().data_ptr()] = 2
         for plan in self._plan[1:]:
             self._run(plan)
         # hand the accumulated gradients to the leaves
@@ -351,6 +388,10 @@ class Schedule(Graph):
             bw[k] = None
             if g is None or not a.requires_grad:
                 continue
+            key = g.untyped_storage().data_ptr()
+            if self._shared.get(key, 1) > 1:   # never hand one storage to two leaves
+                self._shared[key] -= 1
+                g = g.clone()
             if a.is_leaf:
                 if a.grad is None:
                     a.grad = g if g.shape == a.shape else g.reshape(a.shape)
@@ -361,6 +402,7 @@ class Schedule(Graph):
         for k in range(self.lennodes):
             self._regs[k] = self._ints[k] = self._state[k] = self._bw[k] = None
         self._args = []
+        self._shared.clear()
         for op in self._ops0:
             op.params = None
 

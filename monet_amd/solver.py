@@ -520,6 +520,10 @@ def main(argv=None):
     parser.add_argument("--rounds", default=6, type=int,
                         help="tightening-target rounds to fall back on when the direct solve ends "
                              "without a fitting schedule (0: one solve with the whole time limit)")
+    parser.add_argument("--reserve_mb", default=0.0, type=float,
+                        help="MiB of the budget to leave to what the schedule does not hold "
+                             "(optimizer state, loss tensors, allocator rounding): the model is "
+                             "solved against BUDGET minus this, the file keeps BUDGET in its name")
     parser.add_argument("--verbose", action="store_true")
     args = parser.parse_args(argv)
 
@@ -542,7 +546,8 @@ def main(argv=None):
     print("Memory budget", args.budget, "GB; batch size", si.bs, "; model", model_name,
           "; mode", args.mode)
     out = Path(args.data_dir) / solution_file_name(model_name, si.bs, args.mode, args.budget)
-    solution = solve_within_budget(si, args.budget, args.time_limit, args.solver, args.ablation,
+    solution = solve_within_budget(si, args.budget - args.reserve_mb / 1024.0, args.time_limit,
+                                   args.solver, args.ablation,
                                    out_file=str(out), rounds=args.rounds, mip_rel_gap=args.gap,
                                    verbose=args.verbose,
                                    recompute_window=args.window)

@@ -155,6 +155,8 @@ POOL_CASES = [
     ((4, 16, 112, 112), 3, 2, 1, 1, False),
     ((2, 8, 52, 76), 2, 2, 0, 1, False),
     ((3, 5, 7, 7), 3, 2, 1, 1, False),              # odd plane: index pairs straddle planes
+    ((2, 3, 12, 12), 3, 2, 1, 1, True),             # ceil_mode adds a pooled row and column: 7 x 7
+    ((2, 2, 16, 24), 3, 2, 1, 1, True),
 ]
 
 
