@@ -205,13 +205,13 @@ def conv_bench(steps, warmup):
 
     def directions(x, w, dy, peak):
         out = {}
-        for v in range(cv.n_fwd_algos()):
+        for v in range(cv.n_fwd_algos(x.dtype)):
             out["fwd_v%d" % v] = timed(
                 lambda: cv.conv_forward(x, w, None, c["pad"], c["stride"], 1, 1, v), peak)
-        for v in range(cv.n_bwd_ip_algos()):
+        for v in range(cv.n_bwd_ip_algos(x.dtype)):
             out["bwd_data_v%d" % v] = timed(lambda: cv.conv_backward_input(
                 list(x.shape), dy, w, c["pad"], c["stride"], 1, 1, v), peak)
-        for v in range(cv.n_bwd_wt_algos()):
+        for v in range(cv.n_bwd_wt_algos(x.dtype)):
             out["bwd_weight_v%d" % v] = timed(lambda: cv.conv_backward_weight(
                 list(w.shape), dy, x, c["pad"], c["stride"], 1, 1, v), peak)
         return out

@@ -6,7 +6,9 @@
  *   - Every pointer is a raw DEVICE pointer into memory owned by the caller
  *     (inputs, outputs and workspaces).  The library never allocates, frees or
  *     caches device memory and keeps no mutable global state, so it is
- *     re-entrant; the caller's allocator sees every byte that is used.
+ *     re-entrant; the caller's allocator sees every byte that is used.  (One
+ *     exception, marked as such: mn_bn_bwd_from_y_static_f32 works in a
+ *     fixed device array inside the library.)
  *   - `stream` is a hipStream_t passed as void*; all work is enqueued on it and
  *     no entry point synchronises with the host.
  *   - Return value: MN_OK (0) or one of the MN_E* codes below.  Nothing throws
@@ -31,6 +33,7 @@ extern "C" {
 #define MN_EINVAL 1       /* null pointer, negative size, misaligned operand, ws too small */
 #define MN_EUNSUPPORTED 2 /* shape / variant / dtype this build has no kernel for */
 #define MN_ELAUNCH 3      /* hipGetLastError() reported a failed launch */
+#define MN_ELIMIT 4       /* the call needs more than a fixed limit of the entry point allows */
 
 typedef void* mn_stream_t;
 
@@ -160,6 +163,22 @@ int mn_bn_bwd_from_y_f32_limits(const float* dy, const float* y, const float* ga
                                 size_t ws_bytes, uint32_t spin_limit, uint32_t max_workgroups,
                                 mn_stream_t stream);
 
+/* mn_bn_bwd_from_y_f32 for callers that cannot allocate device memory or hand
+ * over a workspace (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): the cross-workgroup partial sums live in a
+ * fixed array of MN_BN_STATIC_WS_BYTES inside the library instead of a caller
+ * workspace, and the call allocates nothing.  Same kernels, same results bit
+ * for bit.  Shapes whose workspace (mn_bn_ws_bytes) exceeds the array are
+ * refused with MN_ELIMIT.  Every GPU holds one copy of the array for the life
+ * of the process and every call on that GPU uses it: calls that overlap on one
+ * GPU (two streams, two threads) race; calls on one stream do not.  No
+ * counterpart in the reference. */
+#define MN_BN_STATIC_WS_BYTES (4u << 20)
+int mn_bn_bwd_from_y_static_f32(const float* dy, const float* y, const float* gamma,
+                                const float* beta, const float* invstd, float* dx, float* dgamma,
+                                float* dbeta, int64_t N, int64_t C, int64_t HW,
+                                mn_stream_t stream);
+
 /* --------------------------------------------------------------- softmax --
  * The tensor is viewed as [outer, dim, inner]; softmax runs over `dim`.
  * Replaces softmax_forward (monet/lm_ops/softmax.cpp:11-15). */
@@ -275,8 +294,8 @@ typedef struct mn_conv2d {
  * cores with fp32 accumulation and rounded once (to nearest even) on output.
  * Needs channel counts that are multiples of 32 on the reduction side
  * (forward: C; backward-data: K) and multiples of 64 for backward-weight (C and
- * K); otherwise MN_EUNSUPPORTED.  Both variant indices of a direction run the
- * same kernel; backward-data always needs K*C*R*S*2 bytes of workspace (the
+ * K); otherwise MN_EUNSUPPORTED.  Variants 0 and 1 of a direction run the
+ * same kernel, further variants are fp32 only; backward-data always needs K*C*R*S*2 bytes of workspace (the
  * transposed weights) and backward-weight its fp32 split partials - ask
  * mn_conv_ws_bytes.  The reference has no reduced-precision path; this dtype
  * serves the bf16 configuration of the layer3 benchmark. */
@@ -297,16 +316,30 @@ typedef struct mn_conv2d {
  *                      output: 0 + a + b and 0 + b + a round identically, so
  *                      the forward gives the same bits on every run (a
  *                      recomputed forward must reproduce masks and indices)
+ *                    2 Winograd F(2x2, 3x3) for 3x3 filters with stride 1 and
+ *                      dilation 1 over a multiple of 16 input channels
+ *                      (MN_EUNSUPPORTED otherwise, and for MN_BF16): 2.25 times
+ *                      fewer multiplications, paid for with a workspace of 16
+ *                      floats per 2x2 output tile and channel, input and output
+ *                      side (the role of the reference's WINOGRAD_NONFUSED
+ *                      slot, monet/lm_ops/conv.cpp:21-27, :314-324)
  *   backward-data    0 implicit GEMM reading the weights through strides
  *                    1 same with the weights repacked [tap][k][c] (c padded
  *                      to a multiple of 128) into the workspace; may split
  *                      the reduction up to 8 ways and add the slices with
  *                      atomics (last bits can differ from run to run; variant
  *                      0 never does)
+ *                    2 Winograd F(2x2, 3x3), as for the forward (the filter
+ *                      rotated by 180 degrees, channel roles swapped)
  *   backward-weight  0 split reduction combined with atomics into a cleared dw
  *                    1 split reduction through per-split partials in the
  *                      workspace, then a fixed-order sum (reproducible) */
 int mn_conv_n_variants(int direction);
+/* The same per dtype: the list above for MN_F32; 1 for MN_BF16 (one kernel and
+ * one memory tier per direction - index 1 is accepted as an alias of 0 so that
+ * an fp32 schedule's choice still runs); 0 for an unknown dtype.  The
+ * reference is fp32 only and has no counterpart. */
+int mn_conv_n_variants_for(int direction, int dtype);
 /* Workspace bytes a (direction, variant, dtype) needs for this geometry
  * (role of the cudnnGet*WorkspaceSize queries at conv.cpp:314-324). */
 int mn_conv_ws_bytes(const mn_conv2d* g, int direction, int variant, int dtype, size_t* bytes);

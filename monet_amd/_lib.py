@@ -16,7 +16,7 @@ LIB_PATH = Path(os.environ.get("MONET_HIP_LIBRARY",
                                Path(__file__).resolve().parent / "libmonet_hip.so"))
 ABI_VERSION = 1
 
-MN_OK, MN_EINVAL, MN_EUNSUPPORTED, MN_ELAUNCH = 0, 1, 2, 3
+MN_OK, MN_EINVAL, MN_EUNSUPPORTED, MN_ELAUNCH, MN_ELIMIT = 0, 1, 2, 3, 4
 
 
 class MonetHipError(RuntimeError):
@@ -73,6 +73,8 @@ _SIGNATURES = {
     "mn_bn_bwd_from_y_f32_limits": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int64,
                                             c_int64, _P, c_size_t, c_uint32, c_uint32, _P]),
     "mn_bn_ws_status": (c_int, [_P, c_size_t, c_int64, c_int64, c_int64, _P]),
+    "mn_bn_bwd_from_y_static_f32": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int64,
+                                            c_int64, _P]),
     "mn_bn_relu_fwd_train_f32": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64,
                                          c_double, c_double, _P, c_size_t, _P]),
     "mn_bn_relu_fwd_apply_f32": (c_int, [_P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, _P]),
@@ -95,6 +97,7 @@ _SIGNATURES = {
     "mn_softmax_bwd_f32": (c_int, [_P, _P, _P, c_int64, c_int64, c_int64, _P]),
     "mn_xent_bwd_f32": (c_int, [_P, _P, _P, c_int64, c_int64, c_int64, c_float, _P]),
     "mn_conv_n_variants": (c_int, [c_int]),
+    "mn_conv_n_variants_for": (c_int, [c_int, c_int]),
     "mn_conv_ws_bytes": (c_int, [POINTER(Conv2d), c_int, c_int, c_int, POINTER(c_size_t)]),
     "mn_conv_fwd": (c_int, [POINTER(Conv2d), _P, _P, _P, _P, _P, c_size_t, c_int, c_int, _P]),
     "mn_conv_bwd_data": (c_int, [POINTER(Conv2d), _P, _P, _P, _P, c_size_t, c_int, c_int, _P]),
@@ -105,7 +108,7 @@ _SIGNATURES = {
                                         _P]),
 }
 # entry points whose int return value is NOT a status code
-_UNCHECKED = {"mn_abi_version", "mn_conv_n_variants"}
+_UNCHECKED = {"mn_abi_version", "mn_conv_n_variants", "mn_conv_n_variants_for"}
 
 _lib = None
 

@@ -14,7 +14,9 @@ const char* mn_status_string(int status) {
     case MN_EUNSUPPORTED:
       return "unsupported shape, variant or dtype";
     case MN_ELAUNCH:
-      return "kernel launch failed";
+      return "kernel launch failed, or a kernel reported that it could not finish its work";
+    case MN_ELIMIT:
+      return "the call needs more than a fixed limit of this entry point allows";
     default:
       return "unknown status";
   }

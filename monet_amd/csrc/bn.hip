@@ -33,6 +33,8 @@
 // (reduce, then apply) that read the operands twice.
 #include "common.h"
 
+#include <mutex>
+
 namespace mn_bn {
 
 constexpr int kThreads = 256;
@@ -1094,6 +1096,45 @@ int mn_bn_bwd_from_y_f32_limits(const float* dy, const float* y, const float* ga
   if (max_workgroups) t.grid = (int)(max_workgroups < 65535u ? max_workgroups : 65535u);
   return mn_bn::bwd_launch(true, dy, y, gamma, beta, invstd, dx, dgamma, dbeta, N, C, HW, ws,
                            ws_bytes, mn_stream(stream), t);
+}
+
+// The workspace of mn_bn_bwd_from_y_static_f32.  In host code this name is only a handle for
+// hipGetSymbolAddress, not a device address: kernels are given the address looked up below.
+static __device__ __align__(256) unsigned char scratch[MN_BN_STATIC_WS_BYTES];
+
+// Device address of `scratch` on the current device (every GPU holds its own copy at its own
+// address); looked up once per device.  Null if the lookup fails.
+static void* static_workspace() {
+  constexpr int kMaxDevices = 64;
+  static std::mutex lock;
+  static void* address[kMaxDevices] = {};
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> hold(lock);
+  if (!address[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess) return nullptr;
+    address[dev] = p;
+  }
+  return address[dev];
+}
+
+int mn_bn_bwd_from_y_static_f32(const float* dy, const float* y, const float* gamma,
+                                const float* beta, const float* invstd, float* dx, float* dgamma,
+                                float* dbeta, int64_t N, int64_t C, int64_t HW,
+                                mn_stream_t stream) {
+  if (N < 0 || C < 0 || HW < 0) return MN_EINVAL;
+  if (N == 0 || C == 0 || HW == 0) return MN_OK;
+  if (!mn_bn::shape_limits(N, C, HW)) return MN_EUNSUPPORTED;
+  const size_t need = mn_bn::ws_bytes_for(N, C, HW);
+  if (need > (size_t)MN_BN_STATIC_WS_BYTES) return MN_ELIMIT;
+  void* ws = static_workspace();
+  if (!ws) return MN_ELAUNCH;
+  // every formulation initialises what it reads of the workspace (slots, ticket and error word
+  // by the prepare launch; partial sums are written before they are read), so whatever the
+  // previous call left there does not matter
+  return mn_bn::bwd_launch(true, dy, y, gamma, beta, invstd, dx, dgamma, dbeta, N, C, HW, ws, need,
+                           mn_stream(stream), mn_bn::Tuning());
 }
 
 int mn_bn_ws_status(const void* ws, size_t ws_bytes, int64_t N, int64_t C, int64_t HW,

@@ -23,6 +23,13 @@
 #include "common.h"
 #include <type_traits>
 
+// Winograd F(2x2, 3x3) tier of forward and backward-data (conv_wino.hip)
+int mn_wino_ws_bytes(const mn_conv2d* g, bool backward_data, size_t* bytes);
+int mn_wino_fwd(const mn_conv2d* g, const float* x, const float* w, const float* bias, float* y,
+                void* ws, size_t ws_bytes, hipStream_t s);
+int mn_wino_bwd_data(const mn_conv2d* g, const float* dy, const float* w, float* dx, bool accum,
+                     void* ws, size_t ws_bytes, hipStream_t s);
+
 // bf16 / channels-last kernels (conv_bf16.hip)
 int mn_conv16_ws_bytes(const mn_conv2d* g, int direction, size_t* bytes);
 int mn_conv16_fwd(const mn_conv2d* g, const void* x, const void* w, const void* bias, void* y,
@@ -117,6 +124,10 @@ struct Gather {
   int chunk;  // tap-major kernels: the reduction visits all taps of `chunk` channels, then the next block
   int accum;                    // add to what dst already holds instead of overwriting it
   uint32_t src_bytes, a_bytes;  // sizes of the source tensor and of the repacked A (PACKED)
+  // batch > 1: grid.z independent problems of this shape (no split reduction then); problem z
+  // reads a + z*a_batch and src + z*src_batch and writes dst + z*dst_batch (floats)
+  int batch;
+  size_t a_batch, src_batch, dst_batch;
   FastDiv divOHW, divOW;        // column -> (image, row, column) by multiplication ...
   int exact_div;                // ... unless ncols * OH*OW is beyond FastDiv's exact range
 };
@@ -152,10 +163,13 @@ constexpr int kPadPacked = 4;  // keeps LDS rows 16-byte aligned for the 128-bit
 constexpr uint32_t kBeyond = 0x80000000u;  // a byte offset past the end of any buffer
 template <class TL, bool FAST, bool PACKED = false, bool POINT = false>
 __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
-                                                               const float* __restrict__ a,
-                                                               const float* __restrict__ src,
+                                                               const float* __restrict__ a_in,
+                                                               const float* __restrict__ src_in,
                                                                const float* __restrict__ bias,
-                                                               float* __restrict__ dst) {
+                                                               float* __restrict__ dst_in) {
+  const float* a = a_in;
+  const float* src = src_in;
+  float* dst = dst_in;
   static_assert(!PACKED || FAST, "the packed operand is only used with the tap-major path");
   static_assert(!POINT || PACKED, "the pointwise path is built on the packed one");
   constexpr int BM = TL::BM, BN = TL::BN;
@@ -176,6 +190,11 @@ __global__ __launch_bounds__(kThreads) void gather_gemm_kernel(const Gather g,
   const uint32_t bx = in_z / gridDim.y, by = in_z - bx * gridDim.y;
   const int m0 = by * BM;
   const uint32_t n0 = bx * BN;
+  if (g.batch > 1) {  // uniform
+    a += (size_t)bz * g.a_batch;
+    src += (size_t)bz * g.src_batch;
+    dst += (size_t)bz * g.dst_batch;
+  }
   if (tid < g.T) {
     tdh[tid] = g.dh[tid];
     tdw[tid] = g.dw[tid];
@@ -1161,7 +1180,8 @@ static bool fast_path(const Gather& g) {
 template <class TL>
 static void launch_gather_t(const Gather& g, const float* a, const float* src, const float* bias,
                             float* dst, hipStream_t s, bool packed) {
-  dim3 grid((g.ncols + TL::BN - 1) / TL::BN, (g.M + TL::BM - 1) / TL::BM, g.ksplit > 1 ? g.ksplit : 1);
+  dim3 grid((g.ncols + TL::BN - 1) / TL::BN, (g.M + TL::BM - 1) / TL::BM,
+            g.batch > 1 ? g.batch : (g.ksplit > 1 ? g.ksplit : 1));
   // pointwise: the gather is the identity and pixels come in whole float4
   const bool point = packed && g.T == 1 && g.dh[0] == 0 && g.dw[0] == 0 && g.ish == 1 &&
                      g.isw == 1 && g.Hs == g.OH && g.Ws == g.OW && (g.OH * g.OW) % 4 == 0 &&
@@ -1211,7 +1231,7 @@ static void launch_gather(Gather g, const float* a, const float* src, const floa
   // multiplication by the reciprocal is exact while dividend * divisor < 2^32
   g.exact_div = ((unsigned long long)(g.ncols + 256) * (unsigned long long)(g.OH * g.OW) >= (1ull << 32)) ? 1 : 0;
   if (tile < 0) tile = pick_tile(g.M, g.ncols, fast_path(g), packed);
-  plan_split(g, tile, split_ok && packed, max_split);
+  plan_split(g, tile, split_ok && packed && g.batch <= 1, max_split);
   // Tap after tap over ALL channels re-reads each pixel once per tap with the whole channel
   // range in between, far more than an L2 holds across the workgroups of an XCD.  Cycling the
   // taps over a block of 2-4 k-tiles keeps the re-reads in cache; shorter blocks re-enter taps
@@ -1293,19 +1313,67 @@ static void wgrad_split(const mn_conv2d* g, int variant, int* splits, int* tiles
 
 }  // namespace mn_conv
 
+// `batch` independent GEMMs in one launch (used by the Winograd variant, conv_wino.hip):
+// dst[b][m][col] = sum over ch of a[b][ch][m] * src[b][ch][col], with a = [batch][Cs][Mp]
+// (rows of Mp floats, Mp a multiple of 128 and >= M, zero padded), src = [batch][Cs][cols],
+// dst = [batch][M][cols]; Cs a multiple of 16, cols a multiple of 4, 16-byte aligned pointers,
+// every slice below 2 GB.  Runs the pointwise path of the gather GEMM (both operands fetched
+// as 16-byte vectors through buffer descriptors).
+int mn_conv_batched_gemm(const float* a, const float* src, float* dst, int M, int Mp, int Cs,
+                         uint32_t cols, int batch, hipStream_t s) {
+  using namespace mn_conv;
+  if (M <= 0 || Cs <= 0 || cols == 0 || batch <= 0) return MN_EINVAL;
+  if (Cs % BK != 0 || cols % 4 != 0 || Mp % 128 != 0 || Mp < M) return MN_EUNSUPPORTED;
+  if (!mn_aligned(a, 16) || !mn_aligned(src, 16) || !mn_aligned(dst, 16)) return MN_EINVAL;
+  if (!buffers_fit((size_t)Cs * cols, (size_t)Cs * Mp) || (size_t)M * cols >= (1ull << 30))
+    return MN_EUNSUPPORTED;
+  Gather q = {};
+  q.M = M;
+  q.T = 1;
+  q.Kd = Cs;
+  q.divT = make_fastdiv(1);
+  q.N = 1;
+  q.OH = 1;
+  q.OW = (int)cols;
+  q.ncols = cols;
+  q.Cs = Cs;
+  q.Hs = 1;
+  q.Ws = (int)cols;
+  q.ish = q.isw = 1;
+  q.DH = 1;
+  q.DW = (int)cols;
+  q.osh = q.osw = 1;
+  q.lda = Mp;
+  q.cha = 1;
+  q.a_bytes = (uint32_t)((size_t)Cs * Mp * sizeof(float));
+  q.batch = batch;
+  q.a_batch = (size_t)Cs * Mp;
+  q.src_batch = (size_t)Cs * cols;
+  q.dst_batch = (size_t)M * cols;
+  launch_gather(q, a, src, nullptr, dst, s, true, false);
+  return mn_launch_status();
+}
+
 extern "C" {
 
 int mn_conv_n_variants(int direction) {
   switch (direction) {
     case MN_CONV_FWD:
-      return 2;
+      return 3;
     case MN_CONV_BWD_DATA:
-      return 2;
+      return 3;
     case MN_CONV_BWD_WEIGHT:
       return 2;
     default:
       return 0;
   }
+}
+
+int mn_conv_n_variants_for(int direction, int dtype) {
+  if (dtype == MN_F32) return mn_conv_n_variants(direction);
+  // bf16: one kernel per direction, a single memory tier
+  if (dtype == MN_BF16) return mn_conv_n_variants(direction) > 0 ? 1 : 0;
+  return 0;
 }
 
 int mn_conv_ws_bytes(const mn_conv2d* g, int direction, int variant, int dtype, size_t* bytes) {
@@ -1315,8 +1383,10 @@ int mn_conv_ws_bytes(const mn_conv2d* g, int direction, int variant, int dtype, 
   const int st = check(g);
   if (st != MN_OK) return st;
   if (variant < 0 || variant >= mn_conv_n_variants(direction)) return MN_EUNSUPPORTED;
-  if (dtype == MN_BF16) return mn_conv16_ws_bytes(g, direction, bytes);  // same for every variant
+  if (dtype == MN_BF16)  // variants 0 and 1 are one kernel; there is no bf16 Winograd tier
+    return variant <= 1 ? mn_conv16_ws_bytes(g, direction, bytes) : MN_EUNSUPPORTED;
   if (dtype != MN_F32) return MN_EUNSUPPORTED;
+  if (variant == 2) return mn_wino_ws_bytes(g, direction == MN_CONV_BWD_DATA, bytes);
   const size_t wsize = (size_t)g->K * g->C * g->R * g->S * sizeof(float);
   // variant 1 of the gather directions: the repacked weight operand (rows padded to 128)
   if (direction == MN_CONV_FWD && variant == 1)
@@ -1337,11 +1407,14 @@ int mn_conv_fwd(const mn_conv2d* g, const void* x, const void* w, const void* bi
   using namespace mn_conv;
   const int st = check(g);
   if (st != MN_OK) return st;
-  if (variant < 0 || variant > 1) return MN_EUNSUPPORTED;
+  if (variant < 0 || variant > 2 || (variant == 2 && dtype != MN_F32)) return MN_EUNSUPPORTED;
   if (g->N == 0) return MN_OK;
   if (!x || !w || !y) return MN_EINVAL;
   if (dtype == MN_BF16) return mn_conv16_fwd(g, x, w, bias, y, mn_stream(stream));
   if (dtype != MN_F32) return MN_EUNSUPPORTED;
+  if (variant == 2)
+    return mn_wino_fwd(g, (const float*)x, (const float*)w, (const float*)bias, (float*)y, ws,
+                       ws_bytes, mn_stream(stream));
   Gather q = {};
   q.M = g->K;
   q.T = g->R * g->S;
@@ -1397,13 +1470,15 @@ static int conv_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void
   using namespace mn_conv;
   const int st = check(g);
   if (st != MN_OK) return st;
-  if (variant < 0 || variant > 1) return MN_EUNSUPPORTED;
+  if (variant < 0 || variant > 2 || (variant == 2 && dtype != MN_F32)) return MN_EUNSUPPORTED;
   if (g->N == 0) return MN_OK;
   if (!dy || !w || !dx) return MN_EINVAL;
   hipStream_t s = mn_stream(stream);
   if (dtype == MN_BF16)
     return accum ? MN_EUNSUPPORTED : mn_conv16_bwd_data(g, dy, w, dx, ws, ws_bytes, s);
   if (dtype != MN_F32) return MN_EUNSUPPORTED;
+  if (variant == 2)
+    return mn_wino_bwd_data(g, (const float*)dy, (const float*)w, (float*)dx, accum, ws, ws_bytes, s);
   const int RS = g->R * g->S;
   const float* a = (const float*)w;
   uint32_t a_bytes = weight_bytes(g);  // size of the A operand: the weights, or their repacked copy

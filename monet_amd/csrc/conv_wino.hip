@@ -1,0 +1,265 @@
+// Winograd F(2x2, 3x3) convolution, fp32: the memory-for-arithmetic tier of the forward and
+// backward-data directions (3x3 filters, stride 1, dilation 1).
+//
+//   Y = A^T [ (G g G^T) .* (B^T d B) ] A          per 4x4 input tile d -> 2x2 output tile Y
+//
+// with the element-wise product summed over the input channels.  Written per transform-domain
+// position (xi, nu) in 0..15 that sum is a plain matrix product
+//   Mt[pos][m][tile] = sum over ch of U[pos][ch][m] * V[pos][ch][tile]
+// so the arithmetic is 16 GEMMs of (output channels) x (tiles) x (input channels): 16 multiplies
+// per 2x2 outputs and channel pair instead of 36, i.e. 2.25 times fewer than the direct form.
+// The price is the workspace: V and Mt hold 16 floats per tile and channel where the tensors
+// themselves hold 4.
+//
+// Four launches: weights -> U, source -> V, one batched GEMM (the pointwise path of the gather
+// GEMM in conv.hip), Mt -> destination (+ bias, or added to what the destination holds).
+// Backward-data is the same computation on dy with the filter rotated by 180 degrees, the two
+// channel roles swapped and padding 2 - pad.
+#include "common.h"
+
+int mn_conv_batched_gemm(const float* a, const float* src, float* dst, int M, int Mp, int Cs,
+                         uint32_t cols, int batch, hipStream_t s);
+
+namespace mn_wino {
+
+constexpr int kThreads = 256;
+
+struct Plan {
+  int N, Cs, Hs, Ws;   // source tensor [N, Cs, Hs, Ws]
+  int M, OH, OW;       // destination tensor [N, M, OH, OW]
+  int pad;             // source coordinate of tile element (i, j) = (2*th - pad + i, 2*tw - pad + j)
+  int TH, TW;          // tiles per image
+  uint32_t T, Tp;      // tiles, and tiles rounded up to a multiple of 4 (row length of V and Mt)
+  int Mp;              // rows of U padded to a multiple of 128
+};
+
+static size_t u_floats(const Plan& p) { return (size_t)16 * p.Cs * p.Mp; }
+static size_t v_floats(const Plan& p) { return (size_t)16 * p.Cs * p.Tp; }
+static size_t m_floats(const Plan& p) { return (size_t)16 * p.M * p.Tp; }
+
+// U[pos][ch][m] = (G g G^T)[pos] for the 3x3 filter g of (m, ch).
+// FLIP = false (forward):      g[r][s] = w[m][ch][r][s]       (w is [M][Cs][3][3])
+// FLIP = true (backward-data): g[r][s] = w[ch][m][2-r][2-s]   (w is [Cs][M][3][3])
+template <bool FLIP>
+__global__ __launch_bounds__(kThreads) void weight_kernel(const float* __restrict__ w,
+                                                          float* __restrict__ U, int M, int Mp,
+                                                          int Cs) {
+  const uint32_t i = blockIdx.x * kThreads + threadIdx.x;
+  if (i >= (uint32_t)Cs * Mp) return;
+  const int m = i % Mp, ch = i / Mp;
+  float g[3][3];
+#pragma unroll
+  for (int r = 0; r < 3; ++r)
+#pragma unroll
+    for (int s = 0; s < 3; ++s) {
+      float v = 0.f;
+      if (m < M)
+        v = FLIP ? w[(((size_t)ch * M + m) * 3 + (2 - r)) * 3 + (2 - s)]
+                 : w[(((size_t)m * Cs + ch) * 3 + r) * 3 + s];
+      g[r][s] = v;
+    }
+  // t = G g (4x3), then u = t G^T (4x4); G = [1 0 0; .5 .5 .5; .5 -.5 .5; 0 0 1]
+  float t[4][3];
+#pragma unroll
+  for (int s = 0; s < 3; ++s) {
+    t[0][s] = g[0][s];
+    t[1][s] = 0.5f * (g[0][s] + g[1][s] + g[2][s]);
+    t[2][s] = 0.5f * (g[0][s] - g[1][s] + g[2][s]);
+    t[3][s] = g[2][s];
+  }
+  const size_t stride = (size_t)Cs * Mp;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const float u0 = t[r][0];
+    const float u1 = 0.5f * (t[r][0] + t[r][1] + t[r][2]);
+    const float u2 = 0.5f * (t[r][0] - t[r][1] + t[r][2]);
+    const float u3 = t[r][2];
+    U[(size_t)(4 * r + 0) * stride + i] = u0;
+    U[(size_t)(4 * r + 1) * stride + i] = u1;
+    U[(size_t)(4 * r + 2) * stride + i] = u2;
+    U[(size_t)(4 * r + 3) * stride + i] = u3;
+  }
+}
+
+// V[pos][ch][tile] = (B^T d B)[pos], d = the 4x4 source patch of the tile (zero outside the
+// image).  One thread per (ch, tile); tiles run fastest, so the 16 stores are coalesced.
+// B^T = [1 0 -1 0; 0 1 1 0; 0 -1 1 0; 0 1 0 -1]
+__global__ __launch_bounds__(kThreads) void input_kernel(const Plan p, const float* __restrict__ src,
+                                                         float* __restrict__ V) {
+  const uint32_t i = blockIdx.x * kThreads + threadIdx.x;
+  const uint32_t row = i / p.Tp, tile = i - row * p.Tp;  // row = ch
+  if (row >= (uint32_t)p.Cs) return;
+  const size_t stride = (size_t)p.Cs * p.Tp;
+  float d[4][4];
+  if (tile < p.T) {
+    const uint32_t per_img = (uint32_t)p.TH * p.TW;
+    const uint32_t n = tile / per_img, r = tile - n * per_img;
+    const int th = r / p.TW, tw = r - th * p.TW;
+    const int h0 = 2 * th - p.pad, w0 = 2 * tw - p.pad;
+    const float* plane = src + ((size_t)n * p.Cs + row) * p.Hs * p.Ws;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      const int h = h0 + a;
+      const bool hok = (unsigned)h < (unsigned)p.Hs;
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const int w = w0 + b;
+        d[a][b] = (hok && (unsigned)w < (unsigned)p.Ws) ? plane[(size_t)h * p.Ws + w] : 0.f;
+      }
+    }
+  } else {
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) d[a][b] = 0.f;  // padding columns of V: defined, never used
+  }
+  float t[4][4];  // t = B^T d
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    t[0][b] = d[0][b] - d[2][b];
+    t[1][b] = d[1][b] + d[2][b];
+    t[2][b] = d[2][b] - d[1][b];
+    t[3][b] = d[1][b] - d[3][b];
+  }
+#pragma unroll
+  for (int a = 0; a < 4; ++a) {  // v = t B
+    st_stream(V + (size_t)(4 * a + 0) * stride + i, t[a][0] - t[a][2]);
+    st_stream(V + (size_t)(4 * a + 1) * stride + i, t[a][1] + t[a][2]);
+    st_stream(V + (size_t)(4 * a + 2) * stride + i, t[a][2] - t[a][1]);
+    st_stream(V + (size_t)(4 * a + 3) * stride + i, t[a][1] - t[a][3]);
+  }
+}
+
+// dst 2x2 tile = A^T m A with m = Mt[.][row][tile]; A^T = [1 1 1 0; 0 1 -1 -1].
+// One thread per (row, tile).  ACCUM: dst += result.
+template <bool ACCUM>
+__global__ __launch_bounds__(kThreads) void output_kernel(const Plan p, const float* __restrict__ Mt,
+                                                          const float* __restrict__ bias,
+                                                          float* __restrict__ dst) {
+  const uint32_t i = blockIdx.x * kThreads + threadIdx.x;
+  const uint32_t row = i / p.Tp, tile = i - row * p.Tp;
+  if (row >= (uint32_t)p.M || tile >= p.T) return;
+  const size_t stride = (size_t)p.M * p.Tp;
+  float m[4][4];
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 4; ++b) m[a][b] = ld_stream(Mt + (size_t)(4 * a + b) * stride + i);
+  float t[2][4];  // t = A^T m
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    t[0][b] = m[0][b] + m[1][b] + m[2][b];
+    t[1][b] = m[1][b] - m[2][b] - m[3][b];
+  }
+  const float bv = bias ? bias[row] : 0.f;
+  float y[2][2];
+#pragma unroll
+  for (int a = 0; a < 2; ++a) {
+    y[a][0] = t[a][0] + t[a][1] + t[a][2] + bv;
+    y[a][1] = t[a][1] - t[a][2] - t[a][3] + bv;
+  }
+  const uint32_t per_img = (uint32_t)p.TH * p.TW;
+  const uint32_t n = tile / per_img, r = tile - n * per_img;
+  const int th = r / p.TW, tw = r - th * p.TW;
+  const int oh = 2 * th, ow = 2 * tw;
+  float* o = dst + (((size_t)n * p.M + row) * p.OH + oh) * p.OW + ow;
+#pragma unroll
+  for (int a = 0; a < 2; ++a) {
+    if (oh + a >= p.OH) break;
+    float* q = o + (size_t)a * p.OW;
+    if (ACCUM) {
+      q[0] += y[a][0];
+      if (ow + 1 < p.OW) q[1] += y[a][1];
+    } else {
+      q[0] = y[a][0];
+      if (ow + 1 < p.OW) q[1] = y[a][1];
+    }
+  }
+}
+
+static bool make_plan(int N, int Cs, int Hs, int Ws, int M, int OH, int OW, int pad, Plan& p) {
+  p.N = N;
+  p.Cs = Cs;
+  p.Hs = Hs;
+  p.Ws = Ws;
+  p.M = M;
+  p.OH = OH;
+  p.OW = OW;
+  p.pad = pad;
+  p.TH = (OH + 1) / 2;
+  p.TW = (OW + 1) / 2;
+  const unsigned long long T = (unsigned long long)N * p.TH * p.TW;
+  if (T == 0 || T >= (1ull << 28)) return false;
+  p.T = (uint32_t)T;
+  p.Tp = (p.T + 3u) & ~3u;
+  p.Mp = (M + 127) / 128 * 128;
+  // one thread per (channel, tile) with 32-bit indices; every GEMM slice below 2 GB
+  if ((unsigned long long)Cs * p.Tp >= (1ull << 29) || (unsigned long long)M * p.Tp >= (1ull << 29) ||
+      (unsigned long long)Cs * p.Mp >= (1ull << 29))
+    return false;
+  return Cs % 16 == 0;
+}
+
+static int run(const Plan& p, const float* src, const float* w, bool flip, const float* bias,
+               float* dst, bool accum, void* ws, size_t ws_bytes, hipStream_t s) {
+  const size_t need = (u_floats(p) + v_floats(p) + m_floats(p)) * sizeof(float);
+  if (!ws || ws_bytes < need || !mn_aligned(ws, 16)) return MN_EINVAL;
+  float* U = static_cast<float*>(ws);
+  float* V = U + u_floats(p);
+  float* Mt = V + v_floats(p);
+  const uint32_t nu = (uint32_t)p.Cs * p.Mp;
+  if (flip)
+    weight_kernel<true><<<(nu + kThreads - 1) / kThreads, kThreads, 0, s>>>(w, U, p.M, p.Mp, p.Cs);
+  else
+    weight_kernel<false><<<(nu + kThreads - 1) / kThreads, kThreads, 0, s>>>(w, U, p.M, p.Mp, p.Cs);
+  const uint32_t nv = (uint32_t)p.Cs * p.Tp;
+  input_kernel<<<(nv + kThreads - 1) / kThreads, kThreads, 0, s>>>(p, src, V);
+  const int st = mn_conv_batched_gemm(U, V, Mt, p.M, p.Mp, p.Cs, p.Tp, 16, s);
+  if (st != MN_OK) return st;
+  const uint32_t no = (uint32_t)p.M * p.Tp;
+  if (accum)
+    output_kernel<true><<<(no + kThreads - 1) / kThreads, kThreads, 0, s>>>(p, Mt, bias, dst);
+  else
+    output_kernel<false><<<(no + kThreads - 1) / kThreads, kThreads, 0, s>>>(p, Mt, bias, dst);
+  return mn_launch_status();
+}
+
+static bool shape_ok(const mn_conv2d* g) {
+  return g->R == 3 && g->S == 3 && g->sH == 1 && g->sW == 1 && g->dH == 1 && g->dW == 1 &&
+         g->pH == g->pW && g->pH <= 2 && g->groups == 1;
+}
+
+}  // namespace mn_wino
+
+// Entry points used by conv.hip (all fp32).  `bytes` = 0 and MN_EUNSUPPORTED when the shape is
+// not a 3x3 / stride 1 / dilation 1 convolution with a reduction over a multiple of 16 channels.
+int mn_wino_ws_bytes(const mn_conv2d* g, bool backward_data, size_t* bytes) {
+  using namespace mn_wino;
+  *bytes = 0;
+  if (!shape_ok(g)) return MN_EUNSUPPORTED;
+  Plan p;
+  const bool ok = backward_data
+                      ? make_plan(g->N, g->K, g->P, g->Q, g->C, g->H, g->W, 2 - g->pH, p)
+                      : make_plan(g->N, g->C, g->H, g->W, g->K, g->P, g->Q, g->pH, p);
+  if (!ok) return MN_EUNSUPPORTED;
+  *bytes = (u_floats(p) + v_floats(p) + m_floats(p)) * sizeof(float);
+  return MN_OK;
+}
+
+int mn_wino_fwd(const mn_conv2d* g, const float* x, const float* w, const float* bias, float* y,
+                void* ws, size_t ws_bytes, hipStream_t s) {
+  using namespace mn_wino;
+  Plan p;
+  if (!shape_ok(g) || !make_plan(g->N, g->C, g->H, g->W, g->K, g->P, g->Q, g->pH, p))
+    return MN_EUNSUPPORTED;
+  return run(p, x, w, false, bias, y, false, ws, ws_bytes, s);
+}
+
+int mn_wino_bwd_data(const mn_conv2d* g, const float* dy, const float* w, float* dx, bool accum,
+                     void* ws, size_t ws_bytes, hipStream_t s) {
+  using namespace mn_wino;
+  Plan p;
+  if (!shape_ok(g) || !make_plan(g->N, g->K, g->P, g->Q, g->C, g->H, g->W, 2 - g->pH, p))
+    return MN_EUNSUPPORTED;
+  return run(p, dy, w, true, nullptr, dx, accum, ws, ws_bytes, s);
+}

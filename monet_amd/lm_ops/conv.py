@@ -58,16 +58,22 @@ def conv_geometry(input_shape, weight_shape, stride, padding, dilation, groups):
     return _lib.Conv2d(N, C, H, W, K, R, S, sH, sW, pH, pW, dH, dW, P, Q, int(groups))
 
 
-def n_fwd_algos():
-    return _lib.load().mn_conv_n_variants(_lib.CONV_FWD)
+def _n_variants(direction, dtype):
+    code = _lib.BF16 if dtype == torch.bfloat16 else _lib.F32
+    return _lib.load().mn_conv_n_variants_for(direction, code)
 
 
-def n_bwd_ip_algos():
-    return _lib.load().mn_conv_n_variants(_lib.CONV_BWD_DATA)
+def n_fwd_algos(dtype=None):
+    """Kernel variants of the forward (fp32 unless `dtype` is torch.bfloat16)."""
+    return _n_variants(_lib.CONV_FWD, dtype)
 
 
-def n_bwd_wt_algos():
-    return _lib.load().mn_conv_n_variants(_lib.CONV_BWD_WEIGHT)
+def n_bwd_ip_algos(dtype=None):
+    return _n_variants(_lib.CONV_BWD_DATA, dtype)
+
+
+def n_bwd_wt_algos(dtype=None):
+    return _n_variants(_lib.CONV_BWD_WEIGHT, dtype)
 
 
 def _workspace(geo, direction, variant, device, dtype=None):

@@ -102,7 +102,7 @@ class Schedule(Graph):
         si, n = self.si, self._nodes[k]
         op = lm_ops.list_ops(si.mode, n.op)[self._implementation(solution, t, j)]()
         if si.select_conv_algo and j in si.conv_list:
-            for c in range(op.n_fwd_algos()):
+            for c in range(min(op.n_fwd_algos(), solution.rf.shape[2])):
                 if solution.rf[t, si.conv_list[j], c]:
                     op.algorithm = c
                     break

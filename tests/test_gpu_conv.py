@@ -36,7 +36,28 @@ CASES = [
     ((2, 32, 13, 17), (48, 32, 3, 3), 2, (2, 1), 2),   # tap-major path with stride, dilation, uneven padding
     ((2, 64, 12, 12), (64, 64, 5, 5), 1, 2, 1),        # 25 taps, windows hanging over every border
     ((1, 128, 6, 10), (128, 128, 3, 3), (1, 2), (1, 0), (1, 1)),  # stride on one axis only
+    ((2, 32, 10, 9), (40, 32, 3, 3), 1, 0, 1),         # 3x3 without padding (Winograd: backward pads by 2)
+    ((2, 16, 6, 7), (16, 16, 3, 3), 1, 2, 1),          # 3x3 padded by 2: output larger than the input
+    ((2, 20, 11, 13), (48, 20, 3, 3), 1, 1, 1),        # Winograd backward-data only (K % 16 == 0, C is not)
+    ((3, 48, 5, 5), (32, 48, 3, 3), 1, 1, 1),          # odd planes: ragged 2x2 output tiles
 ]
+
+
+def winograd_applies(ws, st, pad, dil, reduced_channels):
+    """Variant 2 (Winograd F(2x2, 3x3)) covers 3x3 filters, stride 1, dilation 1, equal
+    padding <= 2 on both axes and a reduction over a multiple of 16 channels; anything else
+    must be refused with MN_EUNSUPPORTED."""
+    pair = lambda v: tuple(v) if isinstance(v, (tuple, list)) else (v, v)
+    return (ws[2] == 3 and ws[3] == 3 and pair(st) == (1, 1) and pair(dil) == (1, 1) and
+            pair(pad)[0] == pair(pad)[1] and pair(pad)[0] <= 2 and reduced_channels % 16 == 0)
+
+
+def refused(call):
+    from monet_amd import _lib
+    with pytest.raises(_lib.MonetHipError) as e:
+        call()
+    assert e.value.status == _lib.MN_EUNSUPPORTED
+    return True
 
 
 def dev(a, cuda):
@@ -68,7 +89,12 @@ def test_conv_forward(cuda, xs, ws, st, pad, dil):
     x, w, b = problem(xs, ws)
     exp = O.conv_fwd(x, w, b, st, pad, dil)
     exp_nobias = O.conv_fwd(x, w, None, st, pad, dil)
+    assert conv_ops.n_fwd_algos() == 3
     for v in range(conv_ops.n_fwd_algos()):
+        if v == 2 and not winograd_applies(ws, st, pad, dil, xs[1]):
+            assert refused(lambda: conv_ops.conv_forward(dev(x, cuda), dev(w, cuda), None, pad, st,
+                                                         dil, 1, v))
+            continue
         y = conv_ops.conv_forward(dev(x, cuda), dev(w, cuda), dev(b, cuda), pad, st, dil, 1, v)
         assert list(y.shape) == list(exp.shape)
         assert_rel(host(y), exp, TOL, f"forward variant {v}")
@@ -82,8 +108,12 @@ def test_conv_backward_data(cuda, xs, ws, st, pad, dil):
     yshape = O.conv_fwd(x, w, None, st, pad, dil).shape
     dy = np.random.default_rng(2).standard_normal(yshape).astype(np.float32)
     exp = O.conv_bwd_data(dy, w, xs, st, pad, dil)
+    assert conv_ops.n_bwd_ip_algos() == 3
     for v in range(conv_ops.n_bwd_ip_algos()):
-        # poison the output: the kernel must write every element
+        if v == 2 and not winograd_applies(ws, st, pad, dil, ws[0]):
+            assert refused(lambda: conv_ops.conv_backward_input(xs, dev(dy, cuda), dev(w, cuda),
+                                                                pad, st, dil, 1, v))
+            continue
         dx = conv_ops.conv_backward_input(xs, dev(dy, cuda), dev(w, cuda), pad, st, dil, 1, v)
         assert_rel(host(dx), exp, TOL, f"backward-data variant {v}")
 
@@ -210,25 +240,28 @@ def test_conv_bf16_all_directions(cuda, xs, ws, st, pad, dil):
     exp = O.conv_fwd(x, w, b, st, pad, dil)
     rng = np.random.default_rng(5)
     dy = bf16_round(rng.standard_normal(exp.shape))
-    for v in range(conv_ops.n_fwd_algos()):
+    assert conv_ops.n_fwd_algos(torch.bfloat16) == 1
+    for v in (0, 1):    # index 1 is accepted as an alias of the one bf16 kernel
         y = conv_ops.conv_forward(dev16(x, cuda), dev16(w, cuda), dev16(b, cuda), pad, st, dil, 1, v)
         assert y.dtype == torch.bfloat16 and y.is_contiguous(memory_format=torch.channels_last)
         assert_rel(host(y.float()), exp, BF16_TOL, f"bf16 forward variant {v}")
     y = conv_ops.conv_forward(dev16(x, cuda), dev16(w, cuda), None, pad, st, dil, 1, 0)
     assert_rel(host(y.float()), O.conv_fwd(x, w, None, st, pad, dil), BF16_TOL, "bf16 forward, no bias")
     exp_dx = O.conv_bwd_data(dy, w, xs, st, pad, dil)
-    for v in range(conv_ops.n_bwd_ip_algos()):
+    for v in (0, 1):
         dx = conv_ops.conv_backward_input(xs, dev16(dy, cuda), dev16(w, cuda), pad, st, dil, 1, v)
         assert dx.dtype == torch.bfloat16 and list(dx.shape) == list(xs)
         assert_rel(host(dx.float()), exp_dx, BF16_TOL, f"bf16 backward-data variant {v}")
     exp_dw = O.conv_bwd_weight(dy, x, ws, st, pad, dil)
-    for v in range(conv_ops.n_bwd_wt_algos()):
+    for v in (0, 1):
         dw = conv_ops.conv_backward_weight(ws, dev16(dy, cuda), dev16(x, cuda), pad, st, dil, 1, v)
         assert dw.dtype == torch.bfloat16 and list(dw.shape) == list(ws)
         assert_rel(host(dw.float()), exp_dw, BF16_TOL, f"bf16 backward-weight variant {v}")
     # reproducible: fixed-order reduction of the split partials
     dw2 = conv_ops.conv_backward_weight(ws, dev16(dy, cuda), dev16(x, cuda), pad, st, dil, 1, 0)
     assert torch.equal(dw, dw2)
+    # there is no bf16 Winograd tier
+    assert refused(lambda: conv_ops.conv_forward(dev16(x, cuda), dev16(w, cuda), None, pad, st, dil, 1, 2))
 
 
 def test_conv_bf16_rejects_channel_counts_the_tiles_cannot_hold(cuda):
@@ -271,6 +304,8 @@ def test_conv_backward_data_accumulates_into_an_existing_gradient(cuda, xs, ws, 
     prior = rng.standard_normal(xs).astype(np.float32)
     exp = prior.astype(np.float64) + O.conv_bwd_data(dy, w, xs, st, pad, dil)
     for v in range(conv_ops.n_bwd_ip_algos()):
+        if v == 2 and not winograd_applies(ws, st, pad, dil, ws[0]):
+            continue
         acc = dev(prior, cuda)
         out = conv_ops.conv_backward_input(xs, dev(dy, cuda), dev(w, cuda), pad, st, dil, 1, v,
                                            accumulate_into=acc)

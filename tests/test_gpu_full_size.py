@@ -125,7 +125,7 @@ def test_convolution_directions_are_adjoint_at_full_size(cuda, dtype, tol):
         x = x.to(dtype).contiguous(memory_format=torch.channels_last)
         w = w.to(dtype).contiguous(memory_format=torch.channels_last)
     dy = None
-    for v in range(conv_ops.n_fwd_algos()):
+    for v in range(conv_ops.n_fwd_algos(dtype)):
         y = conv_ops.conv_forward(x, w, None, 1, 1, 1, 1, v)
         if dy is None:
             dy = _randn(tuple(y.shape), cuda, 9)
@@ -135,10 +135,10 @@ def test_convolution_directions_are_adjoint_at_full_size(cuda, dtype, tol):
         # <conv(x, w), dy> is a sum of 9e6 products of independent values: its natural size is
         # sqrt(n) * rms(y) * rms(dy) (a wrong operand, e.g. transposed weights, is off by ~0.2 of it)
         scale = (y.numel() ** 0.5) * float(y.float().pow(2).mean().sqrt()) * float(dy.float().pow(2).mean().sqrt())
-        for vd in range(conv_ops.n_bwd_ip_algos()):
+        for vd in range(conv_ops.n_bwd_ip_algos(dtype)):
             dx = conv_ops.conv_backward_input(list(xs), dy, w, 1, 1, 1, 1, vd)
             assert abs(lhs - _dot(dx, x)) < tol * scale, (v, vd)
-        for vw in range(conv_ops.n_bwd_wt_algos()):
+        for vw in range(conv_ops.n_bwd_wt_algos(dtype)):
             dw = conv_ops.conv_backward_weight(list(ws), dy, x, 1, 1, 1, 1, vw)
             assert abs(lhs - _dot(dw, w)) < tol * scale, (v, vw)
         # linearity of the forward in x (exact up to rounding of the two results)
