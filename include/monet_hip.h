@@ -153,15 +153,17 @@ int mn_bn_bwd_from_y_f32(const float* dy, const float* y, const float* gamma, co
  * has no cross-block wait and so no counterpart of this call. */
 int mn_bn_ws_status(const void* ws, size_t ws_bytes, int64_t N, int64_t C, int64_t HW,
                     mn_stream_t stream);
-/* mn_bn_bwd_from_y_f32 with the two launch limits given explicitly (0 = the
+/* mn_bn_bwd_from_y_f32 with its launch parameters given explicitly (0 = the
  * default): `spin_limit` polls before a wait gives up, at most
- * `max_workgroups` persistent workgroups.  For diagnosis and for testing the
- * error path above from the host; no counterpart in the reference. */
+ * `max_workgroups` persistent workgroups, pieces of `channel_group`
+ * neighbouring channels handed out interleaved, `cache_hints` = 4 | 1 (loads
+ * non-temporal) | 2 (stores non-temporal).  For diagnosis and for testing
+ * the error path above from the host; no counterpart in the reference. */
 int mn_bn_bwd_from_y_f32_limits(const float* dy, const float* y, const float* gamma,
                                 const float* beta, const float* invstd, float* dx, float* dgamma,
                                 float* dbeta, int64_t N, int64_t C, int64_t HW, void* ws,
                                 size_t ws_bytes, uint32_t spin_limit, uint32_t max_workgroups,
-                                mn_stream_t stream);
+                                uint32_t channel_group, uint32_t cache_hints, mn_stream_t stream);
 
 /* mn_bn_bwd_from_y_f32 for callers that cannot allocate device memory or hand
  * over a workspace (code under HIP graph capture, tight serving loops,

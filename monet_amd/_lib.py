@@ -71,7 +71,8 @@ _SIGNATURES = {
     "mn_bn_bwd_from_y_f32": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64,
                                      _P, c_size_t, _P]),
     "mn_bn_bwd_from_y_f32_limits": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int64,
-                                            c_int64, _P, c_size_t, c_uint32, c_uint32, _P]),
+                                            c_int64, _P, c_size_t, c_uint32, c_uint32, c_uint32, c_uint32,
+                                            _P]),
     "mn_bn_ws_status": (c_int, [_P, c_size_t, c_int64, c_int64, c_int64, _P]),
     "mn_bn_bwd_from_y_static_f32": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int64,
                                             c_int64, _P]),

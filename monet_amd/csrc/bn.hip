@@ -99,13 +99,26 @@ struct CursorT {
 
 typedef CursorT<kThreads> Cursor;
 
-template <int VEC>
+// H: cache hints of the tensor accesses, bit 0 = loads non-temporal, bit 1 = stores non-temporal
+// (around the caches).  Right for planes that are whole cache lines, where every line is
+// touched once; wrong for planes that are not, where the first and last line of a plane are
+// shared with the neighbouring channel's plane: a non-temporal load fetches such a line once per
+// sharer and a non-temporal store writes it to memory in parts ([184,2048,7,7] forward: 2.2 TB/s
+// with both hints, 5.0 without).  A compile-time choice: a run-time one folds into plain accesses.
+constexpr int kNtLoad = 1, kNtStore = 2;
+template <int VEC, int H>
 __device__ __forceinline__ typename Vec<VEC>::type ldv(const float* p) {
-  return ld_stream(reinterpret_cast<const typename Vec<VEC>::type*>(p));
+  const typename Vec<VEC>::type* q = reinterpret_cast<const typename Vec<VEC>::type*>(p);
+  if (H & kNtLoad) return ld_stream(q);
+  return *q;
 }
-template <int VEC>
+template <int VEC, int H>
 __device__ __forceinline__ void stv(float* p, typename Vec<VEC>::type v) {
-  st_stream(reinterpret_cast<typename Vec<VEC>::type*>(p), v);
+  typename Vec<VEC>::type* q = reinterpret_cast<typename Vec<VEC>::type*>(p);
+  if (H & kNtStore)
+    st_stream(q, v);
+  else
+    *q = v;
 }
 __device__ __forceinline__ float comp(const float4_t& v, int k) { return v[k]; }
 __device__ __forceinline__ float comp(const float& v, int) { return v; }
@@ -213,7 +226,7 @@ __device__ __forceinline__ Gate make_gate(const Args& A, int c) {
 // ---------------------------------------------------------------- reduce --
 // (s0, s1) = ( sum a , sum a*(b - shift) )   backward
 //          = ( sum (b - K) , sum (b - K)^2 ) forward, K = first element of the channel
-template <int VEC, int MODE>
+template <int VEC, int MODE, int H>
 __device__ __forceinline__ void reduce_piece(const Args& A, int c, int piece, float sft, float& s0,
                                              float& s1) {
   typedef typename Vec<VEC>::type V;
@@ -230,9 +243,9 @@ __device__ __forceinline__ void reduce_piece(const Args& A, int c, int piece, fl
       ok[u] = cur.valid();
       if (ok[u]) {
         const size_t o = cur.off<VEC>(sh.C, c, sh.HW);
-        vb[u] = ldv<VEC>(A.b + o);
-        if (!is_fwd(MODE)) va[u] = ldv<VEC>(A.a + o);
-        if (MODE == BWD_FROM_X_GATED) va[u] = gate_by(va[u], ldv<VEC>(A.gate_ref + o));
+        vb[u] = ldv<VEC, H>(A.b + o);
+        if (!is_fwd(MODE)) va[u] = ldv<VEC, H>(A.a + o);
+        if (MODE == BWD_FROM_X_GATED) va[u] = gate_by(va[u], ldv<VEC, H>(A.gate_ref + o));
         if (MODE == BWD_FROM_X_MASKED) va[u] = gate_by_mask(va[u], A.mask_in, o);
       }
       cur.next();
@@ -266,7 +279,7 @@ __device__ __forceinline__ float reduce_shift(const Args& A, int c) {
 // ----------------------------------------------------------------- apply --
 // out = (a - (b - sft)*proj - gmean) * gscale     backward
 // out = (b - mean) * scale + bias                 forward (proj = mean, gmean = bias, gscale = scale)
-template <int VEC, int MODE>
+template <int VEC, int MODE, int H>
 __device__ __forceinline__ void apply_piece(const Args& A, int c, int piece, float sft, float proj,
                                             float gmean, float gscale) {
   typedef typename Vec<VEC>::type V;
@@ -283,9 +296,9 @@ __device__ __forceinline__ void apply_piece(const Args& A, int c, int piece, flo
       ok[u] = cur.valid();
       if (ok[u]) {
         o[u] = cur.off<VEC>(sh.C, c, sh.HW);
-        vb[u] = ldv<VEC>(A.b + o[u]);
-        if (MODE != FWD_TRAIN) va[u] = ldv<VEC>(A.a + o[u]);
-        if (MODE == BWD_FROM_X_GATED) va[u] = gate_by(va[u], ldv<VEC>(A.gate_ref + o[u]));
+        vb[u] = ldv<VEC, H>(A.b + o[u]);
+        if (MODE != FWD_TRAIN) va[u] = ldv<VEC, H>(A.a + o[u]);
+        if (MODE == BWD_FROM_X_GATED) va[u] = gate_by(va[u], ldv<VEC, H>(A.gate_ref + o[u]));
         if (MODE == BWD_FROM_X_MASKED) va[u] = gate_by_mask(va[u], A.mask_in, o[u]);
       }
       cur.next();
@@ -305,8 +318,8 @@ __device__ __forceinline__ void apply_piece(const Args& A, int c, int piece, flo
             setc(r, k, (gate(comp(va[u], k), d) - d * proj - gmean) * gscale);
           }
         }
-        stv<VEC>(A.out + o[u], r);
-        if (hands_on_gradient(MODE)) stv<VEC>(A.gated_out + o[u], va[u] * A.ralpha);
+        stv<VEC, H>(A.out + o[u], r);
+        if (hands_on_gradient(MODE)) stv<VEC, H>(A.gated_out + o[u], va[u] * A.ralpha);
         if (MODE == FWD_TRAIN_ADD && VEC == 4 && A.mask_out) put_mask(A.mask_out, o[u], r);
       }
     }
@@ -382,7 +395,7 @@ __device__ __forceinline__ void channel_totals(const float* partial, int c, int 
 }
 
 // ------------------------------------------------- two-launch formulation --
-template <int VEC, int MODE>
+template <int VEC, int MODE, int H>
 __global__ __launch_bounds__(kThreads) void bn_reduce_kernel(const Args A) {
   __shared__ float lds[2 * kWaves];
   const int c = blockIdx.x / A.sh.S;
@@ -391,7 +404,7 @@ __global__ __launch_bounds__(kThreads) void bn_reduce_kernel(const Args A) {
   if (is_fwd(MODE) && piece == 0 && threadIdx.x == 0) A.pivot[c] = sft;
   if (blockIdx.x == 0 && threadIdx.x == 0) *A.error = 0u;  // this formulation never waits
   float s0, s1;
-  reduce_piece<VEC, MODE>(A, c, piece, sft, s0, s1);
+  reduce_piece<VEC, MODE, H>(A, c, piece, sft, s0, s1);
   block_sum2<kWaves>(s0, s1, lds);
   if (threadIdx.x == 0) {
     A.partial[2 * (size_t)blockIdx.x] = s0;
@@ -399,7 +412,7 @@ __global__ __launch_bounds__(kThreads) void bn_reduce_kernel(const Args A) {
   }
 }
 
-template <int VEC, int MODE>
+template <int VEC, int MODE, int H>
 __global__ __launch_bounds__(kThreads) void bn_apply_kernel(const Args A) {
   const int c = blockIdx.x / A.sh.S;
   const int piece = blockIdx.x - c * A.sh.S;
@@ -408,18 +421,18 @@ __global__ __launch_bounds__(kThreads) void bn_apply_kernel(const Args A) {
   coefficients<MODE>(A, c, piece, t0, t1, is_fwd(MODE) ? A.pivot[c] : 0.f, sft, proj, gmean,
                      gscale);
   if (!A.out) return;
-  apply_piece<VEC, MODE>(A, c, piece, sft, proj, gmean, gscale);
+  apply_piece<VEC, MODE, H>(A, c, piece, sft, proj, gmean, gscale);
 }
 
 // Forward from saved statistics (no reduction).
-template <int VEC, int MODE>
+template <int VEC, int MODE, int H>
 __global__ __launch_bounds__(kThreads) void bn_fwd_saved_kernel(const Args A, const float* mean,
                                                                 const float* invstd) {
   const int c = blockIdx.x / A.sh.S;
   const int piece = blockIdx.x - c * A.sh.S;
   const float scale = invstd[c] * (A.gamma ? A.gamma[c] : 1.f);
   const float bias = A.shift ? A.shift[c] : 0.f;
-  apply_piece<VEC, MODE>(A, c, piece, 0.f, mean[c], bias, scale);
+  apply_piece<VEC, MODE, H>(A, c, piece, 0.f, mean[c], bias, scale);
 }
 
 // ------------------------------------------------- one-launch formulation --
@@ -497,7 +510,7 @@ struct Held {
 
 // Load a piece, reduce it and publish its partial pair.  Never waits for
 // another workgroup.
-template <int VEC, int MODE, int KEEP, int THREADS, bool SOLO = false>
+template <int VEC, int MODE, int KEEP, int THREADS, int H, bool SOLO = false>
 __device__ __forceinline__ void hold_piece(const Args& A, uint32_t item, Held<VEC, KEEP>& h,
                                            float* lds) {
   typedef CursorT<THREADS> Cursor;
@@ -524,8 +537,8 @@ __device__ __forceinline__ void hold_piece(const Args& A, uint32_t item, Held<VE
     for (int k = 0; k < KEEP; ++k) {
       if (cur.valid()) {
         const size_t o = cur.template off<VEC>(sh.C, h.c, sh.HW);
-        h.b[k] = ldv<VEC>(A.b + o);
-        if (MODE != FWD_TRAIN) h.a[k] = ldv<VEC>(A.a + o);
+        h.b[k] = ldv<VEC, H>(A.b + o);
+        if (MODE != FWD_TRAIN) h.a[k] = ldv<VEC, H>(A.a + o);
       }
       cur.next();
     }
@@ -536,7 +549,7 @@ __device__ __forceinline__ void hold_piece(const Args& A, uint32_t item, Held<VE
     typename Vec<VEC>::type ref[KEEP];
 #pragma unroll
     for (int k = 0; k < KEEP; ++k) {
-      if (cur.valid()) ref[k] = ldv<VEC>(A.gate_ref + cur.template off<VEC>(sh.C, h.c, sh.HW));
+      if (cur.valid()) ref[k] = ldv<VEC, H>(A.gate_ref + cur.template off<VEC>(sh.C, h.c, sh.HW));
       cur.next();
     }
     Cursor cur2(sh, h.piece);
@@ -544,7 +557,7 @@ __device__ __forceinline__ void hold_piece(const Args& A, uint32_t item, Held<VE
     for (int k = 0; k < KEEP; ++k) {
       if (cur2.valid()) {
         h.a[k] = gate_by(h.a[k], ref[k]);
-        stv<VEC>(A.gated_out + cur2.template off<VEC>(sh.C, h.c, sh.HW), h.a[k] * A.ralpha);
+        stv<VEC, H>(A.gated_out + cur2.template off<VEC>(sh.C, h.c, sh.HW), h.a[k] * A.ralpha);
       }
       cur2.next();
     }
@@ -556,7 +569,7 @@ __device__ __forceinline__ void hold_piece(const Args& A, uint32_t item, Held<VE
       if (cur.valid()) {
         const size_t o = cur.template off<VEC>(sh.C, h.c, sh.HW);
         h.a[k] = gate_by_mask(h.a[k], A.mask_in, o);
-        stv<VEC>(A.gated_out + o, h.a[k] * A.ralpha);
+        stv<VEC, H>(A.gated_out + o, h.a[k] * A.ralpha);
       }
       cur.next();
     }
@@ -594,7 +607,7 @@ __device__ __forceinline__ void hold_piece(const Args& A, uint32_t item, Held<VE
 }
 
 // Wait for the channel totals of a held piece and write its result.
-template <int VEC, int MODE, int KEEP, int THREADS, bool SOLO = false>
+template <int VEC, int MODE, int KEEP, int THREADS, int H, bool SOLO = false>
 __device__ __forceinline__ void finish_piece(const Args& A, const Held<VEC, KEEP>& h, float* lds) {
   typedef typename Vec<VEC>::type V;
   typedef CursorT<THREADS> Cursor;
@@ -627,7 +640,7 @@ __device__ __forceinline__ void finish_piece(const Args& A, const Held<VEC, KEEP
         }
       }
       const size_t o = cur.template off<VEC>(sh.C, h.c, sh.HW);
-      stv<VEC>(A.out + o, r);
+      stv<VEC, H>(A.out + o, r);
       if (MODE == FWD_TRAIN_ADD && VEC == 4 && A.mask_out) put_mask(A.mask_out, o, r);
     }
     cur.next();
@@ -640,7 +653,7 @@ __device__ __forceinline__ void finish_piece(const Args& A, const Held<VEC, KEEP
 // are handed out in ticket order, so the lowest unfinished channel always has
 // all its pieces either published or about to be taken by a running workgroup
 // (at least kMaxResident workgroups run at once).
-template <int VEC, int MODE, int KEEP, int THREADS>
+template <int VEC, int MODE, int KEEP, int THREADS, int H>
 __global__ __launch_bounds__(THREADS) void bn_resident_kernel(const Args A, uint32_t items) {
   __shared__ float lds[2 * (THREADS / MN_WAVE)];
   __shared__ uint32_t s_ticket;
@@ -654,15 +667,15 @@ __global__ __launch_bounds__(THREADS) void bn_resident_kernel(const Args A, uint
   };
   uint32_t i0 = take();
   if (i0 >= items) return;
-  hold_piece<VEC, MODE, KEEP, THREADS>(A, i0, h0, lds);
+  hold_piece<VEC, MODE, KEEP, THREADS, H>(A, i0, h0, lds);
   for (;;) {
     const uint32_t i1 = take();
-    if (i1 < items) hold_piece<VEC, MODE, KEEP, THREADS>(A, i1, h1, lds);
-    finish_piece<VEC, MODE, KEEP, THREADS>(A, h0, lds);
+    if (i1 < items) hold_piece<VEC, MODE, KEEP, THREADS, H>(A, i1, h1, lds);
+    finish_piece<VEC, MODE, KEEP, THREADS, H>(A, h0, lds);
     if (i1 >= items) break;
     i0 = take();
-    if (i0 < items) hold_piece<VEC, MODE, KEEP, THREADS>(A, i0, h0, lds);
-    finish_piece<VEC, MODE, KEEP, THREADS>(A, h1, lds);
+    if (i0 < items) hold_piece<VEC, MODE, KEEP, THREADS, H>(A, i0, h0, lds);
+    finish_piece<VEC, MODE, KEEP, THREADS, H>(A, h1, lds);
     if (i0 >= items) break;
   }
 }
@@ -670,7 +683,7 @@ __global__ __launch_bounds__(THREADS) void bn_resident_kernel(const Args A, uint
 // Channels short enough for ONE workgroup's registers (N*HW <= THREADS * KEEP vectors, e.g.
 // 14 x 14 and 7 x 7 planes at batch 184): a workgroup takes whole channels, so there is nothing
 // to publish, poll or prepare - one launch, no workspace traffic, no atomics.
-template <int VEC, int MODE, int KEEP, int THREADS>
+template <int VEC, int MODE, int KEEP, int THREADS, int H>
 __global__ __launch_bounds__(THREADS) void bn_solo_kernel(const Args A) {
   __shared__ float lds[2 * (THREADS / MN_WAVE)];
   Held<VEC, KEEP> h;
@@ -679,8 +692,8 @@ __global__ __launch_bounds__(THREADS) void bn_solo_kernel(const Args A) {
   // first and last lines.  Each XCD takes a contiguous range of channels, so the shared lines
   // meet in one L2 instead of being fetched (and written back in parts) by two.
   for (uint32_t c = xcd_slot(); c < (uint32_t)A.sh.C; c += gridDim.x) {
-    hold_piece<VEC, MODE, KEEP, THREADS, true>(A, c, h, lds);
-    finish_piece<VEC, MODE, KEEP, THREADS, true>(A, h, lds);
+    hold_piece<VEC, MODE, KEEP, THREADS, H, true>(A, c, h, lds);
+    finish_piece<VEC, MODE, KEEP, THREADS, H, true>(A, h, lds);
   }
 }
 
@@ -695,6 +708,8 @@ struct Tuning {
   int threads = 256;         // workgroup size of the resident kernel
   int grid = 768;            // persistent workgroups of the resident kernel (3 per CU)
   uint32_t spin_limit = 1u << 22;  // polls of one slot (seconds) before a wait gives up
+  int group = 0;             // channels whose pieces are handed out interleaved (0: chosen here)
+  int hints = 0;             // 0: chosen from the plane size; else 4 | kNtLoad and / or kNtStore
 };
 
 static bool shape_limits(int64_t N, int64_t C, int64_t HW) {
@@ -737,10 +752,34 @@ static void fill_shape(int64_t N, int64_t C, int64_t HW, int vec, int64_t S, uin
   sh.G = 1;
 }
 
+// Cache hints by plane size, from measurements at batch 184: planes of whole cache lines stream
+// fastest around the caches (56 x 56, 112 x 112); planes that share their end lines with the
+// neighbouring channel want ordinary stores, so that the parts of a line meet in L2 (28 x 28,
+// 14 x 14: 4.4 -> 5.1 TB/s), and below a few lines per plane ordinary loads as well (7 x 7:
+// 2.4 -> 5.3 TB/s).  With both plain at 14 x 14 / 28 x 28 the two streams evict each other.
+static int cache_hints(int64_t HW, int forced = 0) {
+  const int64_t plane = HW * (int64_t)sizeof(float);
+  if (forced) return forced & (kNtLoad | kNtStore);
+  if (plane % 128 == 0) return kNtLoad | kNtStore;
+  if (plane < 512) return 0;
+  return kNtLoad;
+}
+// Runs `CALL(H)` with the compile-time constant H equal to the run-time `hints`.
+#define MN_BN_WITH_HINTS(hints, CALL)        \
+  do {                                       \
+    switch (hints) {                         \
+      case 0: CALL(0); break;                \
+      case kNtLoad: CALL(kNtLoad); break;    \
+      case kNtStore: CALL(kNtStore); break;  \
+      default: CALL(kNtLoad | kNtStore);     \
+    }                                        \
+  } while (0)
+
 template <int MODE>
 static int run(Args& A, int64_t N, int64_t C, int64_t HW, bool aligned16, void* ws,
                const Tuning& t, hipStream_t s) {
   const int vec = (HW % 4 == 0 && aligned16) ? 4 : 1;
+  const int hints = cache_hints(HW, t.hints);
   A.partial = static_cast<float*>(ws);
   uint32_t* counters = reinterpret_cast<uint32_t*>(A.partial + ws_floats(N, C, HW));
   A.pivot = reinterpret_cast<float*>(counters) - C;  // last C floats of the float area
@@ -771,7 +810,10 @@ static int run(Args& A, int64_t N, int64_t C, int64_t HW, bool aligned16, void* 
 #define MN_BN_SOLO(V, K, T)                                              \
   do {                                                                   \
     fill_shape(N, C, HW, V, 1, (uint64_t)(T) * (K), A.sh);               \
-    bn_solo_kernel<V, MODE, K, T><<<grid, T, 0, s>>>(A);                 \
+    if (hints == 0) bn_solo_kernel<V, MODE, K, T, 0><<<grid, T, 0, s>>>(A);                         \
+    else if (hints == kNtLoad) bn_solo_kernel<V, MODE, K, T, kNtLoad><<<grid, T, 0, s>>>(A);        \
+    else if (hints == kNtStore) bn_solo_kernel<V, MODE, K, T, kNtStore><<<grid, T, 0, s>>>(A);      \
+    else bn_solo_kernel<V, MODE, K, T, kNtLoad | kNtStore><<<grid, T, 0, s>>>(A);                   \
     return mn_launch_status();                                           \
   } while (0)
     if (vec == 4 && chan <= 256u * 9u) MN_BN_SOLO(4, 9, 256);
@@ -790,13 +832,20 @@ static int run(Args& A, int64_t N, int64_t C, int64_t HW, bool aligned16, void* 
     // Not with one workgroup per CU (`wide`): a channel then completes G times later and nothing
     // else on the CU covers the wait (64 x 112 x 112 at batch 184: 0.377 -> 0.454 ms with G = 3).
     A.sh.G = wide ? 1 : (int)(448 / rp < 1 ? 1 : (448 / rp > 8 ? 8 : 448 / rp));
+    if (t.group > 0) A.sh.G = t.group;
     bn_prepare_kernel<<<(blocks + 255) / 256, 256, 0, s>>>(
           reinterpret_cast<uint64_t*>(A.partial), blocks, A.ticket, A.error);
     // persistent grid: enough workgroups to fill 256 CUs at this register footprint
     // (512-thread workgroups: one per CU at this register footprint)
     const unsigned want = (wide && t.grid > 256) ? 256u : (unsigned)t.grid;
     const unsigned grid = blocks < want ? blocks : want;
-#define MN_BN_RES(V, K, T) bn_resident_kernel<V, MODE, K, T><<<grid, T, 0, s>>>(A, blocks)
+#define MN_BN_RES(V, K, T)                                                                          \
+  do {                                                                                              \
+    if (hints == 0) bn_resident_kernel<V, MODE, K, T, 0><<<grid, T, 0, s>>>(A, blocks);             \
+    else if (hints == kNtLoad) bn_resident_kernel<V, MODE, K, T, kNtLoad><<<grid, T, 0, s>>>(A, blocks); \
+    else if (hints == kNtStore) bn_resident_kernel<V, MODE, K, T, kNtStore><<<grid, T, 0, s>>>(A, blocks); \
+    else bn_resident_kernel<V, MODE, K, T, kNtLoad | kNtStore><<<grid, T, 0, s>>>(A, blocks);       \
+  } while (0)
     if (vec == 4) {
       if (wide || long_pieces) MN_BN_RES(4, 8, 512);
       else MN_BN_RES(4, 8, 256);
@@ -814,13 +863,18 @@ static int run(Args& A, int64_t N, int64_t C, int64_t HW, bool aligned16, void* 
   if (S < 1) S = 1;
   fill_shape(N, C, HW, vec, S, (tot + S - 1) / S, A.sh);
   const unsigned blocks = (unsigned)(C * S);
-  if (vec == 4) {
-    bn_reduce_kernel<4, MODE><<<blocks, kThreads, 0, s>>>(A);
-    bn_apply_kernel<4, MODE><<<blocks, kThreads, 0, s>>>(A);
-  } else {
-    bn_reduce_kernel<1, MODE><<<blocks, kThreads, 0, s>>>(A);
-    bn_apply_kernel<1, MODE><<<blocks, kThreads, 0, s>>>(A);
-  }
+#define MN_BN_TWO(H)                                              \
+  do {                                                            \
+    if (vec == 4) {                                               \
+      bn_reduce_kernel<4, MODE, H><<<blocks, kThreads, 0, s>>>(A); \
+      bn_apply_kernel<4, MODE, H><<<blocks, kThreads, 0, s>>>(A);  \
+    } else {                                                      \
+      bn_reduce_kernel<1, MODE, H><<<blocks, kThreads, 0, s>>>(A); \
+      bn_apply_kernel<1, MODE, H><<<blocks, kThreads, 0, s>>>(A);  \
+    }                                                             \
+  } while (0)
+  MN_BN_WITH_HINTS(hints, MN_BN_TWO);
+#undef MN_BN_TWO
   return mn_launch_status();
 }
 
@@ -941,18 +995,24 @@ static int bn_fwd_apply(const float* x, const float* mean, const float* invstd, 
   A.a = added;
   A.ralpha = alpha;
   A.mask_out = (vec == 4 && HW % 8 == 0) ? mask : nullptr;
+  const int hints = cache_hints(HW);
   const unsigned blocks = (unsigned)C * A.sh.S;
   hipStream_t s = mn_stream(stream);
-  if (added) {
-    if (vec == 4)
-      bn_fwd_saved_kernel<4, FWD_TRAIN_ADD><<<blocks, kThreads, 0, s>>>(A, mean, invstd);
-    else
-      bn_fwd_saved_kernel<1, FWD_TRAIN_ADD><<<blocks, kThreads, 0, s>>>(A, mean, invstd);
-  } else if (vec == 4) {
-    bn_fwd_saved_kernel<4, FWD_TRAIN><<<blocks, kThreads, 0, s>>>(A, mean, invstd);
-  } else {
-    bn_fwd_saved_kernel<1, FWD_TRAIN><<<blocks, kThreads, 0, s>>>(A, mean, invstd);
-  }
+#define MN_BN_SAVED(H)                                                                        \
+  do {                                                                                        \
+    if (added) {                                                                              \
+      if (vec == 4)                                                                           \
+        bn_fwd_saved_kernel<4, FWD_TRAIN_ADD, H><<<blocks, kThreads, 0, s>>>(A, mean, invstd); \
+      else                                                                                    \
+        bn_fwd_saved_kernel<1, FWD_TRAIN_ADD, H><<<blocks, kThreads, 0, s>>>(A, mean, invstd); \
+    } else if (vec == 4) {                                                                    \
+      bn_fwd_saved_kernel<4, FWD_TRAIN, H><<<blocks, kThreads, 0, s>>>(A, mean, invstd);      \
+    } else {                                                                                  \
+      bn_fwd_saved_kernel<1, FWD_TRAIN, H><<<blocks, kThreads, 0, s>>>(A, mean, invstd);      \
+    }                                                                                         \
+  } while (0)
+  MN_BN_WITH_HINTS(hints, MN_BN_SAVED);
+#undef MN_BN_SAVED
   return mn_launch_status();
 }
 
@@ -1090,8 +1150,10 @@ int mn_bn_bwd_from_y_f32_limits(const float* dy, const float* y, const float* ga
                                 const float* beta, const float* invstd, float* dx, float* dgamma,
                                 float* dbeta, int64_t N, int64_t C, int64_t HW, void* ws,
                                 size_t ws_bytes, uint32_t spin_limit, uint32_t max_workgroups,
-                                mn_stream_t stream) {
+                                uint32_t channel_group, uint32_t cache_hints, mn_stream_t stream) {
   mn_bn::Tuning t;
+  t.hints = (int)(cache_hints & 7u);
+  t.group = (int)(channel_group < 4096u ? channel_group : 4096u);
   if (spin_limit) t.spin_limit = spin_limit;
   if (max_workgroups) t.grid = (int)(max_workgroups < 65535u ? max_workgroups : 65535u);
   return mn_bn::bwd_launch(true, dy, y, gamma, beta, invstd, dx, dgamma, dbeta, N, C, HW, ws,

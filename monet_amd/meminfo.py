@@ -135,6 +135,8 @@ def computeinfo(n, op, graph, bs, bwd_op, conv_mode, inplace_mode, *params):
             op.algorithm = alg
             try:
                 runtime_fwd.append(_timed(lambda: op.forward(*args)))
+                if op.algorithm != alg:   # refused for this shape: the operator fell back
+                    runtime_fwd[-1] = -1
             except Exception as e:
                 print("C: Failed fwd algo", alg, e)
                 runtime_fwd.append(-1)
@@ -175,6 +177,8 @@ def computeinfo(n, op, graph, bs, bwd_op, conv_mode, inplace_mode, *params):
                 op.algorithm = step + alg
                 try:
                     runtime_bwd.append(_timed(lambda: op.backward(gradin, stored, nodel=True)))
+                    if op.algorithm != step + alg:   # refused: the operator fell back
+                        runtime_bwd[-1] = -1
                 except Exception as e:
                     print("C: Failed bwd algo", alg, e)
                     runtime_bwd.append(-1)

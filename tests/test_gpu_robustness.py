@@ -32,7 +32,7 @@ def _from_y_with_limits(y, gamma, beta, invstd, dy, ws, spin_limit, max_workgrou
     db = torch.empty(C, device=y.device)
     _lib.call("mn_bn_bwd_from_y_f32_limits", _lib.ptr(dy), _lib.ptr(y), _lib.ptr(gamma),
               _lib.ptr(beta), _lib.ptr(invstd), _lib.ptr(dx), _lib.ptr(dg), _lib.ptr(db), N, C, HW,
-              _lib.ptr(ws), ws.numel(), spin_limit, max_workgroups, _lib.stream_ptr(y.device))
+              _lib.ptr(ws), ws.numel(), spin_limit, max_workgroups, 0, 0, _lib.stream_ptr(y.device))
     return dx, dg, db
 
 
