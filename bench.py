@@ -29,10 +29,66 @@ if str(ROOT) not in sys.path:
     sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth, GB/s
-# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `--only lm_ops`, scaled by
-# what the same counters read for a plain copy of known size (FETCH_SIZE x2.000, WRITE_SIZE x1.000);
-# the counter run cannot happen inside this program, so the figures are recorded here
-TRAFFIC = {"bn_bwd_from_output": 1775575040, "relu_bwd_mask": 1200261120, "maxpool_bwd_idx": 778724352}
+# HBM bytes per launch come from hardware counters, which cannot be read inside this program:
+# two `rocprofv3 --pmc` runs of `bench.py --only lm_ops` (FETCH_SIZE, then WRITE_SIZE), turned
+# into this file by `bench.py --traffic-summary FETCH_DIR WRITE_DIR` (counter values scaled by
+# what the same counter reads for the plain copy of known size that `--only lm_ops` makes first)
+TRAFFIC_FILE = ROOT / "profiles" / "lm_ops_bs184_hbm_traffic.json"
+# kernel (substring of its name in the counter output) behind each operator of the step
+TRAFFIC_KERNELS = {"bn_bwd_from_output": "bn_resident_kernel<4, 1,", "relu_bwd_mask": "relu_bwd_mask_vec",
+                   "maxpool_bwd_idx": "maxpool_bwd_k3s2p1_kernel",
+                   "linear_triad_2r1w (torch add, same tensors)": "vectorized_elementwise_kernel"}
+
+
+def load_traffic():
+    """{operator: HBM bytes per launch} from the committed counter summary, {} if absent."""
+    try:
+        return {k: int(v) for k, v in json.loads(TRAFFIC_FILE.read_text())["bytes_per_launch"].items()}
+    except (OSError, ValueError, KeyError):
+        return {}
+
+
+def traffic_summary(fetch_dir, write_dir):
+    """Write TRAFFIC_FILE from the counter_collection.csv files of the two counter runs."""
+    import csv
+    copy_bytes = E * 4   # the yardstick copy reads and writes one tensor of E floats
+
+    def per_kernel(folder, counter):
+        acc = {}
+        for f in Path(folder).rglob("*counter_collection.csv"):
+            with open(f, newline="") as fh:
+                for r in csv.DictReader(fh):
+                    if r["Counter_Name"] == counter:
+                        acc.setdefault(r["Kernel_Name"], []).append(float(r["Counter_Value"]))
+        return acc
+
+    def pick(acc, needle, largest=False):
+        hits = [(k, v) for k, v in acc.items() if needle in k]
+        if not hits:
+            return None
+        if largest:   # torch launches small element-wise kernels too: the triad is the big one
+            hits = [max(hits, key=lambda kv: max(kv[1]))]
+            return max(hits[0][1])
+        vals = [x for _, v in hits for x in v]
+        return sum(vals) / len(vals)
+    fetch, write = per_kernel(fetch_dir, "FETCH_SIZE"), per_kernel(write_dir, "WRITE_SIZE")
+    yard_f, yard_w = pick(fetch, "copyBuffer"), pick(write, "copyBuffer")
+    if not yard_f or not yard_w:
+        raise SystemExit("no copy kernel in the counter output: run `bench.py --only lm_ops`")
+    scale_f, scale_w = copy_bytes / (yard_f * 1024.0), copy_bytes / (yard_w * 1024.0)
+    out = {}
+    for op, needle in TRAFFIC_KERNELS.items():
+        big = "triad" in op
+        f, w = pick(fetch, needle, big), pick(write, needle, big)
+        if f is not None and w is not None:
+            out[op] = int(round(f * 1024.0 * scale_f + w * 1024.0 * scale_w))
+    doc = {"what": "HBM bytes per launch = FETCH_SIZE and WRITE_SIZE (KiB per dispatch) of two rocprofv3 "
+                   "--pmc runs of `python3 bench.py --only lm_ops --steps 3 --warmup 1`, each scaled by "
+                   "what the same counter reads for a plain copy of %d bytes" % copy_bytes,
+           "scale": {"FETCH_SIZE": round(scale_f, 4), "WRITE_SIZE": round(scale_w, 4)},
+           "bytes_per_launch": out}
+    TRAFFIC_FILE.write_text(json.dumps(doc, indent=1) + "\n")
+    print(json.dumps(doc))
 
 N, C, H, W = 184, 256, 56, 56          # BN / ReLU tensor
 PN, PC, PH_IN, PW_IN = 184, 64, 112, 112  # max-pool input
@@ -82,10 +138,16 @@ def gpu_bench(steps, warmup, calibrate=False):
 
     if calibrate:
         # one plain copy of E floats (E*4 bytes read, E*4 written): the yardstick the HBM
-        # traffic counters of the other kernels are scaled by
-        torch.empty_like(dy).copy_(dy)
+        # traffic counters of the other kernels are scaled by; and a 2-read-1-write pass over
+        # the same three tensors in plain address order (the BatchNorm backward visits the
+        # same bytes channel by channel)
+        scratch = torch.empty_like(dy)
+        scratch.copy_(dy)
+        torch.add(dy, y, out=scratch)
+        del scratch
     ops = [("bn_bwd_from_output", op_bn, BYTES_BN), ("relu_bwd_mask", op_relu, BYTES_RELU),
            ("maxpool_bwd_idx", op_pool, BYTES_POOL)]
+    traffic = load_traffic()
     for _ in range(warmup):
         for _, fn, _ in ops:
             fn()
@@ -107,7 +169,24 @@ def gpu_bench(steps, warmup, calibrate=False):
         ms = sum(a.elapsed_time(b) for a, b in ev[name]) / steps
         gbs = nbytes / (ms * 1e-3) / 1e9
         kernels[name] = {"ms": round(ms, 4), "bytes": nbytes, "GB/s": round(gbs, 1),
-                         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC[name]}
+                         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": traffic.get(name)}
+    # ceiling for a 2-read-1-write pass over tensors of this size in plain address order
+    tri_out = torch.empty_like(dy)
+    for _ in range(warmup):
+        torch.add(dy, y, out=tri_out)
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    a.record()
+    for _ in range(steps):
+        torch.add(dy, y, out=tri_out)
+    b.record()
+    torch.cuda.synchronize()
+    ms = a.elapsed_time(b) / steps
+    kernels["linear_triad_2r1w"] = {"ms": round(ms, 4), "bytes": BYTES_BN,
+                                    "GB/s": round(BYTES_BN / (ms * 1e-3) / 1e9, 1),
+                                    "frac": round(BYTES_BN / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                                    "in_step": False, "what": "torch.add over the same three tensors"}
+    del tri_out
     # the forward kernels of the same operators, timed on their own (not part of the step)
     x = torch.randn(N, C, H, W, device=dev)
     px = torch.randn(PN, PC, PH_IN, PW_IN, device=dev)
@@ -227,17 +306,17 @@ def conv_bench(steps, warmup):
 
 E2E_MODE = "inplace_conv_multiway_newnode"
 E2E_BS = 184
+UNET_BS = 11
 
 
-def _train_ms(model, x, target, iters, warmup):
-    """ms per SGD step (forward, cross entropy, backward, momentum update) and peak MB."""
+def _train_ms(model, x, loss_fn, iters, warmup):
+    """ms per SGD step (forward, loss, backward, momentum update) and peak MB."""
     import torch
     opt = torch.optim.SGD(model.parameters(), lr=0.01, momentum=0.9)
-    crit = torch.nn.CrossEntropyLoss()
 
     def step():
         opt.zero_grad(set_to_none=True)
-        crit(model(x), target).backward()
+        loss_fn(model(x)).backward()
         opt.step()
     for _ in range(warmup):
         step()
@@ -253,46 +332,87 @@ def _train_ms(model, x, target, iters, warmup):
     return t0.elapsed_time(t1) / iters, torch.cuda.max_memory_allocated() / 2**20
 
 
-def end_to_end(iters=10, warmup=3):
-    """ResNet-50 (torchvision topology, random init), batch 184, fp32 SGD steps: under the
-    solved 10 GB and 6 GB schedules, under the unconstrained schedule (same kernels, nothing
-    recomputed) and with stock PyTorch autograd.  Overhead is against the unconstrained run."""
+def _schedules(name, bs, make_model, input_shape, x, loss_fn, modes, iters, warmup, res):
+    """Times `make_model()` under every committed schedule of `modes` (unconstrained, 10 GB,
+    6 GB), then with stock PyTorch autograd.  Overhead is against the unconstrained schedule
+    of the same operator set; peak_MB is the allocator's peak over the timed steps, with
+    weights, batch, gradients and optimizer state."""
+    import torch
+
+    from monet_amd.monet_wrapper import MONeTWrapper
+    dev = x.device
+    for suffix, mode in modes:
+        base = None
+        for budget in (100, 10, 6):
+            sol = ROOT / "data" / ("solution_%s_%d_%s_%.2f.pkl" % (name, bs, mode, budget))
+            if not sol.exists():
+                continue
+            model = MONeTWrapper(make_model(), str(sol), input_shape).to(dev)
+            model.train()
+            ms, mb = _train_ms(model, x, loss_fn, iters, warmup)
+            key = ("unconstrained" if budget == 100 else "budget_%dGB" % budget) + suffix
+            res[key] = {"images_per_s": round(bs / ms * 1e3, 1), "ms_per_step": round(ms, 2),
+                        "peak_MB": round(mb, 1)}
+            if budget == 100:
+                base = ms
+            else:
+                res[key]["within_budget"] = bool(mb <= budget * 1024)
+                if base:
+                    res[key]["overhead_vs_unconstrained"] = round(ms / base - 1.0, 4)
+            del model
+            torch.cuda.empty_cache()
+    model = make_model().to(dev).train()
+    ms, mb = _train_ms(model, x, loss_fn, iters, warmup)
+    res["stock_pytorch"] = {"images_per_s": round(bs / ms * 1e3, 1), "ms_per_step": round(ms, 2),
+                            "peak_MB": round(mb, 1)}
+    del model
+    torch.cuda.empty_cache()
+    return res
+
+
+def end_to_end(iters=20, warmup=10):
+    """ResNet-50 (torchvision topology, random init), batch 184, fp32 SGD steps with cross
+    entropy over 1000 classes: under the solved 10 GB and 6 GB schedules, under the
+    unconstrained schedule (same kernels, nothing recomputed) and with stock PyTorch autograd;
+    three operator sets (the reference's; BatchNorm+ReLU and add+ReLU pairs fused; also
+    BatchNorm+add+ReLU at the end of a residual block).  Timing protocol of the reference
+    (monet/schedule.py:430-443) with 10 instead of 100 warm-up steps: 20 timed steps between
+    two events."""
     import torch
 
     from monet_amd.models import resnet50
-    from monet_amd.monet_wrapper import MONeTWrapper
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
     x = torch.randn(E2E_BS, 3, 224, 224, device=dev)
     target = torch.randint(0, 1000, (E2E_BS,), device=dev)
     res = {"model": "resnet50", "batch": E2E_BS, "dtype": "f32", "unit": "images/s",
-           "step": "forward + cross entropy + backward + SGD momentum update"}
-    # op set of the reference, then the same with BatchNorm+ReLU and add+ReLU pairs fused into
-    # one operator each, then also with BatchNorm+add+ReLU triples (the end of a residual block)
-    for suffix, mode in (("", E2E_MODE), ("_fused", "fused_" + E2E_MODE),
-                         ("_fused2", "fused2_" + E2E_MODE)):
-        base = None
-        for budget in (100, 10, 6):
-            sol = ROOT / "data" / ("solution_resnet50_%d_%s_%.2f.pkl" % (E2E_BS, mode, budget))
-            if not sol.exists():
-                continue
-            model = MONeTWrapper(resnet50(), str(sol), (3, 224, 224)).to(dev)
-            model.train()
-            ms, mb = _train_ms(model, x, target, iters, warmup)
-            key = ("unconstrained" if budget == 100 else "budget_%dGB" % budget) + suffix
-            res[key] = {"images_per_s": round(E2E_BS / ms * 1e3, 1), "ms_per_step": round(ms, 2),
-                        "peak_MB": round(mb, 1)}
-            if budget == 100:
-                base = ms
-            elif base:
-                res[key]["overhead_vs_unconstrained"] = round(ms / base - 1.0, 4)
-            del model
-            torch.cuda.empty_cache()
-    model = resnet50().to(dev).train()
-    ms, mb = _train_ms(model, x, target, iters, warmup)
-    res["stock_pytorch"] = {"images_per_s": round(E2E_BS / ms * 1e3, 1),
-                            "ms_per_step": round(ms, 2), "peak_MB": round(mb, 1)}
-    return res
+           "step": "forward + cross entropy + backward + SGD momentum update",
+           "timed_steps": iters, "warmup_steps": warmup}
+    modes = (("", E2E_MODE), ("_fused", "fused_" + E2E_MODE), ("_fused2", "fused2_" + E2E_MODE))
+    return _schedules("resnet50", E2E_BS, resnet50, (3, 224, 224), x,
+                      lambda out: torch.nn.functional.cross_entropy(out, target), modes, iters,
+                      warmup, res)
+
+
+def end_to_end_unet(iters=20, warmup=5):
+    """The reference's UNet (models/unet) with 2 output classes, batch 11, 3 x 416 x 608, fp32
+    SGD steps with softmax cross entropy over per-pixel labels, same runs as for ResNet-50."""
+    import torch
+
+    from monet_amd.models import build_model
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    _, shape, _ = build_model("unet")
+    x = torch.randn((UNET_BS,) + tuple(shape), device=dev)
+    target = torch.randint(0, 2, (UNET_BS, shape[1], shape[2]), device=dev)
+    res = {"model": "unet (2 classes)", "batch": UNET_BS, "input": list(shape), "dtype": "f32",
+           "unit": "images/s",
+           "step": "forward + per-pixel softmax cross entropy + backward + SGD momentum update",
+           "timed_steps": iters, "warmup_steps": warmup}
+    modes = (("", E2E_MODE), ("_fused", "fused_" + E2E_MODE))
+    return _schedules("unet", UNET_BS, lambda: build_model("unet")[0], tuple(shape), x,
+                      lambda out: torch.nn.functional.cross_entropy(out, target), modes, iters,
+                      warmup, res)
 
 
 def main():
@@ -302,9 +422,15 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-end-to-end", action="store_true")
-    ap.add_argument("--only", choices=["conv", "lm_ops"], default=None,
+    ap.add_argument("--only", choices=["conv", "lm_ops", "resnet50", "unet"], default=None,
                     help="run one section alone (for profiling under rocprofv3)")
+    ap.add_argument("--traffic-summary", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"), default=None,
+                    help="no GPU work: turn the output folders of the two counter runs of "
+                         "`--only lm_ops` into profiles/lm_ops_bs184_hbm_traffic.json")
     args = ap.parse_args()
+    if args.traffic_summary:
+        traffic_summary(*args.traffic_summary)
+        return
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
               file=sys.stderr)
@@ -315,6 +441,12 @@ def main():
         sys.exit(2)
     if args.only == "conv":
         print(json.dumps({"conv": conv_bench(args.steps, args.warmup)}))
+        return
+    if args.only == "resnet50":
+        print(json.dumps({"end_to_end": end_to_end()}))
+        return
+    if args.only == "unet":
+        print(json.dumps({"end_to_end_unet": end_to_end_unet()}))
         return
     ms_per_step, kernels = gpu_bench(args.steps, args.warmup, calibrate=args.only == "lm_ops")
     if args.only == "lm_ops":
@@ -340,6 +472,7 @@ def main():
     out["conv"] = conv_bench(args.steps, args.warmup)
     if not args.no_end_to_end:
         out["end_to_end"] = end_to_end()
+        out["end_to_end_unet"] = end_to_end_unet()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))

@@ -817,7 +817,11 @@ static int run(Args& A, int64_t N, int64_t C, int64_t HW, bool aligned16, void* 
     return mn_launch_status();                                           \
   } while (0)
     if (vec == 4 && chan <= 256u * 9u) MN_BN_SOLO(4, 9, 256);
-    if (vec == 4 && chan <= 1024u * 9u) MN_BN_SOLO(4, 18, 512);
+    // (a third tensor - the gate of BWD_FROM_X_GATED - does not fit beside 2 x 18 vectors per
+    // thread: that mode takes the multi-piece kernel for such channels)
+    if constexpr (MODE != BWD_FROM_X_GATED) {
+      if (vec == 4 && chan <= 1024u * 9u) MN_BN_SOLO(4, 18, 512);
+    }
     if (vec == 1 && chan <= 256u * 36u) MN_BN_SOLO(1, 36, 256);
 #undef MN_BN_SOLO
   }

@@ -565,8 +565,14 @@ __global__ __launch_bounds__(kThreads) void wgrad_kernel(const WGrad g,
   __shared__ float lds_b[2][WBK][BN + kPad];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / TL::WN, wn = wave % TL::WN;
-  const int m0 = blockIdx.y * BM;
-  const uint32_t n0 = blockIdx.x * BN;
+  // XCD-aware order: each XCD gets whole slices of the reduction, so the workgroups that read
+  // the same positions of dy and x (other row and column tiles) share one L2
+  const uint32_t slot = xcd_slot();
+  const uint32_t bz = slot / (gridDim.x * gridDim.y);
+  const uint32_t in_z = slot - bz * (gridDim.x * gridDim.y);
+  const uint32_t by = in_z / gridDim.x, bx = in_z - by * gridDim.x;
+  const int m0 = by * BM;
+  const uint32_t n0 = bx * BN;
   const uint32_t PQ = (uint32_t)g.P * g.Q;
 
   // this thread always fetches depth lane kdl and rows row0 + kStep*i of both tiles
@@ -608,10 +614,10 @@ __global__ __launch_bounds__(kThreads) void wgrad_kernel(const WGrad g,
   const char* xp = reinterpret_cast<const char*>(x);
   float ra[kRowsA], rb[kRowsB];
   float row_sum[DB ? kRowsA : 1] = {};
-  const bool sums_rows = DB && blockIdx.x == 0;
+  const bool sums_rows = DB && bx == 0;
   uint32_t a_mask = 0, b_mask = 0;
   const uint32_t total_tiles = (g.depth + WBK - 1) / WBK;
-  const uint32_t t_begin = blockIdx.z * g.tiles_per_split;
+  const uint32_t t_begin = bz * g.tiles_per_split;
   const uint32_t t_end = min(t_begin + g.tiles_per_split, total_tiles);
   DepthPos<WBK> pos(t_begin * WBK + kdl, PQ);
   // fetches the tile at the current depth position and moves on to the next one
@@ -673,11 +679,11 @@ __global__ __launch_bounds__(kThreads) void wgrad_kernel(const WGrad g,
     }
   }
   if constexpr (DB) {
-    if (sums_rows) store_row_sums<WBK, kRowsA>(row_sum, db, g, m0 + row0, kStep, kdl);
+    if (sums_rows) store_row_sums<WBK, kRowsA>(row_sum, db, g, m0 + row0, kStep, kdl, bz);
   }
 
   float* base = out;
-  if (g.mode == 2) base += (size_t)blockIdx.z * g.K * g.ncols;
+  if (g.mode == 2) base += (size_t)bz * g.K * g.ncols;
 #pragma unroll
   for (int nj = 0; nj < TL::TN; ++nj) {
     const uint32_t c = n0 + wn * (TL::TN * 32) + nj * 32 + (lane & 31);
@@ -1192,8 +1198,10 @@ static void launch_gather_t(const Gather& g, const float* a, const float* src, c
     gather_gemm_kernel<TL, true, true><<<grid, kThreads, 0, s>>>(g, a, src, bias, dst);
   else if (fast_path(g))
     gather_gemm_kernel<TL, true><<<grid, kThreads, 0, s>>>(g, a, src, bias, dst);
-  else
+  else if constexpr (TL::BN <= 128)
     gather_gemm_kernel<TL, false><<<grid, kThreads, 0, s>>>(g, a, src, bias, dst);
+  else  // the element-wise path only exists for tiles up to 128 columns: wider ones would spill
+    launch_gather_t<T64x128>(g, a, src, bias, dst, s, packed);
 }
 
 static void tile_dims(int tile, int* bm, int* bn);

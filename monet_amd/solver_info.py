@@ -29,7 +29,8 @@ import numpy as np
 from . import lm_ops
 from .graph import ComputeNode, Graph, Input, Param, fusion_level, is_batch_norm, two_step_backward
 
-MEMORY_MULTIPLIER = 4  # bytes per element: the path is fp32 (solver_info.py:10)
+MEMORY_MULTIPLIER = 4  # bytes per element of an fp32 tensor: the reference's constant
+#                        (solver_info.py:10); SolverInfo.elem_bytes holds the size in use
 
 
 class SolverNode:
@@ -100,9 +101,9 @@ class IntNode(FwdNode):
         return 'Int::%s' % self.gnode
 
 
-def _nbytes(shape, bs):
+def _nbytes(shape, bs, elem_bytes=MEMORY_MULTIPLIER):
     n = int(np.prod(shape)) if len(shape) else 1
-    n = n * MEMORY_MULTIPLIER
+    n = n * elem_bytes
     return -n * bs if n < 0 else n
 
 
@@ -118,6 +119,9 @@ class SolverInfo:
         self.graph_to_solver = {}
 
         self.bs = bs
+        # bytes per element of the activations, parameters and gradients the sizes are
+        # computed for: 4 (fp32) unless `extract` is given tensors of another floating type
+        self.elem_bytes = MEMORY_MULTIPLIER
         self.model_name = model_name
         self.mode = mode
         self.data_path = "%s_%d_%s" % (model_name, bs, mode)
@@ -137,6 +141,8 @@ class SolverInfo:
         """Build the solver graph and profile it.  `args` = (input, *parameters),
         indexed like the graph's nodes.  `cost_fn(n, op, bwd_op)` may replace the
         GPU measurement; it returns (meminfo triple, computeinfo triple)."""
+        if args and hasattr(args[0], "is_floating_point") and args[0].is_floating_point():
+            self.elem_bytes = int(args[0].element_size())   # bf16 / fp16 models: 2
         for i, n in enumerate(graph.nodes):
             if not (isinstance(n, ComputeNode) and n.has_backward):
                 continue
@@ -267,16 +273,19 @@ class SolverInfo:
         self.edge_list = [(u, v, k) for v in self.nodes
                           for k, vdeps in enumerate(self.nodes[v].args) for u in vdeps]
 
+    def _eb(self):
+        return getattr(self, "elem_bytes", MEMORY_MULTIPLIER)   # (older profile files lack it)
+
     def get_mem(self):
         for i, node in self.nodes.items():
             if isinstance(node, BwdNode):
-                node.mem = sum(_nbytes(s, self.bs) for s in node.output_shapes)
+                node.mem = sum(_nbytes(s, self.bs, self._eb()) for s in node.output_shapes)
             else:
-                node.mem = _nbytes(list(node.gnode.shape), self.bs)
+                node.mem = _nbytes(list(node.gnode.shape), self.bs, self._eb())
                 if "int::" in node.op:
                     # an intermediate's "shape" already is its size in bytes (per sample when
                     # the batch is symbolic)
-                    node.mem = int(node.mem / MEMORY_MULTIPLIER)
+                    node.mem = int(node.mem / self._eb())
 
     def get_local_memory(self):
         present = -1
@@ -298,7 +307,7 @@ class SolverInfo:
         for i in range(self.loss):
             for a in self.nodes[i].gnode.args:
                 if isinstance(a, ComputeNode.D) and isinstance(graph.nodes[a.index], (Param, Input)):
-                    fixed += _nbytes(list(graph.nodes[a.index].shape), self.bs)
+                    fixed += _nbytes(list(graph.nodes[a.index].shape), self.bs, self._eb())
         self.nodes[0].fixed_mem = fixed
         for i in self.nodes:
             if i == 0:
@@ -307,7 +316,7 @@ class SolverInfo:
             if i <= self.loss:
                 continue
             for prm in self.nodes[i].stored:  # parameter gradients accumulate through the backward
-                self.nodes[i].fixed_mem += _nbytes(list(prm.shape), self.bs)
+                self.nodes[i].fixed_mem += _nbytes(list(prm.shape), self.bs, self._eb())
 
     def get_conv_info(self):
         self.conv_list = {}

@@ -317,3 +317,25 @@ def test_batch_norm_add_relu_fusion_pass():
     ops = Counter(n.op for n in g.nodes if isinstance(n, ComputeNode))
     assert ops["monet::batch_norm_add_relu"] == 16 and ops["monet::add_relu"] == 0
     assert ops["aten::batch_norm"] == 4 and ops["monet::batch_norm_relu"] == 33
+
+
+def test_solver_sizes_follow_the_element_size_of_the_profiled_tensors():
+    """A model profiled on bf16 tensors budgets 2 bytes per element for activations,
+    parameters and gradients; compact intermediates (1 bit / 4 bits per element) stay as
+    they are (the reference fixes 4 bytes, monet/solver_info.py:10)."""
+    g = Graph.create(SmallNet(), (3, 16, 16))
+
+    def sizes(first_arg):
+        si = SolverInfo(16, "small", "multiway_newnode")
+        si.extract(g, first_arg, cost_fn=synthetic_cost(si))
+        return si
+    f32 = sizes(torch.zeros(1))
+    b16 = sizes(torch.zeros(1, dtype=torch.bfloat16))
+    assert f32.elem_bytes == 4 and b16.elem_bytes == 2
+    for i in f32.nodes:
+        a, b = f32.nodes[i], b16.nodes[i]
+        if isinstance(a, IntNode):
+            assert a.mem == b.mem and a.mem > 0
+        else:
+            assert a.mem == 2 * b.mem
+        assert a.fixed_mem == 2 * b.fixed_mem
