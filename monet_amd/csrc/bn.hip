@@ -754,13 +754,15 @@ static void fill_shape(int64_t N, int64_t C, int64_t HW, int vec, int64_t S, uin
 
 // Cache hints by plane size, from measurements at batch 184: planes of whole cache lines stream
 // fastest around the caches (56 x 56, 112 x 112); planes that share their end lines with the
-// neighbouring channel want ordinary stores, so that the parts of a line meet in L2 (28 x 28,
-// 14 x 14: 4.4 -> 5.1 TB/s), and below a few lines per plane ordinary loads as well (7 x 7:
-// 2.4 -> 5.3 TB/s).  With both plain at 14 x 14 / 28 x 28 the two streams evict each other.
+// neighbouring channel want ordinary stores, so that the parts of a line meet in L2 (14 x 14:
+// 4.4 -> 5.1 TB/s), and below a few lines per plane ordinary loads as well (7 x 7: 2.4 ->
+// 5.3 TB/s).  With both plain at 14 x 14 the two streams evict each other; from 28 x 28 up the
+// shared lines are too few to matter and ordinary stores cost the three-tensor backward of the
+// fused operators a fifth of its rate.
 static int cache_hints(int64_t HW, int forced = 0) {
   const int64_t plane = HW * (int64_t)sizeof(float);
   if (forced) return forced & (kNtLoad | kNtStore);
-  if (plane % 128 == 0) return kNtLoad | kNtStore;
+  if (plane % 128 == 0 || plane >= 2048) return kNtLoad | kNtStore;
   if (plane < 512) return 0;
   return kNtLoad;
 }

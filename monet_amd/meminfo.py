@@ -93,14 +93,24 @@ def _bytes(tensors):
     return sum(t.numel() * t.element_size() for t in tensors if t is not None)
 
 
-def _timed(fn, samples=RUNTIME_SAMPLES):
+def _timed(fn, samples=RUNTIME_SAMPLES, rounds=3):
+    """Seconds per call: one untimed call (the allocator fetches what the call needs), then
+    the smallest mean of `rounds` batches of `samples` calls.  One slow batch - another
+    process's burst, a clock ramp - would otherwise put milliseconds on one operator of the
+    profile and send the solver around it (the reference takes one mean of 20,
+    monet/meminfo.py:46-60)."""
     torch.cuda.empty_cache()
-    torch.cuda.synchronize()
-    t0 = time()
-    for _ in range(samples):
-        fn()
-    torch.cuda.synchronize()
-    return (time() - t0) / samples
+    fn()
+    best = None
+    for _ in range(rounds):
+        torch.cuda.synchronize()
+        t0 = time()
+        for _ in range(samples):
+            fn()
+        torch.cuda.synchronize()
+        dt = (time() - t0) / samples
+        best = dt if best is None else min(best, dt)
+    return best
 
 
 def _peak_over_outputs(fn):
