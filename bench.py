@@ -351,6 +351,8 @@ def _schedules(name, bs, make_model, input_shape, x, loss_fn, modes, iters, warm
             model.train()
             ms, mb = _train_ms(model, x, loss_fn, iters, warmup)
             key = ("unconstrained" if budget == 100 else "budget_%dGB" % budget) + suffix
+            print("[bench] %s %s: %.2f ms/step, peak %.0f MiB" % (name, key, ms, mb),
+                  file=sys.stderr, flush=True)
             res[key] = {"images_per_s": round(bs / ms * 1e3, 1), "ms_per_step": round(ms, 2),
                         "peak_MB": round(mb, 1)}
             if budget == 100:

@@ -420,17 +420,34 @@ def load_solution(filename):
     return si, solution
 
 
+# traced graphs by (architecture, parameter shapes, input shape, fusion level): tracing runs the
+# model once on the CPU (tens of seconds for a UNet at full resolution), and a graph holds
+# structure only, so wrappers of the same architecture share it
+_graph_cache = {}
+
+
+def _traced_graph(model, input_shape, fuse_level):
+    key = (type(model).__module__, type(model).__qualname__, repr(model),
+           tuple((k, tuple(v.shape)) for k, v in model.state_dict().items()),
+           tuple(input_shape), int(fuse_level),
+           tuple(bool(mod.training) for mod in model.modules()))
+    if key not in _graph_cache:
+        m = copy.deepcopy(model)
+        m.cpu()
+        _graph_cache[key] = Graph.create(m, input_shape, fuse_bn_relu=fuse_level)
+        del m
+    return _graph_cache[key]
+
+
 def create_schedule(model, sol_file, input_shape=(3, 224, 224)):
     """Trace `model` (on the CPU), load (solver info, solution) from `sol_file` and
     return the compiled schedule (reference: monet/schedule.py:326-346)."""
-    m = copy.deepcopy(model)
-    m.cpu()
+    m = model
     if m._get_name() == 'MobileNetV2':
         m = torch.nn.Sequential(m.features, torch.nn.AdaptiveAvgPool2d((1, 1)),
                                 torch.nn.Flatten(start_dim=1), m.classifier[0], m.classifier[1])
     solver_info, solution = load_solution(sol_file)
-    graph = Graph.create(m, input_shape, fuse_bn_relu=getattr(solver_info, "fuse_bn_relu", False))
-    del m
+    graph = _traced_graph(m, input_shape, getattr(solver_info, "fuse_bn_relu", False))
     schedule = Schedule(graph, solver_info)
     schedule.init_schedule(solution, solver_info.mode)
     return schedule

@@ -98,9 +98,15 @@ def test_schedule_matches_autograd(cuda, mode):
             y = sched.forward(x, *list(m.state_dict(keep_vars=True).values()))
             assert _rel(y, y_ref) < 1e-5
             sched.backward(gout.clone())
+            worst = 0.0
             for n, p in m.named_parameters():
                 assert p.grad is not None, n
-                assert _rel(p.grad, g_ref[n], floor) < 2e-4, (mode, name, n)
+                worst = max(worst, _rel(p.grad, g_ref[n], floor))
+            print("achieved", mode, name, "step", step, "largest gradient difference to stock fp32 "
+                  "%.2e" % worst, flush=True)
+            # two fp32 evaluations of a 10-operator network with batch statistics: summation
+            # orders differ (achieved: a few 1e-6)
+            assert worst < 5e-5, (mode, name, worst)
         # running statistics advanced exactly once per step, like the stock model's
         assert _rel(m.b1.running_mean, ref.b1.running_mean) < 1e-5
         assert _rel(m.b3.running_var, ref.b3.running_var) < 1e-5

@@ -97,8 +97,8 @@ def test_stem_block(cuda, combo):
     # ---- expected gradients: GPU decisions, float64 arithmetic
     g_a64 = torch.from_numpy(O.maxpool_bwd_idx(dy.numpy(), idx_packed, (8, 64, 112, 112), 3, 2, 1))
     y64.backward(g_a64.double() * sign.double())
-    # within 2e-5 of each tensor's scale (the 1e-5 single-operator bar, two 100k-term fp32
-    # reductions in a row)
-    assert rel(dg, g64.grad) < 2e-5 and rel(db, b64.grad) < 2e-5
-    assert rel(dw, w64.grad) < 2e-5
-    assert rel(dx, x64.grad) < 2e-5
+    # within 1e-5 of each tensor's scale (achieved: 1e-7 to 1e-6)
+    achieved = {"dgamma": rel(dg, g64.grad), "dbeta": rel(db, b64.grad), "dw": rel(dw, w64.grad),
+                "dx": rel(dx, x64.grad)}
+    print("achieved stem block (%s): " % combo + ", ".join("%s %.2e" % kv for kv in achieved.items()))
+    assert all(v < 1e-5 for v in achieved.values()), achieved
