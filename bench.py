@@ -309,8 +309,18 @@ E2E_BS = 184
 UNET_BS = 11
 
 
-def _train_ms(model, x, loss_fn, iters, warmup):
-    """ms per SGD step (forward, loss, backward, momentum update) and peak MB."""
+def _release():
+    """Drop what earlier runs left behind (wrappers and optimizers hold reference cycles)."""
+    import gc
+
+    import torch
+    gc.collect()
+    torch.cuda.empty_cache()
+
+
+def _train_ms(model, x, loss_fn, iters, warmup, foreign=0):
+    """ms per SGD step (forward, loss, backward, momentum update) and peak MB of the job
+    (`foreign` = bytes other parts of this program still hold on the device)."""
     import torch
     opt = torch.optim.SGD(model.parameters(), lr=0.01, momentum=0.9)
 
@@ -329,7 +339,7 @@ def _train_ms(model, x, loss_fn, iters, warmup):
         step()
     t1.record()
     torch.cuda.synchronize()
-    return t0.elapsed_time(t1) / iters, torch.cuda.max_memory_allocated() / 2**20
+    return t0.elapsed_time(t1) / iters, (torch.cuda.max_memory_allocated() - foreign) / 2**20
 
 
 def _schedules(name, bs, make_model, input_shape, x, loss_fn, modes, iters, warmup, res):
@@ -341,6 +351,9 @@ def _schedules(name, bs, make_model, input_shape, x, loss_fn, modes, iters, warm
 
     from monet_amd.monet_wrapper import MONeTWrapper
     dev = x.device
+    _release()
+    # what the device holds that is not this job's batch (and labels): nothing, normally
+    foreign = max(0, torch.cuda.memory_allocated() - x.numel() * x.element_size() - (64 << 20))
     for suffix, mode in modes:
         base = None
         for budget in (100, 10, 6):
@@ -349,7 +362,7 @@ def _schedules(name, bs, make_model, input_shape, x, loss_fn, modes, iters, warm
                 continue
             model = MONeTWrapper(make_model(), str(sol), input_shape).to(dev)
             model.train()
-            ms, mb = _train_ms(model, x, loss_fn, iters, warmup)
+            ms, mb = _train_ms(model, x, loss_fn, iters, warmup, foreign)
             key = ("unconstrained" if budget == 100 else "budget_%dGB" % budget) + suffix
             print("[bench] %s %s: %.2f ms/step, peak %.0f MiB" % (name, key, ms, mb),
                   file=sys.stderr, flush=True)
@@ -362,13 +375,13 @@ def _schedules(name, bs, make_model, input_shape, x, loss_fn, modes, iters, warm
                 if base:
                     res[key]["overhead_vs_unconstrained"] = round(ms / base - 1.0, 4)
             del model
-            torch.cuda.empty_cache()
+            _release()
     model = make_model().to(dev).train()
-    ms, mb = _train_ms(model, x, loss_fn, iters, warmup)
+    ms, mb = _train_ms(model, x, loss_fn, iters, warmup, foreign)
     res["stock_pytorch"] = {"images_per_s": round(bs / ms * 1e3, 1), "ms_per_step": round(ms, 2),
                             "peak_MB": round(mb, 1)}
     del model
-    torch.cuda.empty_cache()
+    _release()
     return res
 
 
