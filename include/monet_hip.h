@@ -335,7 +335,12 @@ typedef struct mn_conv2d {
  *                      rotated by 180 degrees, channel roles swapped)
  *   backward-weight  0 split reduction combined with atomics into a cleared dw
  *                    1 split reduction through per-split partials in the
- *                      workspace, then a fixed-order sum (reproducible) */
+ *                      workspace, then a fixed-order sum (reproducible)
+ *                    2 Winograd (the transposed form of F(2x2, 3x3): the 16
+ *                      transform-domain products reduced over the 2x2 output
+ *                      tiles): 3x3, stride 1, dilation 1, C a multiple of 4,
+ *                      fp32; workspace of 16 floats per tile and channel for
+ *                      dy and x plus the partial results; reproducible */
 int mn_conv_n_variants(int direction);
 /* The same per dtype: the list above for MN_F32; 1 for MN_BF16 (one kernel and
  * one memory tier per direction - index 1 is accepted as an alias of 0 so that

@@ -29,6 +29,9 @@ int mn_wino_fwd(const mn_conv2d* g, const float* x, const float* w, const float*
                 void* ws, size_t ws_bytes, hipStream_t s);
 int mn_wino_bwd_data(const mn_conv2d* g, const float* dy, const float* w, float* dx, bool accum,
                      void* ws, size_t ws_bytes, hipStream_t s);
+int mn_wino_bwd_weight_ws_bytes(const mn_conv2d* g, size_t* bytes);
+int mn_wino_bwd_weight(const mn_conv2d* g, const float* dy, const float* x, float* dw, float* db,
+                       void* ws, size_t ws_bytes, hipStream_t s);
 
 // bf16 / channels-last kernels (conv_bf16.hip)
 int mn_conv16_ws_bytes(const mn_conv2d* g, int direction, size_t* bytes);
@@ -1371,7 +1374,7 @@ int mn_conv_n_variants(int direction) {
     case MN_CONV_BWD_DATA:
       return 3;
     case MN_CONV_BWD_WEIGHT:
-      return 2;
+      return 3;
     default:
       return 0;
   }
@@ -1394,7 +1397,9 @@ int mn_conv_ws_bytes(const mn_conv2d* g, int direction, int variant, int dtype, 
   if (dtype == MN_BF16)  // variants 0 and 1 are one kernel; there is no bf16 Winograd tier
     return variant <= 1 ? mn_conv16_ws_bytes(g, direction, bytes) : MN_EUNSUPPORTED;
   if (dtype != MN_F32) return MN_EUNSUPPORTED;
-  if (variant == 2) return mn_wino_ws_bytes(g, direction == MN_CONV_BWD_DATA, bytes);
+  if (variant == 2)
+    return direction == MN_CONV_BWD_WEIGHT ? mn_wino_bwd_weight_ws_bytes(g, bytes)
+                                           : mn_wino_ws_bytes(g, direction == MN_CONV_BWD_DATA, bytes);
   const size_t wsize = (size_t)g->K * g->C * g->R * g->S * sizeof(float);
   // variant 1 of the gather directions: the repacked weight operand (rows padded to 128)
   if (direction == MN_CONV_FWD && variant == 1)
@@ -1583,9 +1588,15 @@ static int conv_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, vo
   const int st = check(g);
   if (st != MN_OK) return st;
   if (dtype != MN_F32 && dtype != MN_BF16) return MN_EUNSUPPORTED;
-  if (variant < 0 || variant > 1) return MN_EUNSUPPORTED;
+  if (variant < 0 || variant > 2 || (variant == 2 && dtype != MN_F32)) return MN_EUNSUPPORTED;
   if (!dw) return MN_EINVAL;
   hipStream_t s = mn_stream(stream);
+  if (variant == 2) {
+    if (g->N == 0) return MN_EUNSUPPORTED;  // nothing to reduce: variants 0 and 1 clear dw
+    if (!dy || !x) return MN_EINVAL;
+    return mn_wino_bwd_weight(g, (const float*)dy, (const float*)x, (float*)dw, (float*)db_out, ws,
+                              ws_bytes, s);
+  }
   if (dtype == MN_BF16) {
     if (db_out) return MN_EUNSUPPORTED;     // the bf16 kernel has no bias-gradient epilogue
     if (g->N == 0) return MN_EUNSUPPORTED;  // nothing to reduce: the caller clears dw itself

@@ -177,6 +177,220 @@ __global__ __launch_bounds__(kThreads) void output_kernel(const Plan p, const fl
   }
 }
 
+// ------------------------------------------------------------ backward weight --
+// dW (3x3) = sum over tiles of G^T [ (A dY A^T) .* (B^T X B) ] G, with dY the 2x2 tile of the
+// output gradient and X the 4x4 input tile the forward used for it (the transposed form of the
+// forward algorithm).  Per transform-domain position that is a matrix product over the TILES,
+//   Z[pos][k][c] = sum over t of Ud[pos][t][k] * Vx[pos][t][c],
+// 16 multiplies per tile and (k, c) pair instead of 36.  The reduction is long (all tiles) and
+// the result small (K x C), so it is cut into S slices that run as 16 * S independent GEMMs
+// of the same batched launch the forward uses; their partial results are added in a fixed order
+// by the kernel that applies G^T . G (reproducible run to run).
+//
+// Both transforms write [pos][tile][channel], channel fastest, which is the reduction-major
+// layout the GEMM wants; the tensors have the pixel fastest, so a workgroup transposes a block
+// of 32 tiles x 32 channels through LDS (8 positions at a time).
+template <bool DY>
+__global__ __launch_bounds__(kThreads) void wgrad_transform_kernel(const Plan p, int channels,
+                                                                   const float* __restrict__ src,
+                                                                   float* __restrict__ out,
+                                                                   int row_len, uint32_t Tpad) {
+  __shared__ float lds[8][32][33];
+  const int lane_t = threadIdx.x & 31, cg = threadIdx.x >> 5;
+  const uint32_t t0 = blockIdx.x * 32u;
+  const int c0 = blockIdx.y * 32;
+  const uint32_t tile = t0 + lane_t;
+  const bool t_ok = tile < p.T;
+  const uint32_t per_img = (uint32_t)p.TH * p.TW;
+  const uint32_t n = t_ok ? tile / per_img : 0u, r = t_ok ? tile - n * per_img : 0u;
+  const int th = r / p.TW, tw = r - th * p.TW;
+  float v[4][16];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int ch = c0 + cg + 8 * i;
+    const bool ok = t_ok && ch < channels;
+    if (DY) {
+      // 2x2 tile of dy [N, channels, OH, OW] at (2 th, 2 tw), zero beyond the edge
+      float d[2][2];
+      const float* plane = src + ((size_t)n * channels + (ok ? ch : 0)) * p.OH * p.OW;
+#pragma unroll
+      for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+          const int h = 2 * th + a, w = 2 * tw + b;
+          d[a][b] = (ok && h < p.OH && w < p.OW) ? plane[(size_t)h * p.OW + w] : 0.f;
+        }
+      // A d A^T, A = [1 0; 1 1; 1 -1; 0 -1]
+      float t[4][2];
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        t[0][b] = d[0][b];
+        t[1][b] = d[0][b] + d[1][b];
+        t[2][b] = d[0][b] - d[1][b];
+        t[3][b] = -d[1][b];
+      }
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        v[i][4 * a + 0] = t[a][0];
+        v[i][4 * a + 1] = t[a][0] + t[a][1];
+        v[i][4 * a + 2] = t[a][0] - t[a][1];
+        v[i][4 * a + 3] = -t[a][1];
+      }
+    } else {
+      // 4x4 tile of x [N, channels, Hs, Ws] at (2 th - pad, 2 tw - pad), zero outside the image
+      float d[4][4];
+      const float* plane = src + ((size_t)n * channels + (ok ? ch : 0)) * p.Hs * p.Ws;
+      const int h0 = 2 * th - p.pad, w0 = 2 * tw - p.pad;
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        const int h = h0 + a;
+        const bool hok = ok && (unsigned)h < (unsigned)p.Hs;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          const int w = w0 + b;
+          d[a][b] = (hok && (unsigned)w < (unsigned)p.Ws) ? plane[(size_t)h * p.Ws + w] : 0.f;
+        }
+      }
+      float t[4][4];  // B^T d
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        t[0][b] = d[0][b] - d[2][b];
+        t[1][b] = d[1][b] + d[2][b];
+        t[2][b] = d[2][b] - d[1][b];
+        t[3][b] = d[1][b] - d[3][b];
+      }
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {  // (B^T d) B
+        v[i][4 * a + 0] = t[a][0] - t[a][2];
+        v[i][4 * a + 1] = t[a][1] + t[a][2];
+        v[i][4 * a + 2] = t[a][2] - t[a][1];
+        v[i][4 * a + 3] = t[a][1] - t[a][3];
+      }
+    }
+  }
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int pp = 0; pp < 8; ++pp) lds[pp][lane_t][cg + 8 * i] = v[i][8 * half + pp];
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < 8 * 32 * 32; idx += kThreads) {
+      const int pp = idx >> 10, rem = idx & 1023, tl = rem >> 5, ch = rem & 31;
+      if (c0 + ch < row_len && t0 + tl < Tpad)
+        out[((size_t)(8 * half + pp) * Tpad + t0 + tl) * row_len + c0 + ch] = lds[pp][tl][ch];
+    }
+    __syncthreads();
+  }
+}
+
+// dw[k][c] (3x3) = G^T (sum over the S slices of Z[pos][s][k][c]) G; G^T = [1 .5 .5 0; 0 .5 -.5 0; 0 .5 .5 1].
+// A workgroup takes 64 consecutive (k, c) pairs: each wavefront adds up the slices of four
+// positions for them (64 lanes = 64 consecutive floats per load), the sums meet in LDS and the
+// first wavefront applies G^T . G and writes the nine taps.
+__global__ __launch_bounds__(kThreads) void wgrad_output_kernel(const float* __restrict__ Z,
+                                                                float* __restrict__ dw, int K, int C,
+                                                                int S) {
+  __shared__ float lds[16][64];
+  const size_t kc = (size_t)K * C;
+  const int lane = threadIdx.x & 63, pg = threadIdx.x >> 6;
+  const size_t i = (size_t)blockIdx.x * 64 + lane;
+  const bool ok = i < kc;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int pos = 4 * pg + q;
+    const float* base = Z + (size_t)pos * S * kc + (ok ? i : 0);
+    float acc = 0.f;
+    int s = 0;
+    for (; s + 4 <= S; s += 4) {  // four loads in flight, added in slice order
+      const float a0 = base[(size_t)s * kc], a1 = base[(size_t)(s + 1) * kc];
+      const float a2 = base[(size_t)(s + 2) * kc], a3 = base[(size_t)(s + 3) * kc];
+      acc = (((acc + a0) + a1) + a2) + a3;
+    }
+    for (; s < S; ++s) acc += base[(size_t)s * kc];
+    lds[pos][lane] = acc;
+  }
+  __syncthreads();
+  if (pg != 0 || !ok) return;
+  float z[4][4];
+#pragma unroll
+  for (int pos = 0; pos < 16; ++pos) z[pos >> 2][pos & 3] = lds[pos][lane];
+  float t[3][4];
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    t[0][b] = z[0][b] + 0.5f * (z[1][b] + z[2][b]);
+    t[1][b] = 0.5f * (z[1][b] - z[2][b]);
+    t[2][b] = 0.5f * (z[1][b] + z[2][b]) + z[3][b];
+  }
+  float* o = dw + i * 9;
+#pragma unroll
+  for (int a = 0; a < 3; ++a) {
+    o[3 * a + 0] = t[a][0] + 0.5f * (t[a][1] + t[a][2]);
+    o[3 * a + 1] = 0.5f * (t[a][1] - t[a][2]);
+    o[3 * a + 2] = 0.5f * (t[a][1] + t[a][2]) + t[a][3];
+  }
+}
+
+// db[k] = sum over (n, p, q) of dy[n][k][p][q], one workgroup per k, fixed order.
+__global__ __launch_bounds__(kThreads) void bias_grad_kernel(const float* __restrict__ dy,
+                                                             float* __restrict__ db, int N, int K,
+                                                             int PQ) {
+  __shared__ float lds[2 * (kThreads / 64)];
+  const int k = blockIdx.x;
+  float s = 0.f, unused = 0.f;
+  for (int n = 0; n < N; ++n) {
+    const float* plane = dy + ((size_t)n * K + k) * PQ;
+    for (int i = threadIdx.x; i < PQ; i += kThreads) s += plane[i];
+  }
+  block_sum2<kThreads / 64>(s, unused, lds);
+  if (threadIdx.x == 0) db[k] = s;
+}
+
+struct WPlan {
+  Plan p;          // tiles over the OUTPUT of the forward (dy), source = x
+  int K, C, S;     // S slices of the reduction over tiles
+  uint32_t Tc, Tpad;
+  int Kp;
+};
+static size_t wu_floats(const WPlan& w) { return (size_t)16 * w.Tpad * w.Kp; }
+static size_t wv_floats(const WPlan& w) { return (size_t)16 * w.Tpad * w.C; }
+static size_t wz_floats(const WPlan& w) { return (size_t)16 * w.S * w.K * w.C; }
+
+static bool make_wplan(const mn_conv2d* g, WPlan& w) {
+  Plan& p = w.p;
+  p.N = g->N;
+  p.Cs = g->C;
+  p.Hs = g->H;
+  p.Ws = g->W;
+  p.M = g->K;
+  p.OH = g->P;
+  p.OW = g->Q;
+  p.pad = g->pH;
+  p.TH = (g->P + 1) / 2;
+  p.TW = (g->Q + 1) / 2;
+  const unsigned long long T = (unsigned long long)g->N * p.TH * p.TW;
+  if (T == 0 || T >= (1ull << 28) || g->C % 4 != 0) return false;
+  p.T = (uint32_t)T;
+  p.Tp = p.T;
+  p.Mp = 0;
+  w.K = g->K;
+  w.C = g->C;
+  w.Kp = (g->K + 127) / 128 * 128;
+  // enough independent GEMMs for ~8 workgroups per CU, at least 64 tiles per slice
+  const long long per_batch = (long long)((g->C + 63) / 64) * ((g->K + 127) / 128);
+  long long S = (2048 + 16 * per_batch - 1) / (16 * per_batch);
+  if (S > (long long)(T / 64)) S = (long long)(T / 64);
+  if (S > 64) S = 64;
+  if (S < 1) S = 1;
+  w.S = (int)S;
+  w.Tc = (uint32_t)(((T + S - 1) / S + 31) / 32 * 32);
+  w.Tpad = w.Tc * (uint32_t)S;
+  if ((unsigned long long)w.Tc * w.Kp >= (1ull << 29) || (unsigned long long)w.Tc * w.C >= (1ull << 29) ||
+      (unsigned long long)16 * w.Tpad * w.Kp >= (1ull << 36))
+    return false;
+  return true;
+}
+
 static bool make_plan(int N, int Cs, int Hs, int Ws, int M, int OH, int OW, int pad, Plan& p) {
   p.N = N;
   p.Cs = Cs;
@@ -262,4 +476,35 @@ int mn_wino_bwd_data(const mn_conv2d* g, const float* dy, const float* w, float*
   if (!shape_ok(g) || !make_plan(g->N, g->K, g->P, g->Q, g->C, g->H, g->W, 2 - g->pH, p))
     return MN_EUNSUPPORTED;
   return run(p, dy, w, true, nullptr, dx, accum, ws, ws_bytes, s);
+}
+
+// Weight gradient (fp32) through the Winograd form above; db (optional): the bias gradient.
+int mn_wino_bwd_weight_ws_bytes(const mn_conv2d* g, size_t* bytes) {
+  using namespace mn_wino;
+  *bytes = 0;
+  WPlan w;
+  if (!shape_ok(g) || !make_wplan(g, w)) return MN_EUNSUPPORTED;
+  *bytes = (wu_floats(w) + wv_floats(w) + wz_floats(w)) * sizeof(float);
+  return MN_OK;
+}
+
+int mn_wino_bwd_weight(const mn_conv2d* g, const float* dy, const float* x, float* dw, float* db,
+                       void* ws, size_t ws_bytes, hipStream_t s) {
+  using namespace mn_wino;
+  WPlan w;
+  if (!shape_ok(g) || !make_wplan(g, w)) return MN_EUNSUPPORTED;
+  const size_t need = (wu_floats(w) + wv_floats(w) + wz_floats(w)) * sizeof(float);
+  if (!ws || ws_bytes < need || !mn_aligned(ws, 16)) return MN_EINVAL;
+  float* U = static_cast<float*>(ws);
+  float* V = U + wu_floats(w);
+  float* Z = V + wv_floats(w);
+  const dim3 gu(w.Tpad / 32, w.Kp / 32), gv(w.Tpad / 32, (w.C + 31) / 32);
+  wgrad_transform_kernel<true><<<gu, kThreads, 0, s>>>(w.p, w.K, dy, U, w.Kp, w.Tpad);
+  wgrad_transform_kernel<false><<<gv, kThreads, 0, s>>>(w.p, w.C, x, V, w.C, w.Tpad);
+  const int st = mn_conv_batched_gemm(U, V, Z, w.K, w.Kp, (int)w.Tc, (uint32_t)w.C, 16 * w.S, s);
+  if (st != MN_OK) return st;
+  const uint32_t n = (uint32_t)w.K * w.C;
+  wgrad_output_kernel<<<(n + 63) / 64, kThreads, 0, s>>>(Z, dw, w.K, w.C, w.S);
+  if (db) bias_grad_kernel<<<w.K, kThreads, 0, s>>>(dy, db, g->N, g->K, g->P * g->Q);
+  return mn_launch_status();
 }

@@ -52,6 +52,11 @@ def winograd_applies(ws, st, pad, dil, reduced_channels):
             pair(pad)[0] == pair(pad)[1] and pair(pad)[0] <= 2 and reduced_channels % 16 == 0)
 
 
+def winograd_wgrad_applies(xs, ws, st, pad, dil):
+    """Variant 2 of backward-weight: 3x3, stride 1, dilation 1, equal padding <= 2, C % 4 == 0."""
+    return winograd_applies(ws, st, pad, dil, 16) and xs[1] % 4 == 0
+
+
 def refused(call):
     from monet_amd import _lib
     with pytest.raises(_lib.MonetHipError) as e:
@@ -127,10 +132,18 @@ def test_conv_backward_weight(cuda, xs, ws, st, pad, dil):
     dy = np.random.default_rng(4).standard_normal(yshape).astype(np.float32)
     exp = O.conv_bwd_weight(dy, x, ws, st, pad, dil)
     outs = []
+    assert conv_ops.n_bwd_wt_algos() == 3
     for v in range(conv_ops.n_bwd_wt_algos()):
+        if v == 2 and not winograd_wgrad_applies(xs, ws, st, pad, dil):
+            assert refused(lambda: conv_ops.conv_backward_weight(ws, dev(dy, cuda), dev(x, cuda),
+                                                                 pad, st, dil, 1, v))
+            continue
         dw = conv_ops.conv_backward_weight(ws, dev(dy, cuda), dev(x, cuda), pad, st, dil, 1, v)
         assert_rel(host(dw), exp, TOL, f"backward-weight variant {v}")
         outs.append(dw)
+        if v == 2:   # partial results added in a fixed order: bit-identical run to run
+            assert torch.equal(dw, conv_ops.conv_backward_weight(ws, dev(dy, cuda), dev(x, cuda), pad,
+                                                                 st, dil, 1, v))
     # the workspace variant sums its partials in a fixed order: bit-identical run to run
     again = conv_ops.conv_backward_weight(ws, dev(dy, cuda), dev(x, cuda), pad, st, dil, 1, 1)
     assert torch.equal(again, outs[1])
@@ -336,6 +349,8 @@ def test_conv_backward_weight_with_bias_gradient(cuda, xs, ws, st, pad, dil):
     # the largest of K sums
     scale_db = np.sqrt(dy.size / ws[0])
     for v in range(conv_ops.n_bwd_wt_algos()):
+        if v == 2 and not winograd_wgrad_applies(xs, ws, st, pad, dil):
+            continue
         alone = conv_ops.conv_backward_weight(ws, dev(dy, cuda), dev(x, cuda), pad, st, dil, 1, v)
         dw, db = conv_ops.conv_backward_weight(ws, dev(dy, cuda), dev(x, cuda), pad, st, dil, 1, v,
                                                with_bias_grad=True)
@@ -343,7 +358,7 @@ def test_conv_backward_weight_with_bias_gradient(cuda, xs, ws, st, pad, dil):
         assert list(db.shape) == [ws[0]]
         err = np.abs(host(db).astype(np.float64) - exp_db).max()
         assert err <= TOL * scale_db, f"db variant {v}: {err:.3e} vs {scale_db:.3e}"
-        if v == 1:
+        if v >= 1:
             assert torch.equal(dw, alone)
             dw2, db2 = conv_ops.conv_backward_weight(ws, dev(dy, cuda), dev(x, cuda), pad, st, dil,
                                                      1, v, with_bias_grad=True)
