@@ -275,10 +275,15 @@ __global__ __launch_bounds__(kThreads) void wgrad_transform_kernel(const Plan p,
 #pragma unroll
       for (int pp = 0; pp < 8; ++pp) lds[pp][lane_t][cg + 8 * i] = v[i][8 * half + pp];
     __syncthreads();
-    for (int idx = threadIdx.x; idx < 8 * 32 * 32; idx += kThreads) {
-      const int pp = idx >> 10, rem = idx & 1023, tl = rem >> 5, ch = rem & 31;
-      if (c0 + ch < row_len && t0 + tl < Tpad)
-        out[((size_t)(8 * half + pp) * Tpad + t0 + tl) * row_len + c0 + ch] = lds[pp][tl][ch];
+    // rows of 32 channels leave as eight 16-byte stores (row_len is a multiple of 4)
+    for (int idx = threadIdx.x; idx < 8 * 32 * 8; idx += kThreads) {
+      const int pp = idx >> 8, rem = idx & 255, tl = rem >> 3, ch = (rem & 7) * 4;
+      if (c0 + ch < row_len && t0 + tl < Tpad) {
+        const float4_t q = {lds[pp][tl][ch], lds[pp][tl][ch + 1], lds[pp][tl][ch + 2],
+                            lds[pp][tl][ch + 3]};
+        st_stream(reinterpret_cast<float4_t*>(
+                      out + ((size_t)(8 * half + pp) * Tpad + t0 + tl) * row_len + c0 + ch), q);
+      }
     }
     __syncthreads();
   }
