@@ -49,3 +49,14 @@ class MONeTWrapper(torch.nn.Module):
         x.requires_grad_(True)
         state = self.state_dict(keep_vars=True)
         return MONeTWrapperF.apply(x, self.schedule[0], list(state.values()))
+
+
+def reserve_pool(expected_bytes, device=None):
+    """Make the caching allocator hold one block of `expected_bytes` before training starts
+    and hand it back to the allocator's free list, so that the schedule's tensors are carved
+    out of that block instead of out of many smaller segments (the step the reference's
+    README.md:60-65 asks its users to do by hand with `torch.zeros(expected_memory / 4)`).
+    The block is left uninitialised: only the reservation matters."""
+    pool = torch.empty(int(expected_bytes), dtype=torch.uint8,
+                       device=device if device is not None else torch.device("cuda"))
+    del pool

@@ -199,3 +199,16 @@ def test_bottleneck_resnet_against_float64(cuda):
     print("largest relative error against float64: schedule %.3e, stock fp32 %.3e" % (
         worst_ours, worst_stock), flush=True)
     assert worst_ours <= 4 * worst_stock + 1e-5
+
+
+def test_reserve_pool_leaves_one_cached_block(cuda):
+    """`reserve_pool` (the reference's README.md:60-65 advice as a function): afterwards the
+    allocator holds at least the requested bytes in its free list and nothing is allocated."""
+    from monet_amd.monet_wrapper import reserve_pool
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    before = torch.cuda.memory_allocated()
+    reserve_pool(256 << 20, cuda)
+    assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.memory_reserved() - before >= 256 << 20
+    torch.cuda.empty_cache()
