@@ -323,8 +323,10 @@ typedef struct mn_conv2d {
  *                      (MN_EUNSUPPORTED otherwise, and for MN_BF16): 2.25 times
  *                      fewer multiplications, paid for with a workspace of 16
  *                      floats per 2x2 output tile and channel, input and output
- *                      side (the role of the reference's WINOGRAD_NONFUSED
- *                      slot, monet/lm_ops/conv.cpp:21-27, :314-324)
+ *                      side, capped at 512 MB: a larger problem runs in slices
+ *                      of tiles through the same buffers (the role of the
+ *                      reference's WINOGRAD_NONFUSED slot,
+ *                      monet/lm_ops/conv.cpp:21-27, :314-324)
  *   backward-data    0 implicit GEMM reading the weights through strides
  *                    1 same with the weights repacked [tap][k][c] (c padded
  *                      to a multiple of 128) into the workspace; may split
@@ -340,7 +342,9 @@ typedef struct mn_conv2d {
  *                      transform-domain products reduced over the 2x2 output
  *                      tiles): 3x3, stride 1, dilation 1, C a multiple of 4,
  *                      fp32; workspace of 16 floats per tile and channel for
- *                      dy and x plus the partial results; reproducible */
+ *                      dy and x (capped at 512 MB: more tiles are taken in
+ *                      passes added in order) plus the partial results;
+ *                      reproducible */
 int mn_conv_n_variants(int direction);
 /* The same per dtype: the list above for MN_F32; 1 for MN_BF16 (one kernel and
  * one memory tier per direction - index 1 is accepted as an alias of 0 so that

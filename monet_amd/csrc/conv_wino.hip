@@ -23,13 +23,16 @@ int mn_conv_batched_gemm(const float* a, const float* src, float* dst, int M, in
 namespace mn_wino {
 
 constexpr int kThreads = 256;
+constexpr unsigned long long kSliceBytes = 512ull << 20;  // cap of the transformed source + product buffers
 
 struct Plan {
   int N, Cs, Hs, Ws;   // source tensor [N, Cs, Hs, Ws]
   int M, OH, OW;       // destination tensor [N, M, OH, OW]
   int pad;             // source coordinate of tile element (i, j) = (2*th - pad + i, 2*tw - pad + j)
   int TH, TW;          // tiles per image
-  uint32_t T, Tp;      // tiles, and tiles rounded up to a multiple of 4 (row length of V and Mt)
+  uint32_t T, Tp;      // tiles; row capacity of V and Mt (tiles of the largest slice, multiple of 4)
+  uint32_t slice;      // tiles per slice: the transforms and the GEMM run slice after slice
+  uint32_t t0, Ts, Tsp;  // the current slice: first tile, tiles, row length (multiple of 4)
   int Mp;              // rows of U padded to a multiple of 128
 };
 
@@ -87,11 +90,12 @@ __global__ __launch_bounds__(kThreads) void weight_kernel(const float* __restric
 __global__ __launch_bounds__(kThreads) void input_kernel(const Plan p, const float* __restrict__ src,
                                                          float* __restrict__ V) {
   const uint32_t i = blockIdx.x * kThreads + threadIdx.x;
-  const uint32_t row = i / p.Tp, tile = i - row * p.Tp;  // row = ch
+  const uint32_t row = i / p.Tsp, col = i - row * p.Tsp;  // row = ch
   if (row >= (uint32_t)p.Cs) return;
-  const size_t stride = (size_t)p.Cs * p.Tp;
+  const uint32_t tile = p.t0 + col;
+  const size_t stride = (size_t)p.Cs * p.Tsp;
   float d[4][4];
-  if (tile < p.T) {
+  if (col < p.Ts) {
     const uint32_t per_img = (uint32_t)p.TH * p.TW;
     const uint32_t n = tile / per_img, r = tile - n * per_img;
     const int th = r / p.TW, tw = r - th * p.TW;
@@ -137,9 +141,10 @@ __global__ __launch_bounds__(kThreads) void output_kernel(const Plan p, const fl
                                                           const float* __restrict__ bias,
                                                           float* __restrict__ dst) {
   const uint32_t i = blockIdx.x * kThreads + threadIdx.x;
-  const uint32_t row = i / p.Tp, tile = i - row * p.Tp;
-  if (row >= (uint32_t)p.M || tile >= p.T) return;
-  const size_t stride = (size_t)p.M * p.Tp;
+  const uint32_t row = i / p.Tsp, col = i - row * p.Tsp;
+  if (row >= (uint32_t)p.M || col >= p.Ts) return;
+  const uint32_t tile = p.t0 + col;
+  const size_t stride = (size_t)p.M * p.Tsp;
   float m[4][4];
 #pragma unroll
   for (int a = 0; a < 4; ++a)
@@ -199,7 +204,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_transform_kernel(const Plan p,
   const int lane_t = threadIdx.x & 31, cg = threadIdx.x >> 5;
   const uint32_t t0 = blockIdx.x * 32u;
   const int c0 = blockIdx.y * 32;
-  const uint32_t tile = t0 + lane_t;
+  const uint32_t tile = p.t0 + t0 + lane_t;  // p.t0: first tile of this pass
   const bool t_ok = tile < p.T;
   const uint32_t per_img = (uint32_t)p.TH * p.TW;
   const uint32_t n = t_ok ? tile / per_img : 0u, r = t_ok ? tile - n * per_img : 0u;
@@ -293,6 +298,8 @@ __global__ __launch_bounds__(kThreads) void wgrad_transform_kernel(const Plan p,
 // A workgroup takes 64 consecutive (k, c) pairs: each wavefront adds up the slices of four
 // positions for them (64 lanes = 64 consecutive floats per load), the sums meet in LDS and the
 // first wavefront applies G^T . G and writes the nine taps.
+// ACCUM: dw += (a later pass over the tiles; the passes run in order, so the sum is reproducible).
+template <bool ACCUM>
 __global__ __launch_bounds__(kThreads) void wgrad_output_kernel(const float* __restrict__ Z,
                                                                 float* __restrict__ dw, int K, int C,
                                                                 int S) {
@@ -330,9 +337,12 @@ __global__ __launch_bounds__(kThreads) void wgrad_output_kernel(const float* __r
   float* o = dw + i * 9;
 #pragma unroll
   for (int a = 0; a < 3; ++a) {
-    o[3 * a + 0] = t[a][0] + 0.5f * (t[a][1] + t[a][2]);
-    o[3 * a + 1] = 0.5f * (t[a][1] - t[a][2]);
-    o[3 * a + 2] = 0.5f * (t[a][1] + t[a][2]) + t[a][3];
+    const float r0 = t[a][0] + 0.5f * (t[a][1] + t[a][2]);
+    const float r1 = 0.5f * (t[a][1] - t[a][2]);
+    const float r2 = 0.5f * (t[a][1] + t[a][2]) + t[a][3];
+    o[3 * a + 0] = ACCUM ? o[3 * a + 0] + r0 : r0;
+    o[3 * a + 1] = ACCUM ? o[3 * a + 1] + r1 : r1;
+    o[3 * a + 2] = ACCUM ? o[3 * a + 2] + r2 : r2;
   }
 }
 
@@ -353,8 +363,9 @@ __global__ __launch_bounds__(kThreads) void bias_grad_kernel(const float* __rest
 
 struct WPlan {
   Plan p;          // tiles over the OUTPUT of the forward (dy), source = x
-  int K, C, S;     // S slices of the reduction over tiles
-  uint32_t Tc, Tpad;
+  int K, C, S;     // S slices of the reduction over the tiles of one pass
+  uint32_t Tc, Tpad;  // tiles per slice, tiles per pass (= S * Tc)
+  uint32_t passes;    // the tiles are taken Tpad at a time so that the transforms fit kSliceBytes
   int Kp;
 };
 static size_t wu_floats(const WPlan& w) { return (size_t)16 * w.Tpad * w.Kp; }
@@ -381,15 +392,25 @@ static bool make_wplan(const mn_conv2d* g, WPlan& w) {
   w.K = g->K;
   w.C = g->C;
   w.Kp = (g->K + 127) / 128 * 128;
+  // tiles per pass: both transforms together under kSliceBytes
+  const unsigned long long per_tile = 64ull * ((unsigned long long)w.Kp + g->C);
+  unsigned long long Tpass = T;
+  if (per_tile * T > kSliceBytes) {
+    Tpass = kSliceBytes / per_tile / 2048 * 2048;
+    if (Tpass < 2048) Tpass = 2048;
+    if (Tpass > T) Tpass = T;
+  }
   // enough independent GEMMs for ~8 workgroups per CU, at least 64 tiles per slice
   const long long per_batch = (long long)((g->C + 63) / 64) * ((g->K + 127) / 128);
   long long S = (2048 + 16 * per_batch - 1) / (16 * per_batch);
-  if (S > (long long)(T / 64)) S = (long long)(T / 64);
+  if (S > (long long)(Tpass / 64)) S = (long long)(Tpass / 64);
   if (S > 64) S = 64;
   if (S < 1) S = 1;
   w.S = (int)S;
-  w.Tc = (uint32_t)(((T + S - 1) / S + 31) / 32 * 32);
+  w.Tc = (uint32_t)(((Tpass + S - 1) / S + 31) / 32 * 32);
   w.Tpad = w.Tc * (uint32_t)S;
+  w.passes = (uint32_t)((T + w.Tpad - 1) / w.Tpad);
+  p.t0 = 0;
   if ((unsigned long long)w.Tc * w.Kp >= (1ull << 29) || (unsigned long long)w.Tc * w.C >= (1ull << 29) ||
       (unsigned long long)16 * w.Tpad * w.Kp >= (1ull << 36))
     return false;
@@ -410,8 +431,21 @@ static bool make_plan(int N, int Cs, int Hs, int Ws, int M, int OH, int OW, int 
   const unsigned long long T = (unsigned long long)N * p.TH * p.TW;
   if (T == 0 || T >= (1ull << 28)) return false;
   p.T = (uint32_t)T;
-  p.Tp = (p.T + 3u) & ~3u;
   p.Mp = (M + 127) / 128 * 128;
+  // V and Mt together stay under kSliceBytes: larger problems run slice after slice through the
+  // same two buffers (measured at 512 MB: within 1 % of the unsliced time from 256 channels up,
+  // where this variant is the fastest; 192 MB costs 4-10 %, 48 MB 25-35 %)
+  p.slice = p.T;
+  const unsigned long long per_tile = 64ull * ((unsigned long long)Cs + M);
+  if (per_tile * p.T > kSliceBytes) {
+    const unsigned long long t = kSliceBytes / per_tile / 256 * 256;
+    p.slice = (uint32_t)(t < 256 ? 256 : t);
+    if (p.slice > p.T) p.slice = p.T;
+  }
+  p.Tp = (p.slice + 3u) & ~3u;
+  p.t0 = 0;
+  p.Ts = p.slice;
+  p.Tsp = p.Tp;
   // one thread per (channel, tile) with 32-bit indices; every GEMM slice below 2 GB
   if ((unsigned long long)Cs * p.Tp >= (1ull << 29) || (unsigned long long)M * p.Tp >= (1ull << 29) ||
       (unsigned long long)Cs * p.Mp >= (1ull << 29))
@@ -419,7 +453,7 @@ static bool make_plan(int N, int Cs, int Hs, int Ws, int M, int OH, int OW, int 
   return Cs % 16 == 0;
 }
 
-static int run(const Plan& p, const float* src, const float* w, bool flip, const float* bias,
+static int run(Plan p, const float* src, const float* w, bool flip, const float* bias,
                float* dst, bool accum, void* ws, size_t ws_bytes, hipStream_t s) {
   const size_t need = (u_floats(p) + v_floats(p) + m_floats(p)) * sizeof(float);
   if (!ws || ws_bytes < need || !mn_aligned(ws, 16)) return MN_EINVAL;
@@ -431,15 +465,20 @@ static int run(const Plan& p, const float* src, const float* w, bool flip, const
     weight_kernel<true><<<(nu + kThreads - 1) / kThreads, kThreads, 0, s>>>(w, U, p.M, p.Mp, p.Cs);
   else
     weight_kernel<false><<<(nu + kThreads - 1) / kThreads, kThreads, 0, s>>>(w, U, p.M, p.Mp, p.Cs);
-  const uint32_t nv = (uint32_t)p.Cs * p.Tp;
-  input_kernel<<<(nv + kThreads - 1) / kThreads, kThreads, 0, s>>>(p, src, V);
-  const int st = mn_conv_batched_gemm(U, V, Mt, p.M, p.Mp, p.Cs, p.Tp, 16, s);
-  if (st != MN_OK) return st;
-  const uint32_t no = (uint32_t)p.M * p.Tp;
-  if (accum)
-    output_kernel<true><<<(no + kThreads - 1) / kThreads, kThreads, 0, s>>>(p, Mt, bias, dst);
-  else
-    output_kernel<false><<<(no + kThreads - 1) / kThreads, kThreads, 0, s>>>(p, Mt, bias, dst);
+  for (uint32_t t0 = 0; t0 < p.T; t0 += p.slice) {
+    p.t0 = t0;
+    p.Ts = p.T - t0 < p.slice ? p.T - t0 : p.slice;
+    p.Tsp = (p.Ts + 3u) & ~3u;
+    const uint32_t nv = (uint32_t)p.Cs * p.Tsp;
+    input_kernel<<<(nv + kThreads - 1) / kThreads, kThreads, 0, s>>>(p, src, V);
+    const int st = mn_conv_batched_gemm(U, V, Mt, p.M, p.Mp, p.Cs, p.Tsp, 16, s);
+    if (st != MN_OK) return st;
+    const uint32_t no = (uint32_t)p.M * p.Tsp;
+    if (accum)
+      output_kernel<true><<<(no + kThreads - 1) / kThreads, kThreads, 0, s>>>(p, Mt, bias, dst);
+    else
+      output_kernel<false><<<(no + kThreads - 1) / kThreads, kThreads, 0, s>>>(p, Mt, bias, dst);
+  }
   return mn_launch_status();
 }
 
@@ -504,12 +543,18 @@ int mn_wino_bwd_weight(const mn_conv2d* g, const float* dy, const float* x, floa
   float* V = U + wu_floats(w);
   float* Z = V + wv_floats(w);
   const dim3 gu(w.Tpad / 32, w.Kp / 32), gv(w.Tpad / 32, (w.C + 31) / 32);
-  wgrad_transform_kernel<true><<<gu, kThreads, 0, s>>>(w.p, w.K, dy, U, w.Kp, w.Tpad);
-  wgrad_transform_kernel<false><<<gv, kThreads, 0, s>>>(w.p, w.C, x, V, w.C, w.Tpad);
-  const int st = mn_conv_batched_gemm(U, V, Z, w.K, w.Kp, (int)w.Tc, (uint32_t)w.C, 16 * w.S, s);
-  if (st != MN_OK) return st;
   const uint32_t n = (uint32_t)w.K * w.C;
-  wgrad_output_kernel<<<(n + 63) / 64, kThreads, 0, s>>>(Z, dw, w.K, w.C, w.S);
+  for (uint32_t pass = 0; pass < w.passes; ++pass) {
+    w.p.t0 = pass * w.Tpad;
+    wgrad_transform_kernel<true><<<gu, kThreads, 0, s>>>(w.p, w.K, dy, U, w.Kp, w.Tpad);
+    wgrad_transform_kernel<false><<<gv, kThreads, 0, s>>>(w.p, w.C, x, V, w.C, w.Tpad);
+    const int st = mn_conv_batched_gemm(U, V, Z, w.K, w.Kp, (int)w.Tc, (uint32_t)w.C, 16 * w.S, s);
+    if (st != MN_OK) return st;
+    if (pass == 0)
+      wgrad_output_kernel<false><<<(n + 63) / 64, kThreads, 0, s>>>(Z, dw, w.K, w.C, w.S);
+    else
+      wgrad_output_kernel<true><<<(n + 63) / 64, kThreads, 0, s>>>(Z, dw, w.K, w.C, w.S);
+  }
   if (db) bias_grad_kernel<<<w.K, kThreads, 0, s>>>(dy, db, g->N, g->K, g->P * g->Q);
   return mn_launch_status();
 }

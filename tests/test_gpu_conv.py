@@ -377,3 +377,52 @@ def test_conv_bias_gradient_entry_point_rejects_bf16_and_null(cuda):
         _lib.call("mn_conv_bwd_weight_bias", geo, _lib.ptr(buf), _lib.ptr(buf), _lib.ptr(buf),
                   None, None, 0, 0, _lib.F32, _lib.stream_ptr(buf.device))
     assert e.value.status == _lib.MN_EINVAL
+
+
+def test_winograd_runs_slice_after_slice_when_its_buffers_would_pass_512_MB(cuda):
+    """Variant 2 keeps its transformed tensors under 512 MB: a larger problem is cut into
+    ranges of tiles that run one after the other through the same buffers (forward and
+    backward-data), or into passes whose results are added in order (backward-weight).
+    [4, 256, 161, 159] -> 256 channels is 25 920 tiles of 32 KB = two slices, the second one
+    shorter, with ragged tiles at the right and bottom edges.  Checked against float64 on
+    sampled output elements and against variant 1 everywhere."""
+    xs, ws, pad = (4, 256, 161, 159), (256, 256, 3, 3), 1
+    rng = np.random.default_rng(5)
+    x, w, b = problem(xs, ws, 7)
+    dy = rng.standard_normal((xs[0], ws[0], xs[2], xs[3])).astype(np.float32)
+    xd, wd, bd, dyd = dev(x, cuda), dev(w, cuda), dev(b, cuda), dev(dy, cuda)
+    xp = np.pad(x.astype(np.float64), ((0, 0), (0, 0), (1, 1), (1, 1)))
+    dyp = np.pad(dy.astype(np.float64), ((0, 0), (0, 0), (1, 1), (1, 1)))
+    w64 = w.astype(np.float64)
+
+    y1 = conv_ops.conv_forward(xd, wd, bd, pad, 1, 1, 1, 1)
+    y2 = conv_ops.conv_forward(xd, wd, bd, pad, 1, 1, 1, 2)
+    assert_rel(host(y2), host(y1), 2e-5, "sliced Winograd forward vs variant 1")
+    idx = [(rng.integers(xs[0]), rng.integers(ws[0]), rng.integers(xs[2]), rng.integers(xs[3]))
+           for _ in range(256)] + [(3, 255, 160, 158), (0, 0, 0, 0), (2, 17, 160, 0)]
+    exp = np.array([(xp[n, :, h:h + 3, q:q + 3] * w64[k]).sum() + b[k] for n, k, h, q in idx])
+    got = host(y2)[tuple(np.array(idx).T)]
+    assert_rel(got, exp, TOL, "sliced Winograd forward vs float64 samples")
+
+    dx1 = conv_ops.conv_backward_input(xs, dyd, wd, pad, 1, 1, 1, 1)
+    dx2 = conv_ops.conv_backward_input(xs, dyd, wd, pad, 1, 1, 1, 2)
+    assert_rel(host(dx2), host(dx1), 2e-5, "sliced Winograd backward-data vs variant 1")
+    idx = [(rng.integers(xs[0]), rng.integers(xs[1]), rng.integers(xs[2]), rng.integers(xs[3]))
+           for _ in range(256)] + [(3, 255, 160, 158), (0, 0, 0, 0)]
+    # dx[n, c, h, q] = sum over k, r, s of dy[n, k, h + 1 - r, q + 1 - s] w[k, c, r, s]
+    exp = np.array([(dyp[n, :, h:h + 3, q:q + 3][:, ::-1, ::-1] * w64[:, c]).sum()
+                    for n, c, h, q in idx])
+    got = host(dx2)[tuple(np.array(idx).T)]
+    assert_rel(got, exp, TOL, "sliced Winograd backward-data vs float64 samples")
+
+    dw1 = conv_ops.conv_backward_weight(ws, dyd, xd, pad, 1, 1, 1, 1)
+    dw2 = conv_ops.conv_backward_weight(ws, dyd, xd, pad, 1, 1, 1, 2)
+    assert_rel(host(dw2), host(dw1), 2e-5, "Winograd backward-weight in passes vs variant 1")
+    idx = [(rng.integers(ws[0]), rng.integers(ws[1]), rng.integers(3), rng.integers(3))
+           for _ in range(48)]
+    dy64 = dy.astype(np.float64)
+    exp = np.array([(dy64[:, k] * xp[:, c, r:r + xs[2], s:s + xs[3]]).sum() for k, c, r, s in idx])
+    got = host(dw2)[tuple(np.array(idx).T)]
+    assert_rel(got, exp, TOL, "Winograd backward-weight in passes vs float64 samples")
+    # the same call again gives the same bits (fixed order of slices and passes)
+    assert torch.equal(dw2, conv_ops.conv_backward_weight(ws, dyd, xd, pad, 1, 1, 1, 2))
