@@ -29,6 +29,11 @@ int mn_wino_fwd(const mn_conv2d* g, const float* x, const float* w, const float*
                 void* ws, size_t ws_bytes, hipStream_t s);
 int mn_wino_bwd_data(const mn_conv2d* g, const float* dy, const float* w, float* dx, bool accum,
                      void* ws, size_t ws_bytes, hipStream_t s);
+int mn_wino_fused_ws_bytes(const mn_conv2d* g, bool backward_data, size_t* bytes);
+int mn_wino_fused_fwd(const mn_conv2d* g, const float* x, const float* w, const float* bias, float* y,
+                      void* ws, size_t ws_bytes, hipStream_t s);
+int mn_wino_fused_bwd_data(const mn_conv2d* g, const float* dy, const float* w, float* dx, bool accum,
+                           void* ws, size_t ws_bytes, hipStream_t s);
 int mn_wino_bwd_weight_ws_bytes(const mn_conv2d* g, size_t* bytes);
 int mn_wino_bwd_weight(const mn_conv2d* g, const float* dy, const float* x, float* dw, float* db,
                        void* ws, size_t ws_bytes, hipStream_t s);
@@ -1370,9 +1375,9 @@ extern "C" {
 int mn_conv_n_variants(int direction) {
   switch (direction) {
     case MN_CONV_FWD:
-      return 3;
+      return 4;
     case MN_CONV_BWD_DATA:
-      return 3;
+      return 4;
     case MN_CONV_BWD_WEIGHT:
       return 3;
     default:
@@ -1400,6 +1405,7 @@ int mn_conv_ws_bytes(const mn_conv2d* g, int direction, int variant, int dtype, 
   if (variant == 2)
     return direction == MN_CONV_BWD_WEIGHT ? mn_wino_bwd_weight_ws_bytes(g, bytes)
                                            : mn_wino_ws_bytes(g, direction == MN_CONV_BWD_DATA, bytes);
+  if (variant == 3) return mn_wino_fused_ws_bytes(g, direction == MN_CONV_BWD_DATA, bytes);
   const size_t wsize = (size_t)g->K * g->C * g->R * g->S * sizeof(float);
   // variant 1 of the gather directions: the repacked weight operand (rows padded to 128)
   if (direction == MN_CONV_FWD && variant == 1)
@@ -1420,7 +1426,7 @@ int mn_conv_fwd(const mn_conv2d* g, const void* x, const void* w, const void* bi
   using namespace mn_conv;
   const int st = check(g);
   if (st != MN_OK) return st;
-  if (variant < 0 || variant > 2 || (variant == 2 && dtype != MN_F32)) return MN_EUNSUPPORTED;
+  if (variant < 0 || variant > 3 || (variant >= 2 && dtype != MN_F32)) return MN_EUNSUPPORTED;
   if (g->N == 0) return MN_OK;
   if (!x || !w || !y) return MN_EINVAL;
   if (dtype == MN_BF16) return mn_conv16_fwd(g, x, w, bias, y, mn_stream(stream));
@@ -1428,6 +1434,9 @@ int mn_conv_fwd(const mn_conv2d* g, const void* x, const void* w, const void* bi
   if (variant == 2)
     return mn_wino_fwd(g, (const float*)x, (const float*)w, (const float*)bias, (float*)y, ws,
                        ws_bytes, mn_stream(stream));
+  if (variant == 3)
+    return mn_wino_fused_fwd(g, (const float*)x, (const float*)w, (const float*)bias, (float*)y, ws,
+                             ws_bytes, mn_stream(stream));
   Gather q = {};
   q.M = g->K;
   q.T = g->R * g->S;
@@ -1483,7 +1492,7 @@ static int conv_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void
   using namespace mn_conv;
   const int st = check(g);
   if (st != MN_OK) return st;
-  if (variant < 0 || variant > 2 || (variant == 2 && dtype != MN_F32)) return MN_EUNSUPPORTED;
+  if (variant < 0 || variant > 3 || (variant >= 2 && dtype != MN_F32)) return MN_EUNSUPPORTED;
   if (g->N == 0) return MN_OK;
   if (!dy || !w || !dx) return MN_EINVAL;
   hipStream_t s = mn_stream(stream);
@@ -1492,6 +1501,8 @@ static int conv_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void
   if (dtype != MN_F32) return MN_EUNSUPPORTED;
   if (variant == 2)
     return mn_wino_bwd_data(g, (const float*)dy, (const float*)w, (float*)dx, accum, ws, ws_bytes, s);
+  if (variant == 3)
+    return mn_wino_fused_bwd_data(g, (const float*)dy, (const float*)w, (float*)dx, accum, ws, ws_bytes, s);
   const int RS = g->R * g->S;
   const float* a = (const float*)w;
   uint32_t a_bytes = weight_bytes(g);  // size of the A operand: the weights, or their repacked copy

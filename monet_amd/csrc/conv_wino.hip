@@ -23,6 +23,7 @@ int mn_conv_batched_gemm(const float* a, const float* src, float* dst, int M, in
 namespace mn_wino {
 
 constexpr int kThreads = 256;
+constexpr int FK = 64, FT = 64, FC = 4;  // fused kernel: outputs, tiles per workgroup; channels per chunk
 constexpr unsigned long long kSliceBytes = 512ull << 20;  // cap of the transformed source + product buffers
 
 struct Plan {
@@ -43,7 +44,11 @@ static size_t m_floats(const Plan& p) { return (size_t)16 * p.M * p.Tp; }
 // U[pos][ch][m] = (G g G^T)[pos] for the 3x3 filter g of (m, ch).
 // FLIP = false (forward):      g[r][s] = w[m][ch][r][s]       (w is [M][Cs][3][3])
 // FLIP = true (backward-data): g[r][s] = w[ch][m][2-r][2-s]   (w is [Cs][M][3][3])
-template <bool FLIP>
+// BLOCKED (for the fused kernel): U[m / FK][ch / FC][pos][ch % FC][m % FK], so that what one
+// workgroup stages per chunk is 16 KB in one piece.  With rows of Mp floats every workgroup
+// reads 64 rows Mp * 4 bytes apart, at the same moment as all the others: for 512 outputs those
+// rows fall into two of an L2's sixteen channels and the loads queue up behind each other.
+template <bool FLIP, bool BLOCKED = false>
 __global__ __launch_bounds__(kThreads) void weight_kernel(const float* __restrict__ w,
                                                           float* __restrict__ U, int M, int Mp,
                                                           int Cs) {
@@ -70,17 +75,19 @@ __global__ __launch_bounds__(kThreads) void weight_kernel(const float* __restric
     t[2][s] = 0.5f * (g[0][s] - g[1][s] + g[2][s]);
     t[3][s] = g[2][s];
   }
-  const size_t stride = (size_t)Cs * Mp;
+  const size_t stride = BLOCKED ? (size_t)FC * FK : (size_t)Cs * Mp;
+  const size_t at = BLOCKED ? ((((size_t)(m / FK) * (Cs / FC) + ch / FC) * 16 * FC + ch % FC) * FK + m % FK)
+                            : (size_t)i;
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const float u0 = t[r][0];
     const float u1 = 0.5f * (t[r][0] + t[r][1] + t[r][2]);
     const float u2 = 0.5f * (t[r][0] - t[r][1] + t[r][2]);
     const float u3 = t[r][2];
-    U[(size_t)(4 * r + 0) * stride + i] = u0;
-    U[(size_t)(4 * r + 1) * stride + i] = u1;
-    U[(size_t)(4 * r + 2) * stride + i] = u2;
-    U[(size_t)(4 * r + 3) * stride + i] = u3;
+    U[(size_t)(4 * r + 0) * stride + at] = u0;
+    U[(size_t)(4 * r + 1) * stride + at] = u1;
+    U[(size_t)(4 * r + 2) * stride + at] = u2;
+    U[(size_t)(4 * r + 3) * stride + at] = u3;
   }
 }
 
@@ -178,6 +185,205 @@ __global__ __launch_bounds__(kThreads) void output_kernel(const Plan p, const fl
     } else {
       q[0] = y[a][0];
       if (ow + 1 < p.OW) q[1] = y[a][1];
+    }
+  }
+}
+
+// ------------------------------------------------------------------- fused --
+// The same algorithm in ONE kernel, with no transformed tensors in HBM (workspace = U only):
+// a workgroup owns 64 outputs x 64 tiles and keeps all 16 transform-domain products of that
+// block in registers (16 accumulator tiles of 32x32 per wavefront = 256 registers, one
+// wavefront per SIMD).  Per chunk of 4 channels it stages U[16][4][64] (copied) and
+// V[16][4][64] (each thread loads one 4x4 source patch and applies B^T . B) in LDS, double
+// buffered (odd channels with the column xor 32: an MFMA step reads an even and an odd channel
+// row in one instruction, which would otherwise meet in the same banks), and every wavefront
+// issues 16 positions x 2 steps of v_mfma_f32_32x32x2_f32.
+// At the end each lane holds, for its 16 (output, tile) pairs, the 16 values A^T . A needs.
+// It pays where the transforms of the unfused form dominate (few channels, large planes).
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ void input_transform(const float (&d)[4][4], float (&v)[16]) {
+  float t[4][4];  // t = B^T d
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    t[0][b] = d[0][b] - d[2][b];
+    t[1][b] = d[1][b] + d[2][b];
+    t[2][b] = d[2][b] - d[1][b];
+    t[3][b] = d[1][b] - d[3][b];
+  }
+#pragma unroll
+  for (int a = 0; a < 4; ++a) {  // v = t B
+    v[4 * a + 0] = t[a][0] - t[a][2];
+    v[4 * a + 1] = t[a][1] + t[a][2];
+    v[4 * a + 2] = t[a][2] - t[a][1];
+    v[4 * a + 3] = t[a][1] - t[a][3];
+  }
+}
+
+template <bool ACCUM>
+__global__ __launch_bounds__(kThreads) void fused_kernel(const Plan p, const float* __restrict__ src,
+                                                         const float* __restrict__ U,
+                                                         const float* __restrict__ bias,
+                                                         float* __restrict__ dst, uint32_t nkb) {
+  __shared__ __attribute__((aligned(16))) float Us[2][16][FC][FK];
+  __shared__ __attribute__((aligned(16))) float Vs[2][16][FC][FT];
+  const uint32_t slot = xcd_slot();
+  const uint32_t kb = slot % nkb, tb = slot / nkb;  // neighbours share the source patches
+  const int k0 = (int)kb * FK;
+  const uint32_t t0 = tb * FT;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint32_t per_img = (uint32_t)p.TH * p.TW;
+  const size_t plane = (size_t)p.Hs * p.Ws;
+
+  // loader role: the patch of tile t0 + lane in channel `wave` of every chunk
+  const uint32_t ltile = t0 + lane;
+  const bool lt_ok = ltile < p.T;
+  const uint32_t ln = lt_ok ? ltile / per_img : 0u, lr = lt_ok ? ltile - ln * per_img : 0u;
+  const int lth = lr / p.TW, ltw = lr - lth * p.TW;
+  const int h0 = 2 * lth - p.pad, w0 = 2 * ltw - p.pad;
+  // every load is issued unconditionally (straight-line code the scheduler can interleave with
+  // the MFMAs): rows and columns outside the image are read from the clamped coordinate and
+  // replaced by zero afterwards
+  bool rok[4], cok[4];
+  int roff[4], coff[4];
+#pragma unroll
+  for (int a = 0; a < 4; ++a) {
+    rok[a] = lt_ok && (unsigned)(h0 + a) < (unsigned)p.Hs;
+    cok[a] = (unsigned)(w0 + a) < (unsigned)p.Ws;
+    roff[a] = min(max(h0 + a, 0), p.Hs - 1) * p.Ws;
+    coff[a] = min(max(w0 + a, 0), p.Ws - 1);
+  }
+  const float* pp = src + ((size_t)ln * p.Cs + wave) * plane;  // advances FC planes per chunk
+  // U loader: four 16-byte pieces per thread and chunk, piece j = 16 bytes number tid + 256 j of
+  // the chunk's [16][FC][FK] block, which is contiguous in the blocked U
+  const float* up = U + (size_t)kb * (p.Cs / FC) * (16 * FC * FK) + 4 * tid;
+  const size_t ujump = (size_t)4 * kThreads;
+  const size_t ustep = (size_t)16 * FC * FK, pstep = (size_t)FC * plane;
+
+  // four register sets: the loads of chunks ch + 1 .. ch + 4 are in flight while chunk ch is
+  // multiplied (with a single wavefront per SIMD nothing else covers a trip to HBM, and the
+  // patch loads of a chunk were measured to take longer than two chunks of MFMAs)
+  float d0[4][4], d1[4][4], d2[4][4], d3[4][4];
+  float4_t u0[4], u1[4], u2[4], u3[4];
+  // `advance` = 0 near the end: the loop body has no branch (a conditional load would make the
+  // compiler wait for every load in flight at the join), so the last iterations load the last
+  // chunk again and nobody uses it
+  auto fetch = [&](float (&d)[4][4], float4_t (&uq)[4], bool advance) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) uq[j] = *reinterpret_cast<const float4_t*>(up + j * ujump);
+    up += advance ? ustep : 0;
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) d[a][b] = pp[roff[a] + coff[b]];
+    pp += advance ? pstep : 0;
+  };
+  auto stage = [&](int buf, float (&d)[4][4], const float4_t (&uq)[4]) {
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) d[a][b] = (rok[a] && cok[b]) ? d[a][b] : 0.f;
+    float v[16];
+    input_transform(d, v);
+#pragma unroll
+    for (int pos = 0; pos < 16; ++pos) Vs[buf][pos][wave][lane ^ ((wave & 1) << 5)] = v[pos];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      *reinterpret_cast<float4_t*>(&Us[buf][0][0][0] + 4 * ((tid + kThreads * j) ^ ((tid >> 1) & 8))) = uq[j];
+  };
+
+  float16_t acc[16];
+#pragma unroll
+  for (int pos = 0; pos < 16; ++pos)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[pos][v] = 0.f;
+
+  const int wk = (wave >> 1) * 32, wt = (wave & 1) * 32;
+  const int r = lane & 31, half = lane >> 5;
+  // all 64 operands of a chunk are requested from LDS first and the 32 MFMAs follow, each
+  // waiting only for its own pair: left to itself under this register pressure the scheduler
+  // reads one pair, waits, multiplies, and the LDS latency shows between every two MFMAs
+  auto multiply = [&](int buf) {
+    float av[FC / 2][16], bv[FC / 2][16];
+#pragma unroll
+    for (int cs = 0; cs < FC; cs += 2)
+#pragma unroll
+      for (int pos = 0; pos < 16; ++pos) {
+        av[cs / 2][pos] = Us[buf][pos][cs + half][(wk + r) ^ (half << 5)];
+        bv[cs / 2][pos] = Vs[buf][pos][cs + half][(wt + r) ^ (half << 5)];
+      }
+#pragma unroll
+    for (int cs = 0; cs < FC; cs += 2)
+#pragma unroll
+      for (int pos = 0; pos < 16; ++pos)
+        acc[pos] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[cs / 2][pos], bv[cs / 2][pos], acc[pos], 0, 0, 0);
+  };
+  // Order of one step, for the instruction scheduler: the MFMA of a 32x32x2 tile keeps the matrix
+  // pipe busy for 64 cycles after its issue, and this wavefront is alone on its SIMD, so
+  // everything else of the step (LDS reads of the operands, the global loads of a later chunk,
+  // the transform and the LDS writes of the next one) goes into the gaps between two MFMAs
+  // instead of before and after all 32 of them.
+  auto interleave = [&]() {
+    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);  // the operands of the first MFMAs
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);              // one MFMA
+      if (i < 24) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+      if (i < 20) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global load
+      __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);              // VALU
+      if (i >= 20) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); // one LDS write
+    }
+  };
+  // the channel count is a multiple of 16, so the number of chunks is a multiple of 4
+  const int nchunks = p.Cs / FC;
+  fetch(d0, u0, 1 < nchunks);
+  fetch(d1, u1, 2 < nchunks);
+  fetch(d2, u2, 3 < nchunks);
+  fetch(d3, u3, 4 < nchunks);  // the pointers now stand at chunk 4, or stay at the last one
+  stage(0, d0, u0);
+  __syncthreads();
+  // one step: load chunk c + 4 into the set chunk c came from, multiply chunk c, stage chunk c + 1
+#define MN_WINO_STEP(c, buf, dk, uk, dn, un)  \
+  fetch(dk, uk, (c) + 5 < nchunks);           \
+  multiply(buf);                              \
+  stage((buf) ^ 1, dn, un);                   \
+  interleave();                               \
+  __syncthreads();
+  for (int ch = 0; ch < nchunks; ch += 4) {
+    MN_WINO_STEP(ch, 0, d0, u0, d1, u1)
+    MN_WINO_STEP(ch + 1, 1, d1, u1, d2, u2)
+    MN_WINO_STEP(ch + 2, 0, d2, u2, d3, u3)
+    MN_WINO_STEP(ch + 3, 1, d3, u3, d0, u0)
+  }
+#undef MN_WINO_STEP
+
+  // output transform: this lane's tile is t0 + wt + r, its outputs k0 + wk + row(v)
+  const uint32_t etile = t0 + wt + r;
+  if (etile >= p.T) return;
+  const uint32_t en = etile / per_img, er = etile - en * per_img;
+  const int eth = er / p.TW, etw = er - eth * p.TW;
+  const int oh = 2 * eth, ow = 2 * etw;
+  const bool row1 = oh + 1 < p.OH, col1 = ow + 1 < p.OW;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const int k = k0 + wk + 8 * (v >> 2) + 4 * half + (v & 3);
+    if (k >= p.M) continue;
+    float t[2][4];  // t = A^T m, m[a][b] = acc[4a + b][v]
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      t[0][b] = acc[b][v] + acc[4 + b][v] + acc[8 + b][v];
+      t[1][b] = acc[4 + b][v] - acc[8 + b][v] - acc[12 + b][v];
+    }
+    const float bv = bias ? bias[k] : 0.f;
+    float* o = dst + (((size_t)en * p.M + k) * p.OH + oh) * p.OW + ow;
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+      if (a == 1 && !row1) break;
+      float* q = o + (size_t)a * p.OW;
+      const float y0 = t[a][0] + t[a][1] + t[a][2] + bv;
+      const float y1 = t[a][1] - t[a][2] - t[a][3] + bv;
+      q[0] = ACCUM ? q[0] + y0 : y0;
+      if (col1) q[1] = ACCUM ? q[1] + y1 : y1;
     }
   }
 }
@@ -482,6 +688,25 @@ static int run(Plan p, const float* src, const float* w, bool flip, const float*
   return mn_launch_status();
 }
 
+static int run_fused(const Plan& p, const float* src, const float* w, bool flip, const float* bias,
+                     float* dst, bool accum, void* ws, size_t ws_bytes, hipStream_t s) {
+  const size_t need = u_floats(p) * sizeof(float);
+  if (!ws || ws_bytes < need || !mn_aligned(ws, 16)) return MN_EINVAL;
+  float* U = static_cast<float*>(ws);
+  const uint32_t nu = (uint32_t)p.Cs * p.Mp;
+  if (flip)
+    weight_kernel<true, true><<<(nu + kThreads - 1) / kThreads, kThreads, 0, s>>>(w, U, p.M, p.Mp, p.Cs);
+  else
+    weight_kernel<false, true><<<(nu + kThreads - 1) / kThreads, kThreads, 0, s>>>(w, U, p.M, p.Mp, p.Cs);
+  const uint32_t nkb = (uint32_t)(p.M + FK - 1) / FK, ntb = (p.T + FT - 1) / FT;
+  if ((unsigned long long)nkb * ntb >= (1ull << 31)) return MN_EUNSUPPORTED;
+  if (accum)
+    fused_kernel<true><<<nkb * ntb, kThreads, 0, s>>>(p, src, U, bias, dst, nkb);
+  else
+    fused_kernel<false><<<nkb * ntb, kThreads, 0, s>>>(p, src, U, bias, dst, nkb);
+  return mn_launch_status();
+}
+
 static bool shape_ok(const mn_conv2d* g) {
   return g->R == 3 && g->S == 3 && g->sH == 1 && g->sW == 1 && g->dH == 1 && g->dW == 1 &&
          g->pH == g->pW && g->pH <= 2 && g->groups == 1;
@@ -520,6 +745,38 @@ int mn_wino_bwd_data(const mn_conv2d* g, const float* dy, const float* w, float*
   if (!shape_ok(g) || !make_plan(g->N, g->K, g->P, g->Q, g->C, g->H, g->W, 2 - g->pH, p))
     return MN_EUNSUPPORTED;
   return run(p, dy, w, true, nullptr, dx, accum, ws, ws_bytes, s);
+}
+
+// The fused kernel: workspace = the transformed weights only.
+int mn_wino_fused_ws_bytes(const mn_conv2d* g, bool backward_data, size_t* bytes) {
+  using namespace mn_wino;
+  *bytes = 0;
+  if (!shape_ok(g)) return MN_EUNSUPPORTED;
+  Plan p;
+  const bool ok = backward_data
+                      ? make_plan(g->N, g->K, g->P, g->Q, g->C, g->H, g->W, 2 - g->pH, p)
+                      : make_plan(g->N, g->C, g->H, g->W, g->K, g->P, g->Q, g->pH, p);
+  if (!ok) return MN_EUNSUPPORTED;
+  *bytes = u_floats(p) * sizeof(float);
+  return MN_OK;
+}
+
+int mn_wino_fused_fwd(const mn_conv2d* g, const float* x, const float* w, const float* bias, float* y,
+                      void* ws, size_t ws_bytes, hipStream_t s) {
+  using namespace mn_wino;
+  Plan p;
+  if (!shape_ok(g) || !make_plan(g->N, g->C, g->H, g->W, g->K, g->P, g->Q, g->pH, p))
+    return MN_EUNSUPPORTED;
+  return run_fused(p, x, w, false, bias, y, false, ws, ws_bytes, s);
+}
+
+int mn_wino_fused_bwd_data(const mn_conv2d* g, const float* dy, const float* w, float* dx, bool accum,
+                           void* ws, size_t ws_bytes, hipStream_t s) {
+  using namespace mn_wino;
+  Plan p;
+  if (!shape_ok(g) || !make_plan(g->N, g->K, g->P, g->Q, g->C, g->H, g->W, 2 - g->pH, p))
+    return MN_EUNSUPPORTED;
+  return run_fused(p, dy, w, true, nullptr, dx, accum, ws, ws_bytes, s);
 }
 
 // Weight gradient (fp32) through the Winograd form above; db (optional): the bias gradient.

@@ -44,7 +44,8 @@ CASES = [
 
 
 def winograd_applies(ws, st, pad, dil, reduced_channels):
-    """Variant 2 (Winograd F(2x2, 3x3)) covers 3x3 filters, stride 1, dilation 1, equal
+    """Variants 2 and 3 (Winograd F(2x2, 3x3), through transformed tensors in the workspace /
+    in one kernel) cover 3x3 filters, stride 1, dilation 1, equal
     padding <= 2 on both axes and a reduction over a multiple of 16 channels; anything else
     must be refused with MN_EUNSUPPORTED."""
     pair = lambda v: tuple(v) if isinstance(v, (tuple, list)) else (v, v)
@@ -96,9 +97,9 @@ def test_conv_forward(cuda, xs, ws, st, pad, dil):
     x, w, b = problem(xs, ws)
     exp = O.conv_fwd(x, w, b, st, pad, dil)
     exp_nobias = O.conv_fwd(x, w, None, st, pad, dil)
-    assert conv_ops.n_fwd_algos() == 3
+    assert conv_ops.n_fwd_algos() == 4
     for v in range(conv_ops.n_fwd_algos()):
-        if v == 2 and not winograd_applies(ws, st, pad, dil, xs[1]):
+        if v >= 2 and not winograd_applies(ws, st, pad, dil, xs[1]):
             assert refused(lambda: conv_ops.conv_forward(dev(x, cuda), dev(w, cuda), None, pad, st,
                                                          dil, 1, v))
             continue
@@ -115,9 +116,9 @@ def test_conv_backward_data(cuda, xs, ws, st, pad, dil):
     yshape = O.conv_fwd(x, w, None, st, pad, dil).shape
     dy = np.random.default_rng(2).standard_normal(yshape).astype(np.float32)
     exp = O.conv_bwd_data(dy, w, xs, st, pad, dil)
-    assert conv_ops.n_bwd_ip_algos() == 3
+    assert conv_ops.n_bwd_ip_algos() == 4
     for v in range(conv_ops.n_bwd_ip_algos()):
-        if v == 2 and not winograd_applies(ws, st, pad, dil, ws[0]):
+        if v >= 2 and not winograd_applies(ws, st, pad, dil, ws[0]):
             assert refused(lambda: conv_ops.conv_backward_input(xs, dev(dy, cuda), dev(w, cuda),
                                                                 pad, st, dil, 1, v))
             continue
@@ -319,7 +320,7 @@ def test_conv_backward_data_accumulates_into_an_existing_gradient(cuda, xs, ws, 
     prior = rng.standard_normal(xs).astype(np.float32)
     exp = prior.astype(np.float64) + O.conv_bwd_data(dy, w, xs, st, pad, dil)
     for v in range(conv_ops.n_bwd_ip_algos()):
-        if v == 2 and not winograd_applies(ws, st, pad, dil, ws[0]):
+        if v >= 2 and not winograd_applies(ws, st, pad, dil, ws[0]):
             continue
         acc = dev(prior, cuda)
         out = conv_ops.conv_backward_input(xs, dev(dy, cuda), dev(w, cuda), pad, st, dil, 1, v,
