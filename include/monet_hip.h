@@ -327,6 +327,14 @@ typedef struct mn_conv2d {
  *                      of tiles through the same buffers (the role of the
  *                      reference's WINOGRAD_NONFUSED slot,
  *                      monet/lm_ops/conv.cpp:21-27, :314-324)
+ *                    3 the same algorithm in one kernel: source patches and
+ *                      weights are transformed on the way into LDS and the 16
+ *                      products of a block of 64 outputs x 64 tiles stay in
+ *                      registers until the output transform, so the only
+ *                      workspace is the transformed weights (16 * C *
+ *                      pad128(K) floats; the role of the reference's fused
+ *                      WINOGRAD slot).  Same shapes as variant 2; faster than
+ *                      it where channels are few and planes large
  *   backward-data    0 implicit GEMM reading the weights through strides
  *                    1 same with the weights repacked [tap][k][c] (c padded
  *                      to a multiple of 128) into the workspace; may split
@@ -335,6 +343,7 @@ typedef struct mn_conv2d {
  *                      0 never does)
  *                    2 Winograd F(2x2, 3x3), as for the forward (the filter
  *                      rotated by 180 degrees, channel roles swapped)
+ *                    3 the one-kernel Winograd form, as for the forward
  *   backward-weight  0 split reduction combined with atomics into a cleared dw
  *                    1 split reduction through per-split partials in the
  *                      workspace, then a fixed-order sum (reproducible)

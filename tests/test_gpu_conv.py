@@ -397,24 +397,28 @@ def test_winograd_runs_slice_after_slice_when_its_buffers_would_pass_512_MB(cuda
     w64 = w.astype(np.float64)
 
     y1 = conv_ops.conv_forward(xd, wd, bd, pad, 1, 1, 1, 1)
-    y2 = conv_ops.conv_forward(xd, wd, bd, pad, 1, 1, 1, 2)
-    assert_rel(host(y2), host(y1), 2e-5, "sliced Winograd forward vs variant 1")
     idx = [(rng.integers(xs[0]), rng.integers(ws[0]), rng.integers(xs[2]), rng.integers(xs[3]))
            for _ in range(256)] + [(3, 255, 160, 158), (0, 0, 0, 0), (2, 17, 160, 0)]
     exp = np.array([(xp[n, :, h:h + 3, q:q + 3] * w64[k]).sum() + b[k] for n, k, h, q in idx])
-    got = host(y2)[tuple(np.array(idx).T)]
-    assert_rel(got, exp, TOL, "sliced Winograd forward vs float64 samples")
+    for v in (2, 3):   # in slices through the workspace; in one kernel (405 blocks of 64 tiles)
+        y = conv_ops.conv_forward(xd, wd, bd, pad, 1, 1, 1, v)
+        assert_rel(host(y), host(y1), 2e-5, f"Winograd forward variant {v} vs variant 1")
+        assert_rel(host(y)[tuple(np.array(idx).T)], exp, TOL,
+                   f"Winograd forward variant {v} vs float64 samples")
+        del y
 
     dx1 = conv_ops.conv_backward_input(xs, dyd, wd, pad, 1, 1, 1, 1)
-    dx2 = conv_ops.conv_backward_input(xs, dyd, wd, pad, 1, 1, 1, 2)
-    assert_rel(host(dx2), host(dx1), 2e-5, "sliced Winograd backward-data vs variant 1")
     idx = [(rng.integers(xs[0]), rng.integers(xs[1]), rng.integers(xs[2]), rng.integers(xs[3]))
            for _ in range(256)] + [(3, 255, 160, 158), (0, 0, 0, 0)]
     # dx[n, c, h, q] = sum over k, r, s of dy[n, k, h + 1 - r, q + 1 - s] w[k, c, r, s]
     exp = np.array([(dyp[n, :, h:h + 3, q:q + 3][:, ::-1, ::-1] * w64[:, c]).sum()
                     for n, c, h, q in idx])
-    got = host(dx2)[tuple(np.array(idx).T)]
-    assert_rel(got, exp, TOL, "sliced Winograd backward-data vs float64 samples")
+    for v in (2, 3):
+        dx = conv_ops.conv_backward_input(xs, dyd, wd, pad, 1, 1, 1, v)
+        assert_rel(host(dx), host(dx1), 2e-5, f"Winograd backward-data variant {v} vs variant 1")
+        assert_rel(host(dx)[tuple(np.array(idx).T)], exp, TOL,
+                   f"Winograd backward-data variant {v} vs float64 samples")
+        del dx
 
     dw1 = conv_ops.conv_backward_weight(ws, dyd, xd, pad, 1, 1, 1, 1)
     dw2 = conv_ops.conv_backward_weight(ws, dyd, xd, pad, 1, 1, 1, 2)
