@@ -34,6 +34,7 @@ struct Plan {
   uint32_t T, Tp;      // tiles; row capacity of V and Mt (tiles of the largest slice, multiple of 4)
   uint32_t slice;      // tiles per slice: the transforms and the GEMM run slice after slice
   uint32_t t0, Ts, Tsp;  // the current slice: first tile, tiles, row length (multiple of 4)
+  uint32_t src_bytes, u_bytes;  // fused kernel: sizes of the source tensor and of U (0: 2 GB or more)
   int Mp;              // rows of U padded to a multiple of 128
 };
 
@@ -241,24 +242,31 @@ __global__ __launch_bounds__(kThreads) void fused_kernel(const Plan p, const flo
   const uint32_t ln = lt_ok ? ltile / per_img : 0u, lr = lt_ok ? ltile - ln * per_img : 0u;
   const int lth = lr / p.TW, ltw = lr - lth * p.TW;
   const int h0 = 2 * lth - p.pad, w0 = 2 * ltw - p.pad;
-  // every load is issued unconditionally (straight-line code the scheduler can interleave with
-  // the MFMAs): rows and columns outside the image are read from the clamped coordinate and
-  // replaced by zero afterwards
-  bool rok[4], cok[4];
-  int roff[4], coff[4];
+  // Every load is issued unconditionally (straight-line code the scheduler can interleave with
+  // the MFMAs) through a buffer descriptor: the per-lane part of an address is a byte offset
+  // that stays the same for all chunks, the per-chunk part is uniform and travels in the
+  // scalar offset of the load, so a load costs no address arithmetic; a patch element outside
+  // the image gets an offset beyond the buffer, which the hardware answers with zero.
+  constexpr uint32_t kBeyond = 0x80000000u;
+  const __amdgpu_buffer_rsrc_t src_buf =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(src), 0, p.src_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t u_buf =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(U), 0, p.u_bytes, 0x00020000);
+  uint32_t eoff[4][4];
+  const uint32_t pbase = (uint32_t)(((size_t)ln * p.Cs + wave) * plane);
 #pragma unroll
-  for (int a = 0; a < 4; ++a) {
-    rok[a] = lt_ok && (unsigned)(h0 + a) < (unsigned)p.Hs;
-    cok[a] = (unsigned)(w0 + a) < (unsigned)p.Ws;
-    roff[a] = min(max(h0 + a, 0), p.Hs - 1) * p.Ws;
-    coff[a] = min(max(w0 + a, 0), p.Ws - 1);
-  }
-  const float* pp = src + ((size_t)ln * p.Cs + wave) * plane;  // advances FC planes per chunk
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const bool ok = lt_ok && (unsigned)(h0 + a) < (unsigned)p.Hs && (unsigned)(w0 + b) < (unsigned)p.Ws;
+      eoff[a][b] = ok ? (pbase + (uint32_t)((h0 + a) * p.Ws + (w0 + b))) * 4u : kBeyond;
+    }
   // U loader: four 16-byte pieces per thread and chunk, piece j = 16 bytes number tid + 256 j of
   // the chunk's [16][FC][FK] block, which is contiguous in the blocked U
-  const float* up = U + (size_t)kb * (p.Cs / FC) * (16 * FC * FK) + 4 * tid;
-  const size_t ujump = (size_t)4 * kThreads;
-  const size_t ustep = (size_t)16 * FC * FK, pstep = (size_t)FC * plane;
+  const uint32_t uoff = 16u * tid;
+  uint32_t u_so = kb * (uint32_t)(p.Cs / FC) * (16u * FC * FK * 4u);  // byte offset of the next chunk of U
+  uint32_t p_so = 0;                                                    // ... and of the source planes
+  const uint32_t ustep = 16u * FC * FK * 4u, pstep = (uint32_t)(FC * plane * 4);
 
   // four register sets: the loads of chunks ch + 1 .. ch + 4 are in flight while chunk ch is
   // multiplied (with a single wavefront per SIMD nothing else covers a trip to HBM, and the
@@ -270,19 +278,18 @@ __global__ __launch_bounds__(kThreads) void fused_kernel(const Plan p, const flo
   // chunk again and nobody uses it
   auto fetch = [&](float (&d)[4][4], float4_t (&uq)[4], bool advance) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) uq[j] = *reinterpret_cast<const float4_t*>(up + j * ujump);
-    up += advance ? ustep : 0;
+    for (int j = 0; j < 4; ++j)
+      uq[j] = __builtin_bit_cast(
+          float4_t, __builtin_amdgcn_raw_buffer_load_b128(u_buf, uoff, u_so + 16u * kThreads * j, 0));
+    u_so += advance ? ustep : 0u;
 #pragma unroll
     for (int a = 0; a < 4; ++a)
 #pragma unroll
-      for (int b = 0; b < 4; ++b) d[a][b] = pp[roff[a] + coff[b]];
-    pp += advance ? pstep : 0;
+      for (int b = 0; b < 4; ++b)
+        d[a][b] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(src_buf, eoff[a][b], p_so, 0));
+    p_so += advance ? pstep : 0u;
   };
   auto stage = [&](int buf, float (&d)[4][4], const float4_t (&uq)[4]) {
-#pragma unroll
-    for (int a = 0; a < 4; ++a)
-#pragma unroll
-      for (int b = 0; b < 4; ++b) d[a][b] = (rok[a] && cok[b]) ? d[a][b] : 0.f;
     float v[16];
     input_transform(d, v);
 #pragma unroll
@@ -330,7 +337,7 @@ __global__ __launch_bounds__(kThreads) void fused_kernel(const Plan p, const flo
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);              // one MFMA
       if (i < 24) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
       if (i < 20) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global load
-      __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);              // VALU
+      __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);              // VALU
       if (i >= 20) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); // one LDS write
     }
   };
@@ -648,6 +655,10 @@ static bool make_plan(int N, int Cs, int Hs, int Ws, int M, int OH, int OW, int 
     p.slice = (uint32_t)(t < 256 ? 256 : t);
     if (p.slice > p.T) p.slice = p.T;
   }
+  // the fused kernel addresses its operands through buffer descriptors with 31-bit byte offsets
+  const unsigned long long sb = (unsigned long long)N * Cs * Hs * Ws * 4ull, ub = 64ull * Cs * p.Mp;
+  p.src_bytes = sb < (1ull << 31) ? (uint32_t)sb : 0u;
+  p.u_bytes = ub < (1ull << 31) ? (uint32_t)ub : 0u;
   p.Tp = (p.slice + 3u) & ~3u;
   p.t0 = 0;
   p.Ts = p.slice;
@@ -699,7 +710,7 @@ static int run_fused(const Plan& p, const float* src, const float* w, bool flip,
   else
     weight_kernel<false, true><<<(nu + kThreads - 1) / kThreads, kThreads, 0, s>>>(w, U, p.M, p.Mp, p.Cs);
   const uint32_t nkb = (uint32_t)(p.M + FK - 1) / FK, ntb = (p.T + FT - 1) / FT;
-  if ((unsigned long long)nkb * ntb >= (1ull << 31)) return MN_EUNSUPPORTED;
+  if ((unsigned long long)nkb * ntb >= (1ull << 31) || !p.src_bytes || !p.u_bytes) return MN_EUNSUPPORTED;
   if (accum)
     fused_kernel<true><<<nkb * ntb, kThreads, 0, s>>>(p, src, U, bias, dst, nkb);
   else
@@ -756,7 +767,7 @@ int mn_wino_fused_ws_bytes(const mn_conv2d* g, bool backward_data, size_t* bytes
   const bool ok = backward_data
                       ? make_plan(g->N, g->K, g->P, g->Q, g->C, g->H, g->W, 2 - g->pH, p)
                       : make_plan(g->N, g->C, g->H, g->W, g->K, g->P, g->Q, g->pH, p);
-  if (!ok) return MN_EUNSUPPORTED;
+  if (!ok || !p.src_bytes || !p.u_bytes) return MN_EUNSUPPORTED;  // 2 GB or more: not through this kernel
   *bytes = u_floats(p) * sizeof(float);
   return MN_OK;
 }
