@@ -15,6 +15,8 @@
 // GEMM in conv.hip), Mt -> destination (+ bias, or added to what the destination holds).
 // Backward-data is the same computation on dy with the filter rotated by 180 degrees, the two
 // channel roles swapped and padding 2 - pad.
+#include <mutex>
+
 #include "common.h"
 
 int mn_conv_batched_gemm(const float* a, const float* src, float* dst, int M, int Mp, int Cs,
@@ -45,10 +47,10 @@ static size_t m_floats(const Plan& p) { return (size_t)16 * p.M * p.Tp; }
 // U[pos][ch][m] = (G g G^T)[pos] for the 3x3 filter g of (m, ch).
 // FLIP = false (forward):      g[r][s] = w[m][ch][r][s]       (w is [M][Cs][3][3])
 // FLIP = true (backward-data): g[r][s] = w[ch][m][2-r][2-s]   (w is [Cs][M][3][3])
-// BLOCKED (for the fused kernel): U[m / FK][ch / FC][pos][ch % FC][m % FK], so that what one
-// workgroup stages per chunk is 16 KB in one piece.  With rows of Mp floats every workgroup
-// reads 64 rows Mp * 4 bytes apart, at the same moment as all the others: for 512 outputs those
-// rows fall into two of an L2's sixteen channels and the loads queue up behind each other.
+// BLOCKED (for the fused kernel): U[m / FK][ch / FC][ch % FC][m % FK][pos], so that what one
+// workgroup stages per chunk is 16 KB in one piece (with rows of Mp floats every workgroup
+// reads 64 rows Mp * 4 bytes apart at the same moment as all the others) and the 16 positions
+// of one (channel, output) pair are 64 bytes in a row, as the kernel's LDS layout wants them.
 template <bool FLIP, bool BLOCKED = false>
 __global__ __launch_bounds__(kThreads) void weight_kernel(const float* __restrict__ w,
                                                           float* __restrict__ U, int M, int Mp,
@@ -76,8 +78,8 @@ __global__ __launch_bounds__(kThreads) void weight_kernel(const float* __restric
     t[2][s] = 0.5f * (g[0][s] - g[1][s] + g[2][s]);
     t[3][s] = g[2][s];
   }
-  const size_t stride = BLOCKED ? (size_t)FC * FK : (size_t)Cs * Mp;
-  const size_t at = BLOCKED ? ((((size_t)(m / FK) * (Cs / FC) + ch / FC) * 16 * FC + ch % FC) * FK + m % FK)
+  const size_t stride = BLOCKED ? (size_t)1 : (size_t)Cs * Mp;
+  const size_t at = BLOCKED ? ((((size_t)(m / FK) * (Cs / FC) + ch / FC) * FC + ch % FC) * FK + m % FK) * 16
                             : (size_t)i;
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
@@ -194,13 +196,18 @@ __global__ __launch_bounds__(kThreads) void output_kernel(const Plan p, const fl
 // The same algorithm in ONE kernel, with no transformed tensors in HBM (workspace = U only):
 // a workgroup owns 64 outputs x 64 tiles and keeps all 16 transform-domain products of that
 // block in registers (16 accumulator tiles of 32x32 per wavefront = 256 registers, one
-// wavefront per SIMD).  Per chunk of 4 channels it stages U[16][4][64] (copied) and
-// V[16][4][64] (each thread loads one 4x4 source patch and applies B^T . B) in LDS, double
-// buffered (odd channels with the column xor 32: an MFMA step reads an even and an odd channel
-// row in one instruction, which would otherwise meet in the same banks), and every wavefront
-// issues 16 positions x 2 steps of v_mfma_f32_32x32x2_f32.
+// wavefront per SIMD).  Per chunk of 4 channels it stages U[4][64][16] (copied) and
+// V[4][64][16] (each thread loads one 4x4 source patch and applies B^T . B) in LDS, double
+// buffered, the 16 positions of a (channel, output) or (channel, tile) pair next to each other
+// so that a lane fetches its operands of 16 MFMAs with four 16-byte reads and a patch is staged
+// with four 16-byte writes (rows padded from 16 to 20 floats: 16 consecutive lanes then cover
+// all 64 banks once).  Every wavefront issues 16 positions x 2 steps of
+// v_mfma_f32_32x32x2_f32 per chunk.
 // At the end each lane holds, for its 16 (output, tile) pairs, the 16 values A^T . A needs.
 // It pays where the transforms of the unfused form dominate (few channels, large planes).
+constexpr int LP = 20;                                  // floats per LDS row of 16 positions
+constexpr int kFusedHalf = FC * FK * LP;                // floats of U (or V) in one buffer
+constexpr size_t kFusedLds = (size_t)4 * kFusedHalf * sizeof(float);  // U and V, two buffers: 80 KB
 typedef float float16_t __attribute__((ext_vector_type(16)));
 
 __device__ __forceinline__ void input_transform(const float (&d)[4][4], float (&v)[16]) {
@@ -226,8 +233,8 @@ __global__ __launch_bounds__(kThreads) void fused_kernel(const Plan p, const flo
                                                          const float* __restrict__ U,
                                                          const float* __restrict__ bias,
                                                          float* __restrict__ dst, uint32_t nkb) {
-  __shared__ __attribute__((aligned(16))) float Us[2][16][FC][FK];
-  __shared__ __attribute__((aligned(16))) float Vs[2][16][FC][FT];
+  extern __shared__ float4_t fused_lds[];  // [buffer][U | V][channel][output | tile][LP]
+  float* const lds = reinterpret_cast<float*>(fused_lds);
   const uint32_t slot = xcd_slot();
   const uint32_t kb = slot % nkb, tb = slot / nkb;  // neighbours share the source patches
   const int k0 = (int)kb * FK;
@@ -289,14 +296,20 @@ __global__ __launch_bounds__(kThreads) void fused_kernel(const Plan p, const flo
         d[a][b] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(src_buf, eoff[a][b], p_so, 0));
     p_so += advance ? pstep : 0u;
   };
+  // this thread's patch goes to row (channel = wave, tile = lane) of V; piece j of U (16 bytes
+  // number tid + 256 j of the chunk) is positions 4 (tid & 3) .. + 3 of row (tid >> 2) + 64 j
+  float* const vrow = lds + kFusedHalf + (wave * FT + lane) * LP;
+  float* const urow = lds + (tid >> 2) * LP + 4 * (tid & 3);
   auto stage = [&](int buf, float (&d)[4][4], const float4_t (&uq)[4]) {
     float v[16];
     input_transform(d, v);
 #pragma unroll
-    for (int pos = 0; pos < 16; ++pos) Vs[buf][pos][wave][lane ^ ((wave & 1) << 5)] = v[pos];
+    for (int q = 0; q < 4; ++q)
+      *reinterpret_cast<float4_t*>(vrow + buf * 2 * kFusedHalf + 4 * q) =
+          float4_t{v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]};
 #pragma unroll
     for (int j = 0; j < 4; ++j)
-      *reinterpret_cast<float4_t*>(&Us[buf][0][0][0] + 4 * ((tid + kThreads * j) ^ ((tid >> 1) & 8))) = uq[j];
+      *reinterpret_cast<float4_t*>(urow + buf * 2 * kFusedHalf + 64 * j * LP) = uq[j];
   };
 
   float16_t acc[16];
@@ -307,23 +320,25 @@ __global__ __launch_bounds__(kThreads) void fused_kernel(const Plan p, const flo
 
   const int wk = (wave >> 1) * 32, wt = (wave & 1) * 32;
   const int r = lane & 31, half = lane >> 5;
-  // all 64 operands of a chunk are requested from LDS first and the 32 MFMAs follow, each
-  // waiting only for its own pair: left to itself under this register pressure the scheduler
-  // reads one pair, waits, multiplies, and the LDS latency shows between every two MFMAs
+  // operands: row (channel 2 s + half, output wk + r) of U and (channel 2 s + half, tile wt + r)
+  // of V, 16 positions each, for the two steps s of a chunk
+  const float* const arow = lds + (half * FK + wk + r) * LP;
+  const float* const brow = lds + kFusedHalf + (half * FT + wt + r) * LP;
   auto multiply = [&](int buf) {
-    float av[FC / 2][16], bv[FC / 2][16];
+    float4_t av[FC / 2][4], bv[FC / 2][4];
 #pragma unroll
-    for (int cs = 0; cs < FC; cs += 2)
+    for (int cs = 0; cs < FC / 2; ++cs)
 #pragma unroll
-      for (int pos = 0; pos < 16; ++pos) {
-        av[cs / 2][pos] = Us[buf][pos][cs + half][(wk + r) ^ (half << 5)];
-        bv[cs / 2][pos] = Vs[buf][pos][cs + half][(wt + r) ^ (half << 5)];
+      for (int q = 0; q < 4; ++q) {
+        av[cs][q] = *reinterpret_cast<const float4_t*>(arow + buf * 2 * kFusedHalf + 2 * cs * FK * LP + 4 * q);
+        bv[cs][q] = *reinterpret_cast<const float4_t*>(brow + buf * 2 * kFusedHalf + 2 * cs * FT * LP + 4 * q);
       }
 #pragma unroll
-    for (int cs = 0; cs < FC; cs += 2)
+    for (int cs = 0; cs < FC / 2; ++cs)
 #pragma unroll
       for (int pos = 0; pos < 16; ++pos)
-        acc[pos] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[cs / 2][pos], bv[cs / 2][pos], acc[pos], 0, 0, 0);
+        acc[pos] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[cs][pos >> 2][pos & 3], bv[cs][pos >> 2][pos & 3],
+                                                        acc[pos], 0, 0, 0);
   };
   // Order of one step, for the instruction scheduler: the MFMA of a 32x32x2 tile keeps the matrix
   // pipe busy for 64 cycles after its issue, and this wavefront is alone on its SIMD, so
@@ -331,14 +346,14 @@ __global__ __launch_bounds__(kThreads) void fused_kernel(const Plan p, const flo
   // the transform and the LDS writes of the next one) goes into the gaps between two MFMAs
   // instead of before and after all 32 of them.
   auto interleave = [&]() {
-    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);  // the operands of the first MFMAs
+    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // the operands of the first four MFMAs
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);              // one MFMA
-      if (i < 24) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+      if (i < 14) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
       if (i < 20) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global load
       __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);              // VALU
-      if (i >= 20) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); // one LDS write
+      if (i >= 24) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); // one LDS write
     }
   };
   // the channel count is a multiple of 16, so the number of chunks is a multiple of 4
@@ -699,6 +714,24 @@ static int run(Plan p, const float* src, const float* w, bool flip, const float*
   return mn_launch_status();
 }
 
+// The fused kernel uses 80 KB of LDS per workgroup, more than a kernel gets without asking:
+// raise its limit once per device (gfx950 has 160 KB per CU).
+static bool fused_lds_allowed() {
+  static std::mutex lock;
+  static bool done[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
+  std::lock_guard<std::mutex> hold(lock);
+  if (done[dev]) return true;
+  const bool ok =
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_kernel<true>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kFusedLds) == hipSuccess &&
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_kernel<false>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kFusedLds) == hipSuccess;
+  done[dev] = ok;
+  return ok;
+}
+
 static int run_fused(const Plan& p, const float* src, const float* w, bool flip, const float* bias,
                      float* dst, bool accum, void* ws, size_t ws_bytes, hipStream_t s) {
   const size_t need = u_floats(p) * sizeof(float);
@@ -711,10 +744,11 @@ static int run_fused(const Plan& p, const float* src, const float* w, bool flip,
     weight_kernel<false, true><<<(nu + kThreads - 1) / kThreads, kThreads, 0, s>>>(w, U, p.M, p.Mp, p.Cs);
   const uint32_t nkb = (uint32_t)(p.M + FK - 1) / FK, ntb = (p.T + FT - 1) / FT;
   if ((unsigned long long)nkb * ntb >= (1ull << 31) || !p.src_bytes || !p.u_bytes) return MN_EUNSUPPORTED;
+  if (!fused_lds_allowed()) return MN_ELAUNCH;
   if (accum)
-    fused_kernel<true><<<nkb * ntb, kThreads, 0, s>>>(p, src, U, bias, dst, nkb);
+    fused_kernel<true><<<nkb * ntb, kThreads, kFusedLds, s>>>(p, src, U, bias, dst, nkb);
   else
-    fused_kernel<false><<<nkb * ntb, kThreads, 0, s>>>(p, src, U, bias, dst, nkb);
+    fused_kernel<false><<<nkb * ntb, kThreads, kFusedLds, s>>>(p, src, U, bias, dst, nkb);
   return mn_launch_status();
 }
 
