@@ -324,7 +324,21 @@ __global__ __launch_bounds__(kThreads) void fused_kernel(const Plan p, const flo
   // of V, 16 positions each, for the two steps s of a chunk
   const float* const arow = lds + (half * FK + wk + r) * LP;
   const float* const brow = lds + kFusedHalf + (half * FT + wt + r) * LP;
-  auto multiply = [&](int buf) {
+  // The last 8 MFMAs of a chunk (second step, positions 8..15) are issued at the START of the
+  // next step, from operands that wait in registers across the barrier: the new chunk's first
+  // LDS reads then travel while the matrix pipe is busy, instead of every step beginning with an
+  // idle pipe until the first operands arrive.
+  float4_t ca[2], cb[2];
+#pragma unroll
+  for (int q = 0; q < 2; ++q) ca[q] = cb[q] = float4_t{0.f, 0.f, 0.f, 0.f};
+  auto tail = [&]() {
+#pragma unroll
+    for (int q = 0; q < 2; ++q)
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        acc[8 + 4 * q + e] = __builtin_amdgcn_mfma_f32_32x32x2f32(ca[q][e], cb[q][e], acc[8 + 4 * q + e], 0, 0, 0);
+  };
+  auto head = [&](int buf) {
     float4_t av[FC / 2][4], bv[FC / 2][4];
 #pragma unroll
     for (int cs = 0; cs < FC / 2; ++cs)
@@ -334,11 +348,16 @@ __global__ __launch_bounds__(kThreads) void fused_kernel(const Plan p, const flo
         bv[cs][q] = *reinterpret_cast<const float4_t*>(brow + buf * 2 * kFusedHalf + 2 * cs * FT * LP + 4 * q);
       }
 #pragma unroll
-    for (int cs = 0; cs < FC / 2; ++cs)
+    for (int i = 0; i < 24; ++i) {  // step 0: 16 positions, step 1: positions 0..7
+      const int cs = i >> 4, pos = i & 15;
+      acc[pos] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[cs][pos >> 2][pos & 3], bv[cs][pos >> 2][pos & 3],
+                                                      acc[pos], 0, 0, 0);
+    }
 #pragma unroll
-      for (int pos = 0; pos < 16; ++pos)
-        acc[pos] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[cs][pos >> 2][pos & 3], bv[cs][pos >> 2][pos & 3],
-                                                        acc[pos], 0, 0, 0);
+    for (int q = 0; q < 2; ++q) {
+      ca[q] = av[1][2 + q];
+      cb[q] = bv[1][2 + q];
+    }
   };
   // Order of one step, for the instruction scheduler: the MFMA of a 32x32x2 tile keeps the matrix
   // pipe busy for 64 cycles after its issue, and this wavefront is alone on its SIMD, so
@@ -346,12 +365,11 @@ __global__ __launch_bounds__(kThreads) void fused_kernel(const Plan p, const flo
   // the transform and the LDS writes of the next one) goes into the gaps between two MFMAs
   // instead of before and after all 32 of them.
   auto interleave = [&]() {
-    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // the operands of the first four MFMAs
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);              // one MFMA
-      if (i < 14) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
-      if (i < 20) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global load
+      if (i < 8) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);   // two LDS reads
+      if (i >= 4 && i < 24) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global load
       __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);              // VALU
       if (i >= 24) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); // one LDS write
     }
@@ -367,7 +385,8 @@ __global__ __launch_bounds__(kThreads) void fused_kernel(const Plan p, const flo
   // one step: load chunk c + 4 into the set chunk c came from, multiply chunk c, stage chunk c + 1
 #define MN_WINO_STEP(c, buf, dk, uk, dn, un)  \
   fetch(dk, uk, (c) + 5 < nchunks);           \
-  multiply(buf);                              \
+  tail();                                     \
+  head(buf);                                  \
   stage((buf) ^ 1, dn, un);                   \
   interleave();                               \
   __syncthreads();
@@ -378,6 +397,7 @@ __global__ __launch_bounds__(kThreads) void fused_kernel(const Plan p, const flo
     MN_WINO_STEP(ch + 3, 1, d3, u3, d0, u0)
   }
 #undef MN_WINO_STEP
+  tail();
 
   // output transform: this lane's tile is t0 + wt + r, its outputs k0 + wk + row(v)
   const uint32_t etile = t0 + wt + r;
