@@ -764,7 +764,7 @@ static int run_fused(const Plan& p, const float* src, const float* w, bool flip,
     weight_kernel<false, true><<<(nu + kThreads - 1) / kThreads, kThreads, 0, s>>>(w, U, p.M, p.Mp, p.Cs);
   const uint32_t nkb = (uint32_t)(p.M + FK - 1) / FK, ntb = (p.T + FT - 1) / FT;
   if ((unsigned long long)nkb * ntb >= (1ull << 31) || !p.src_bytes || !p.u_bytes) return MN_EUNSUPPORTED;
-  if (!fused_lds_allowed()) return MN_ELAUNCH;
+  if (!fused_lds_allowed()) return MN_EUNSUPPORTED;  // this device does not grant 80 KB of LDS to a workgroup
   if (accum)
     fused_kernel<true><<<nkb * ntb, kThreads, kFusedLds, s>>>(p, src, U, bias, dst, nkb);
   else
