@@ -297,6 +297,18 @@ def conv_bench(steps, warmup):
 
     res = {"shape": c, "dtype": "f32", "flops_per_call": flops, "peak_TFLOP/s": MFMA_F32_PEAK_TFLOPS}
     res.update(directions(x, w, dy, MFMA_F32_PEAK_TFLOPS))
+    # one large-plane shape beside it (UNet batch 11, 128 -> 128 channels at 208 x 304), forward only:
+    # where the one-kernel Winograd variant is the fastest
+    u = dict(N=11, C=128, K=128, H=208, W=304)
+    xu = torch.randn(u["N"], u["C"], u["H"], u["W"], device=dev)
+    wu = torch.randn(u["K"], u["C"], 3, 3, device=dev) * (2.0 / (u["K"] * 9)) ** 0.5
+    flops = 2.0 * u["N"] * u["K"] * u["H"] * u["W"] * u["C"] * 9
+    res["unet_128ch_208x304"] = {"shape": u, "flops_per_call": flops}
+    for v in range(cv.n_fwd_algos(xu.dtype)):
+        res["unet_128ch_208x304"]["fwd_v%d" % v] = timed(
+            lambda: cv.conv_forward(xu, wu, None, 1, 1, 1, 1, v), MFMA_F32_PEAK_TFLOPS)
+    del xu, wu
+    flops = 2.0 * y.numel() * c["C"] * c["R"] * c["S"]
     # the same problem on bf16 channels-last tensors (bf16 matrix cores, fp32 accumulation)
     cl = lambda t: t.to(torch.bfloat16).contiguous(memory_format=torch.channels_last)
     res["bf16"] = {"layout": "channels-last", "peak_TFLOP/s": MFMA_BF16_PEAK_TFLOPS}
