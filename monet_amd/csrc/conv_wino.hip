@@ -754,6 +754,11 @@ static bool fused_lds_allowed() {
 
 static int run_fused(const Plan& p, const float* src, const float* w, bool flip, const float* bias,
                      float* dst, bool accum, void* ws, size_t ws_bytes, hipStream_t s) {
+  // every refusal comes before the first launch: a caller that falls back to another variant
+  // (and one that accumulates into dst) must find nothing done
+  const uint32_t nkb = (uint32_t)(p.M + FK - 1) / FK, ntb = (p.T + FT - 1) / FT;
+  if ((unsigned long long)nkb * ntb >= (1ull << 31) || !p.src_bytes || !p.u_bytes) return MN_EUNSUPPORTED;
+  if (!fused_lds_allowed()) return MN_EUNSUPPORTED;  // this device does not grant 80 KB of LDS to a workgroup
   const size_t need = u_floats(p) * sizeof(float);
   if (!ws || ws_bytes < need || !mn_aligned(ws, 16)) return MN_EINVAL;
   float* U = static_cast<float*>(ws);
@@ -762,9 +767,6 @@ static int run_fused(const Plan& p, const float* src, const float* w, bool flip,
     weight_kernel<true, true><<<(nu + kThreads - 1) / kThreads, kThreads, 0, s>>>(w, U, p.M, p.Mp, p.Cs);
   else
     weight_kernel<false, true><<<(nu + kThreads - 1) / kThreads, kThreads, 0, s>>>(w, U, p.M, p.Mp, p.Cs);
-  const uint32_t nkb = (uint32_t)(p.M + FK - 1) / FK, ntb = (p.T + FT - 1) / FT;
-  if ((unsigned long long)nkb * ntb >= (1ull << 31) || !p.src_bytes || !p.u_bytes) return MN_EUNSUPPORTED;
-  if (!fused_lds_allowed()) return MN_EUNSUPPORTED;  // this device does not grant 80 KB of LDS to a workgroup
   if (accum)
     fused_kernel<true><<<nkb * ntb, kThreads, kFusedLds, s>>>(p, src, U, bias, dst, nkb);
   else
