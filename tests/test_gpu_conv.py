@@ -431,3 +431,40 @@ def test_winograd_runs_slice_after_slice_when_its_buffers_would_pass_512_MB(cuda
     assert_rel(got, exp, TOL, "Winograd backward-weight in passes vs float64 samples")
     # the same call again gives the same bits (fixed order of slices and passes)
     assert torch.equal(dw2, conv_ops.conv_backward_weight(ws, dyd, xd, pad, 1, 1, 1, 2))
+
+
+def _random_winograd_shapes(count, seed):
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(count):
+        n = int(rng.integers(1, 4))
+        c = int(rng.choice([16, 32, 48, 64, 80]))
+        k = int(rng.choice([4, 16, 24, 64, 72, 130]))
+        h, w = int(rng.integers(4, 41)), int(rng.integers(4, 41))
+        pad = int(rng.integers(0, 3))
+        out.append(((n, c, h, w), (k, c, 3, 3), pad))
+    return out
+
+
+@pytest.mark.parametrize("xs,ws,pad", _random_winograd_shapes(16, 2024))
+def test_winograd_variants_on_random_shapes(cuda, xs, ws, pad):
+    """Both Winograd forms (through the workspace, in one kernel) in every direction they serve,
+    on shapes drawn at random: planes from 4 x 4 to 40 x 40 (ragged tiles, rows shorter than a
+    wavefront, tile blocks that span several images), outputs that do not fill a block of 64,
+    every padding; against the float64 oracle.  Backward-data also in its accumulating form."""
+    x, w, b = problem(xs, ws, 11)
+    exp = O.conv_fwd(x, w, b, 1, pad, 1)
+    dy = np.random.default_rng(12).standard_normal(exp.shape).astype(np.float32)
+    exp_dx = O.conv_bwd_data(dy, w, xs, 1, pad, 1)
+    exp_dw = O.conv_bwd_weight(dy, x, ws, 1, pad, 1)
+    xd, wd, bd, dyd = dev(x, cuda), dev(w, cuda), dev(b, cuda), dev(dy, cuda)
+    for v in (2, 3):
+        y = conv_ops.conv_forward(xd, wd, bd, pad, 1, 1, 1, v)
+        assert_rel(host(y), exp, TOL, f"forward variant {v} {xs} {ws} pad {pad}")
+        if ws[0] % 16 == 0:   # backward-data reduces over K
+            dx = conv_ops.conv_backward_input(xs, dyd, wd, pad, 1, 1, 1, v)
+            assert_rel(host(dx), exp_dx, TOL, f"backward-data variant {v} {xs} {ws} pad {pad}")
+        else:
+            assert refused(lambda: conv_ops.conv_backward_input(xs, dyd, wd, pad, 1, 1, 1, v))
+    dw = conv_ops.conv_backward_weight(ws, dyd, xd, pad, 1, 1, 1, 2)
+    assert_rel(host(dw), exp_dw, TOL, f"backward-weight variant 2 {xs} {ws} pad {pad}")
