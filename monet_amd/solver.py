@@ -426,6 +426,8 @@ class Model:
             raise ValueError("Model infeasible" if res.status == 2 else
                              f"no schedule found: {res.message}")
         self.last_excess = float(res.x[excess]) if excess is not None else 0.0
+        # how far the incumbent may be from the optimum (large when the time limit ended the search)
+        self.last_gap = float(getattr(res, "mip_gap", float("nan")))
         if excess is not None and \
                 self.budget + res.x[excess] > self.accept_up_to * (1.0 + EXCESS_TOLERANCE):
             raise ValueError("Model infeasible: the cheapest schedule found needs %.3f GB, budget "
@@ -449,6 +451,7 @@ class Model:
         if excess is not None:  # without what an accepted overshoot of the target was charged
             run_time -= float(cvec[excess] * res.x[excess])
         solution = Solution(r, s, m, rf, ip, pp, solve_time, float("nan"), float("nan"), run_time)
+        solution.mip_gap = self.last_gap
         if out_file is not None:
             with open(out_file, 'wb') as f:
                 pickle.dump([si, solution], f)
@@ -463,10 +466,12 @@ def solve_within_budget(si, budget, time_limit=86400, solver="HIGHS", ablation=F
     a slightly LOWER target with a MODERATE price on the overshoot - any schedule is then an
     acceptable incumbent and the price steers the search - and tightens the target until a
     schedule fits the real budget.  What comes out fits the budget; it need not be optimal."""
-    per_solve = max(30.0, time_limit / (rounds + 1.0))
+    # the plain model gets the larger share: an incumbent it returns at its time limit is
+    # accepted as it is, however far from the optimum (the achieved gap is reported)
+    first = max(30.0, 0.6 * time_limit) if rounds else time_limit
+    per_solve = max(30.0, (time_limit - first) / max(rounds, 1))
     try:
-        return Model(si, budget, per_solve if rounds else time_limit, solver, ablation,
-                     **options).solve(out_file=out_file)
+        return Model(si, budget, first, solver, ablation, **options).solve(out_file=out_file)
     except ValueError as e:
         if "cheapest schedule found" not in str(e) or not rounds:
             raise
@@ -551,8 +556,12 @@ def main(argv=None):
                                    out_file=str(out), rounds=args.rounds, mip_rel_gap=args.gap,
                                    verbose=args.verbose,
                                    recompute_window=args.window)
-    print("solved in %.1f s, expected run time %.2f ms -> %s" % (
-        solution.solve_time, solution.runtime_expected / CPU_GCD_MULTIPLIER, out))
+    gap = getattr(solution, "mip_gap", float("nan"))
+    print("solved in %.1f s, expected run time %.2f ms, gap %.2f %% -> %s" % (
+        solution.solve_time, solution.runtime_expected / CPU_GCD_MULTIPLIER, 100.0 * gap, out))
+    if gap == gap and gap > max(0.05, 10.0 * args.gap):
+        print("warning: the search ended at its time limit %.0f %% above the best bound; "
+              "a longer --time_limit (or --rounds 0) may find a cheaper schedule" % (100.0 * gap))
     return solution
 
 
