@@ -333,8 +333,10 @@ typedef struct mn_conv2d {
  *                      registers until the output transform, so the only
  *                      workspace is the transformed weights (16 * C *
  *                      pad128(K) floats; the role of the reference's fused
- *                      WINOGRAD slot).  Same shapes as variant 2; faster than
- *                      it where channels are few and planes large
+ *                      WINOGRAD slot).  Same shapes as variant 2, tensors
+ *                      below 2 GB (MN_EUNSUPPORTED otherwise, and on a device
+ *                      that does not grant a workgroup 80 KB of LDS); faster
+ *                      than variant 2 where channels are few and planes large
  *   backward-data    0 implicit GEMM reading the weights through strides
  *                    1 same with the weights repacked [tap][k][c] (c padded
  *                      to a multiple of 128) into the workspace; may split
