@@ -296,10 +296,16 @@ typedef struct mn_conv2d {
  * cores with fp32 accumulation and rounded once (to nearest even) on output.
  * Needs channel counts that are multiples of 32 on the reduction side
  * (forward: C; backward-data: K) and multiples of 64 for backward-weight (C and
- * K); otherwise MN_EUNSUPPORTED.  Variants 0 and 1 of a direction run the
- * same kernel, further variants are fp32 only; backward-data always needs K*C*R*S*2 bytes of workspace (the
- * transposed weights) and backward-weight its fp32 split partials - ask
- * mn_conv_ws_bytes.  The reference has no reduced-precision path; this dtype
+ * K); otherwise MN_EUNSUPPORTED.  Two variants per direction, further ones
+ * are fp32 only.  Forward and backward-data multiply pixel tiles staged in
+ * LDS with weight fragments that every wavefront loads straight into the
+ * registers the matrix instruction reads: variant 0 reads them from the
+ * weight rows where they lie (forward: no workspace; backward-data: the
+ * transposed weights, K*C*R*S*2 bytes), variant 1 from a copy packed in
+ * fragment order in the workspace (rows padded to 32: one contiguous KB per
+ * fragment instead of 32 pieces of 32 bytes; 1.6 times faster at the
+ * ResNet-50 layer3 shape).  Backward-weight: both variants run one kernel
+ * with fp32 split partials in the workspace - ask mn_conv_ws_bytes.  The reference has no reduced-precision path; this dtype
  * serves the bf16 configuration of the layer3 benchmark. */
 #define MN_BF16 1
 
@@ -337,6 +343,20 @@ typedef struct mn_conv2d {
  *                      below 2 GB (MN_EUNSUPPORTED otherwise, and on a device
  *                      that does not grant a workgroup 80 KB of LDS); faster
  *                      than variant 2 where channels are few and planes large
+ *                    4 fp32 on the bf16 matrix cores: every fp32 operand is cut
+ *                      into three bf16 slices (x = x0 + x1 + x2, the remainders
+ *                      exact) and the six slice products down to 2^-16 of the
+ *                      full product are accumulated in fp32, which keeps fp32
+ *                      accuracy (measured 1e-7..5e-7 of the output's scale,
+ *                      like the fp32 matrix instruction) at 3/8 of its matrix
+ *                      time.  1x1 filters, stride 1, no padding, H*W a
+ *                      multiple of 4, C a multiple of 16, tensors below 2 GB
+ *                      (MN_EUNSUPPORTED otherwise, and for MN_BF16).
+ *                      Workspace: the three slices of the weights, rows padded
+ *                      to 256 (3 * pad256(K) * C * 2 bytes).  Non-finite inputs
+ *                      give NaN.  Takes the place of the reference's slots
+ *                      that trade workspace for time on shapes Winograd cannot
+ *                      take (monet/lm_ops/conv.cpp:21-46)
  *   backward-data    0 implicit GEMM reading the weights through strides
  *                    1 same with the weights repacked [tap][k][c] (c padded
  *                      to a multiple of 128) into the workspace; may split
@@ -346,6 +366,9 @@ typedef struct mn_conv2d {
  *                    2 Winograd F(2x2, 3x3), as for the forward (the filter
  *                      rotated by 180 degrees, channel roles swapped)
  *                    3 the one-kernel Winograd form, as for the forward
+ *                    4 three bf16 slices per operand, as for the forward (K
+ *                      a multiple of 16; the weights are transposed as they
+ *                      are split)
  *   backward-weight  0 split reduction combined with atomics into a cleared dw
  *                    1 split reduction through per-split partials in the
  *                      workspace, then a fixed-order sum (reproducible)
@@ -357,10 +380,8 @@ typedef struct mn_conv2d {
  *                      passes added in order) plus the partial results;
  *                      reproducible */
 int mn_conv_n_variants(int direction);
-/* The same per dtype: the list above for MN_F32; 1 for MN_BF16 (one kernel and
- * one memory tier per direction - index 1 is accepted as an alias of 0 so that
- * an fp32 schedule's choice still runs); 0 for an unknown dtype.  The
- * reference is fp32 only and has no counterpart. */
+/* The same per dtype: the list above for MN_F32; 2 for MN_BF16 (see MN_BF16);
+ * 0 for an unknown dtype.  The reference is fp32 only and has no counterpart. */
 int mn_conv_n_variants_for(int direction, int dtype);
 /* Workspace bytes a (direction, variant, dtype) needs for this geometry
  * (role of the cudnnGet*WorkspaceSize queries at conv.cpp:314-324). */

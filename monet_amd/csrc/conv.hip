@@ -39,13 +39,19 @@ int mn_wino_bwd_weight(const mn_conv2d* g, const float* dy, const float* x, floa
                        void* ws, size_t ws_bytes, hipStream_t s);
 
 // bf16 / channels-last kernels (conv_bf16.hip)
-int mn_conv16_ws_bytes(const mn_conv2d* g, int direction, size_t* bytes);
+int mn_conv16_ws_bytes(const mn_conv2d* g, int direction, int variant, size_t* bytes);
 int mn_conv16_fwd(const mn_conv2d* g, const void* x, const void* w, const void* bias, void* y,
-                  hipStream_t s);
+                  void* ws, size_t ws_bytes, int variant, hipStream_t s);
 int mn_conv16_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void* dx, void* ws,
-                       size_t ws_bytes, hipStream_t s);
+                       size_t ws_bytes, int variant, hipStream_t s);
 int mn_conv16_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, void* dw, void* ws,
-                         size_t ws_bytes, hipStream_t s);
+                         size_t ws_bytes, int variant, hipStream_t s);
+
+// fp32 through three bf16 slices per operand (conv_split.hip)
+int mn_split_ws_bytes(const mn_conv2d* g, int direction, size_t* bytes);
+int mn_split_pointwise(const mn_conv2d* g, int direction, const float* in, const float* w,
+                       const float* bias, float* out, bool accumulate, void* ws, size_t ws_bytes,
+                       hipStream_t s);
 
 namespace mn_conv {
 
@@ -1375,9 +1381,9 @@ extern "C" {
 int mn_conv_n_variants(int direction) {
   switch (direction) {
     case MN_CONV_FWD:
-      return 4;
+      return 5;
     case MN_CONV_BWD_DATA:
-      return 4;
+      return 5;
     case MN_CONV_BWD_WEIGHT:
       return 3;
     default:
@@ -1387,8 +1393,8 @@ int mn_conv_n_variants(int direction) {
 
 int mn_conv_n_variants_for(int direction, int dtype) {
   if (dtype == MN_F32) return mn_conv_n_variants(direction);
-  // bf16: one kernel per direction, a single memory tier
-  if (dtype == MN_BF16) return mn_conv_n_variants(direction) > 0 ? 1 : 0;
+  // bf16: two tiers per direction (conv_bf16.hip)
+  if (dtype == MN_BF16) return mn_conv_n_variants(direction) > 0 ? 2 : 0;
   return 0;
 }
 
@@ -1399,13 +1405,14 @@ int mn_conv_ws_bytes(const mn_conv2d* g, int direction, int variant, int dtype, 
   const int st = check(g);
   if (st != MN_OK) return st;
   if (variant < 0 || variant >= mn_conv_n_variants(direction)) return MN_EUNSUPPORTED;
-  if (dtype == MN_BF16)  // variants 0 and 1 are one kernel; there is no bf16 Winograd tier
-    return variant <= 1 ? mn_conv16_ws_bytes(g, direction, bytes) : MN_EUNSUPPORTED;
+  if (dtype == MN_BF16)  // there is no bf16 Winograd tier
+    return variant <= 1 ? mn_conv16_ws_bytes(g, direction, variant, bytes) : MN_EUNSUPPORTED;
   if (dtype != MN_F32) return MN_EUNSUPPORTED;
   if (variant == 2)
     return direction == MN_CONV_BWD_WEIGHT ? mn_wino_bwd_weight_ws_bytes(g, bytes)
                                            : mn_wino_ws_bytes(g, direction == MN_CONV_BWD_DATA, bytes);
   if (variant == 3) return mn_wino_fused_ws_bytes(g, direction == MN_CONV_BWD_DATA, bytes);
+  if (variant == 4) return mn_split_ws_bytes(g, direction, bytes);
   const size_t wsize = (size_t)g->K * g->C * g->R * g->S * sizeof(float);
   // variant 1 of the gather directions: the repacked weight operand (rows padded to 128)
   if (direction == MN_CONV_FWD && variant == 1)
@@ -1426,10 +1433,10 @@ int mn_conv_fwd(const mn_conv2d* g, const void* x, const void* w, const void* bi
   using namespace mn_conv;
   const int st = check(g);
   if (st != MN_OK) return st;
-  if (variant < 0 || variant > 3 || (variant >= 2 && dtype != MN_F32)) return MN_EUNSUPPORTED;
+  if (variant < 0 || variant > 4 || (variant >= 2 && dtype != MN_F32)) return MN_EUNSUPPORTED;
   if (g->N == 0) return MN_OK;
   if (!x || !w || !y) return MN_EINVAL;
-  if (dtype == MN_BF16) return mn_conv16_fwd(g, x, w, bias, y, mn_stream(stream));
+  if (dtype == MN_BF16) return mn_conv16_fwd(g, x, w, bias, y, ws, ws_bytes, variant, mn_stream(stream));
   if (dtype != MN_F32) return MN_EUNSUPPORTED;
   if (variant == 2)
     return mn_wino_fwd(g, (const float*)x, (const float*)w, (const float*)bias, (float*)y, ws,
@@ -1437,6 +1444,9 @@ int mn_conv_fwd(const mn_conv2d* g, const void* x, const void* w, const void* bi
   if (variant == 3)
     return mn_wino_fused_fwd(g, (const float*)x, (const float*)w, (const float*)bias, (float*)y, ws,
                              ws_bytes, mn_stream(stream));
+  if (variant == 4)
+    return mn_split_pointwise(g, MN_CONV_FWD, (const float*)x, (const float*)w, (const float*)bias,
+                              (float*)y, false, ws, ws_bytes, mn_stream(stream));
   Gather q = {};
   q.M = g->K;
   q.T = g->R * g->S;
@@ -1492,17 +1502,20 @@ static int conv_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void
   using namespace mn_conv;
   const int st = check(g);
   if (st != MN_OK) return st;
-  if (variant < 0 || variant > 3 || (variant >= 2 && dtype != MN_F32)) return MN_EUNSUPPORTED;
+  if (variant < 0 || variant > 4 || (variant >= 2 && dtype != MN_F32)) return MN_EUNSUPPORTED;
   if (g->N == 0) return MN_OK;
   if (!dy || !w || !dx) return MN_EINVAL;
   hipStream_t s = mn_stream(stream);
   if (dtype == MN_BF16)
-    return accum ? MN_EUNSUPPORTED : mn_conv16_bwd_data(g, dy, w, dx, ws, ws_bytes, s);
+    return accum ? MN_EUNSUPPORTED : mn_conv16_bwd_data(g, dy, w, dx, ws, ws_bytes, variant, s);
   if (dtype != MN_F32) return MN_EUNSUPPORTED;
   if (variant == 2)
     return mn_wino_bwd_data(g, (const float*)dy, (const float*)w, (float*)dx, accum, ws, ws_bytes, s);
   if (variant == 3)
     return mn_wino_fused_bwd_data(g, (const float*)dy, (const float*)w, (float*)dx, accum, ws, ws_bytes, s);
+  if (variant == 4)
+    return mn_split_pointwise(g, MN_CONV_BWD_DATA, (const float*)dy, (const float*)w, nullptr,
+                              (float*)dx, accum, ws, ws_bytes, s);
   const int RS = g->R * g->S;
   const float* a = (const float*)w;
   uint32_t a_bytes = weight_bytes(g);  // size of the A operand: the weights, or their repacked copy
@@ -1612,7 +1625,7 @@ static int conv_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, vo
     if (db_out) return MN_EUNSUPPORTED;     // the bf16 kernel has no bias-gradient epilogue
     if (g->N == 0) return MN_EUNSUPPORTED;  // nothing to reduce: the caller clears dw itself
     if (!dy || !x) return MN_EINVAL;
-    return mn_conv16_bwd_weight(g, dy, x, dw, ws, ws_bytes, s);
+    return mn_conv16_bwd_weight(g, dy, x, dw, ws, ws_bytes, variant, s);
   }
   if (db_out && !mn_aligned(db_out, 4)) return MN_EINVAL;
   const size_t nw = (size_t)g->K * g->C * g->R * g->S;

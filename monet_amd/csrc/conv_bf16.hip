@@ -89,18 +89,27 @@ struct GatherH {
   int DH, DW, osh, osw, oh0, ow0;  // dst [N, DH, DW, Nout], position = oh*osh + oh0
   int T;                  // taps of this launch
   uint32_t wrow;          // elements between consecutive weight rows
+  uint32_t wstep;         // bytes between consecutive 16-deep steps of the weight operand: 32 for
+                          // rows in place, 1024 for the fragment-packed layout
   uint32_t src_bytes, w_bytes;  // sizes of the two operand tensors (set by the launcher)
   int16_t dh[kMaxTaps], dw[kMaxTaps];
   int32_t woff[kMaxTaps]; // element offset of tap t inside a weight row
 };
 
-// DEPTH = reduction elements staged per barrier.
-// A bf16 matrix instruction is short (a workgroup tile of 128 x 128 x 32 is 8 of them per
-// wavefront, ~256 cycles), so anything else a wavefront has to issue per tile shows directly,
-// and a load must be in flight for more than one tile to be hidden.  Hence:
-//  * operands are fetched with raw buffer loads: the per-thread byte offset of a row is fixed
-//    for a whole tap (a row outside the window or the tensor gets an offset beyond the buffer
-//    and reads as zero: no masks when staging), the per-tile part (channel offset) is the
+// The channel operand (weights) never passes through LDS: every wavefront loads the fragments
+// of its own 32-channel blocks straight from global memory into the registers the matrix
+// instruction reads (a lane's fragment is 16 contiguous bytes of one weight row), one
+// 64-deep tile ahead of their use.  Only the pixel operand (gathered rows, shared by the
+// wavefronts of a workgroup row) is staged in LDS.  That halves the LDS traffic per matrix
+// instruction, which is what bounded a kernel that staged both operands (a 128 x 128 x 32
+// tile is 8 instructions = 256 cycles per wavefront, and read 32 KB + wrote 16 KB of LDS).
+// The weights come in one of two layouts, told apart by `wstep`:
+//  * in place ([rows][reduction], wstep = 32): a fragment load touches 32 rows, 32 bytes each;
+//  * packed ([32-row block][16-deep step][lane], wstep = 1024): a fragment is 1 KB contiguous.
+// Everything else a wavefront issues per tile is kept small:
+//  * the pixel operand is fetched with raw buffer loads: the per-thread byte offset of a row is
+//    fixed for a whole tap (a row outside the window or the tensor gets an offset beyond the
+//    buffer and reads as zero: no masks when staging), the per-tile part (channel offset) is the
 //    scalar offset of the instruction: no vector arithmetic per tile;
 //  * two register sets: the loads of tile t+2 are issued before tile t is multiplied and
 //    are staged during tile t+1.
@@ -111,13 +120,13 @@ __global__ __launch_bounds__(kThreads) void gather_bf16_kernel(const GatherH g,
                                                                const bf16_t* __restrict__ bias,
                                                                bf16_t* __restrict__ dst) {
   constexpr int TN = BN / 64;                 // MFMA tiles per wavefront along the columns
+  constexpr int KS = DEPTH / 16;              // matrix steps per staged tile
   constexpr int kCPR = DEPTH / 8;             // 16-byte chunks per staged row
   constexpr int kRPP = kThreads / kCPR;       // rows covered by one pass of the workgroup
-  constexpr int kARows = BM / kRPP, kBRows = BN / kRPP;  // chunks per thread
+  constexpr int kARows = BM / kRPP;           // chunks per thread
   constexpr int LDR = DEPTH + 8;              // LDS row length (elements): 80 or 144 bytes
   constexpr uint32_t kBeyond = 0x80000000u;   // byte offset past any buffer (tensors are < 2 GB)
   __shared__ __attribute__((aligned(16))) bf16_t lds_a[2][BM][LDR];
-  __shared__ __attribute__((aligned(16))) bf16_t lds_b[2][BN][LDR];
   __shared__ int tdh[kMaxTaps], tdw[kMaxTaps], twoff[kMaxTaps];
   __shared__ uint32_t row_dst[BM];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -160,12 +169,16 @@ __global__ __launch_bounds__(kThreads) void gather_bf16_kernel(const GatherH g,
     ows[i] = ow * g.isw;
     abase[i] = n * (uint32_t)g.Hs * g.Ws;
   }
-  // B loader: chunk `chunk` of weight rows n0 + arow + kRPP*i; byte offsets, fixed for the launch
-  uint32_t b_off[kBRows];
+  // weight fragments of this wavefront's column blocks: per-lane byte offset, fixed for the launch
+  uint32_t b_off[TN];
 #pragma unroll
-  for (int i = 0; i < kBRows; ++i) {
-    const int col = n0 + arow + kRPP * i;
-    b_off[i] = col < g.Nout ? ((uint32_t)col * g.wrow + chunk * 8) * 2u : kBeyond;
+  for (int j = 0; j < TN; ++j) {
+    const int blk = (n0 + wn * (BN / 2) + 32 * j) / 32;   // 32-row block of the weight operand
+    const int col = blk * 32 + (lane & 31);
+    if (g.wstep == 1024)
+      b_off[j] = ((uint32_t)blk * (g.wrow / 16) * 64 + lane) * 16u;
+    else
+      b_off[j] = col < g.Nout ? ((uint32_t)col * g.wrow + (lane >> 5) * 8) * 2u : kBeyond;
   }
   __syncthreads();
 
@@ -173,10 +186,8 @@ __global__ __launch_bounds__(kThreads) void gather_bf16_kernel(const GatherH g,
       __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(src), 0, g.src_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t w_buf =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(w), 0, g.w_bytes, 0x00020000);
-  // per-tap state: byte offsets of this thread's rows of the source (or kBeyond), and the
-  // uniform byte offset of the tap inside a weight row
+  // per-tap state: byte offsets of this thread's rows of the source (or kBeyond)
   uint32_t a_off[kARows];
-  int w_tap = 0;
   auto enter_tap = [&](int t) {  // t uniform
     const int dh = tdh[t], dw = tdw[t];
 #pragma unroll
@@ -185,23 +196,16 @@ __global__ __launch_bounds__(kThreads) void gather_bf16_kernel(const GatherH g,
       const bool ok = aok[i] && (unsigned)hh < (unsigned)g.Hs && (unsigned)ww < (unsigned)g.Ws;
       a_off[i] = ok ? ((abase[i] + hh * g.Ws + ww) * (uint32_t)g.Cs + chunk * 8) * 2u : kBeyond;
     }
-    w_tap = __builtin_amdgcn_readfirstlane(twoff[t]) * 2;
   };
-  auto fetch = [&](uint4_t (&ra)[kARows], uint4_t (&rb)[kBRows], int c0) {  // c0 uniform
+  auto fetch = [&](uint4_t (&ra)[kARows], int c0) {  // c0 uniform
 #pragma unroll
     for (int i = 0; i < kARows; ++i)
       ra[i] = __builtin_amdgcn_raw_buffer_load_b128(src_buf, a_off[i], c0 * 2, 0);
-#pragma unroll
-    for (int i = 0; i < kBRows; ++i)
-      rb[i] = __builtin_amdgcn_raw_buffer_load_b128(w_buf, b_off[i], w_tap + c0 * 2, 0);
   };
-  auto stage = [&](int buf, const uint4_t (&ra)[kARows], const uint4_t (&rb)[kBRows]) {
+  auto stage = [&](int buf, const uint4_t (&ra)[kARows]) {
 #pragma unroll
     for (int i = 0; i < kARows; ++i)
       *reinterpret_cast<uint4_t*>(&lds_a[buf][arow + kRPP * i][chunk * 8]) = ra[i];
-#pragma unroll
-    for (int i = 0; i < kBRows; ++i)
-      *reinterpret_cast<uint4_t*>(&lds_b[buf][arow + kRPP * i][chunk * 8]) = rb[i];
   };
 
   float16_t acc[2][TN];
@@ -215,8 +219,14 @@ __global__ __launch_bounds__(kThreads) void gather_bf16_kernel(const GatherH g,
   const int per_tap = g.Cs / DEPTH;
   const int ktiles = g.T * per_tap;
   if (ktiles > 0) {
-    uint4_t ra0[kARows], rb0[kBRows], ra1[kARows], rb1[kBRows];
-    int t = 0, c0 = 0;  // position of the next tile to fetch
+    uint4_t ra0[kARows], ra1[kARows];
+    // weight fragments of the two tiles in flight: set b holds the tile that LDS buffer b holds;
+    // a step's fragments are reloaded with those of the tile after next as soon as it is done.
+    // Loads complete in issue order, so every operand is fetched the same distance (two tiles)
+    // ahead: a deeper prefetch of one operand would only make the waits for the other longer
+    uint4_t bq[2][KS][TN];
+    int t = 0, c0 = 0;    // position of the next pixel tile to fetch
+    int tb = 0, cb = 0;   // position of the next weight tile to fetch
     enter_tap(0);
     auto advance = [&]() {
       c0 += DEPTH;
@@ -226,34 +236,74 @@ __global__ __launch_bounds__(kThreads) void gather_bf16_kernel(const GatherH g,
         if (t < g.T) enter_tap(t);
       }
     };
-    fetch(ra0, rb0, c0);  // tile 0
+    // uniform byte offset of weight tile (tb, cb), then move to the next tile (the last tile is
+    // loaded again instead of branching around the loads)
+    auto wtile = [&]() {
+      const uint32_t k16 = (uint32_t)(__builtin_amdgcn_readfirstlane(twoff[tb]) + cb) / 16u;
+      if (tb * per_tap * DEPTH + cb + DEPTH < ktiles * DEPTH) {
+        cb += DEPTH;
+        if (cb == g.Cs) {
+          cb = 0;
+          ++tb;
+        }
+      }
+      return k16 * g.wstep;
+    };
+    auto wfetch = [&](uint4_t (&b)[KS][TN], uint32_t woff) {
+#pragma unroll
+      for (int s = 0; s < KS; ++s)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          b[s][j] = __builtin_amdgcn_raw_buffer_load_b128(w_buf, b_off[j], woff + s * g.wstep, 0);
+    };
+    auto mma_tile = [&](int buf, uint4_t (&b)[KS][TN], uint32_t wnext) {
+      const int r = lane & 31, kq = (lane >> 5) * 8;
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        bf16x8 af[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+          af[i] = *reinterpret_cast<const bf16x8*>(&lds_a[buf][wm * 64 + 32 * i + r][s * 16 + kq]);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const bf16x8 bfr = __builtin_bit_cast(bf16x8, b[s][j]);
+#pragma unroll
+          for (int i = 0; i < 2; ++i)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr, acc[i][j], 0, 0, 0);
+          b[s][j] = __builtin_amdgcn_raw_buffer_load_b128(w_buf, b_off[j], wnext + s * g.wstep, 0);
+        }
+      }
+    };
+    wfetch(bq[0], wtile());   // tile 0
+    fetch(ra0, c0);
     advance();
+    wfetch(bq[1], wtile());   // tile 1 (tile 0 again if there is only one)
     if (ktiles > 1) {
-      fetch(ra1, rb1, c0);  // tile 1
+      fetch(ra1, c0);
       advance();
     }
-    stage(0, ra0, rb0);
+    stage(0, ra0);
     __syncthreads();
     for (int kt = 0; kt + 1 < ktiles; kt += 2) {
       // tile kt is in LDS buffer 0, tile kt+1 in flight in set 1
       if (kt + 2 < ktiles) {
-        fetch(ra0, rb0, c0);
+        fetch(ra0, c0);
         advance();
       }
-      mma_tile<2, TN, BM, BN, DEPTH>(lds_a[0], lds_b[0], wm, wn, lane, acc);
-      stage(1, ra1, rb1);
+      mma_tile(0, bq[0], wtile());
+      stage(1, ra1);
       __syncthreads();
       // tile kt+1 is in LDS buffer 1, tile kt+2 in flight in set 0
       if (kt + 3 < ktiles) {
-        fetch(ra1, rb1, c0);
+        fetch(ra1, c0);
         advance();
       }
-      mma_tile<2, TN, BM, BN, DEPTH>(lds_a[1], lds_b[1], wm, wn, lane, acc);
-      if (kt + 2 < ktiles) stage(0, ra0, rb0);
+      mma_tile(1, bq[1], wtile());
+      if (kt + 2 < ktiles) stage(0, ra0);
       __syncthreads();
     }
     // an odd number of tiles: the last one was staged into buffer 0
-    if (ktiles & 1) mma_tile<2, TN, BM, BN, DEPTH>(lds_a[0], lds_b[0], wm, wn, lane, acc);
+    if (ktiles & 1) mma_tile(0, bq[0], wtile());
   }
 
   // epilogue: for a fixed register, lanes 0..31 hold 32 consecutive channels of one position
@@ -271,6 +321,41 @@ __global__ __launch_bounds__(kThreads) void gather_bf16_kernel(const GatherH g,
       }
     }
   }
+}
+
+// Weight operand in fragment order: wp[(blk * steps + s) * 64 + lane] (16-byte units) = the 8
+// elements rows[blk * 32 + lane % 32][s * 16 + (lane / 32) * 8 ...] of a [rows][len] matrix
+// (rows beyond the matrix are zero).  With transposed == 0 the matrix is the weight tensor
+// itself (rows = K, len = T * C); with transposed == 1 it is wt[c][t * K + k] = w[k][t][c]
+// (rows = C, len = T * K), the operand of backward-data.
+__global__ __launch_bounds__(kThreads) void pack_weights_bf16_kernel(
+    const bf16_t* __restrict__ w, bf16_t* __restrict__ wp, int K, int C, int T, int transposed) {
+  const int rows = transposed ? C : K, len = T * (transposed ? K : C);
+  const int steps = len / 16, blocks = (rows + 31) / 32;
+  const size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x;   // 16-byte unit
+  if (i >= (size_t)blocks * steps * 64) return;
+  const int lane = (int)(i % 64);
+  const size_t bs = i / 64;
+  const int s = (int)(bs % steps), blk = (int)(bs / steps);
+  const int row = blk * 32 + (lane & 31), k0 = s * 16 + (lane >> 5) * 8;
+  bf16_t v[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    bf16_t x = 0;
+    if (row < rows) {
+      if (!transposed) {
+        x = w[(size_t)row * len + k0 + e];
+      } else {
+        const int t = (k0 + e) / K, k = (k0 + e) - t * K;
+        x = w[((size_t)k * T + t) * C + row];
+      }
+    }
+    v[e] = x;
+  }
+  uint4_t o;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) o[e] = (uint32_t)v[2 * e] | ((uint32_t)v[2 * e + 1] << 16);
+  reinterpret_cast<uint4_t*>(wp)[i] = o;
 }
 
 // wt[(c*T + t)*K + k] = w[(k*T + t)*C + c]
@@ -496,20 +581,38 @@ static int launch_gather16(GatherH q, const bf16_t* src, const bf16_t* w, const 
   // the kernel addresses its operands through buffer descriptors with byte offsets below 2^31
   const unsigned long long n_img = q.npix / ((unsigned long long)q.OH * q.OW);
   const unsigned long long src_bytes = n_img * q.Hs * q.Ws * q.Cs * 2ull;
-  const unsigned long long w_bytes = (unsigned long long)q.Nout * q.wrow * 2ull;
+  const unsigned long long w_rows = q.wstep == 1024 ? (q.Nout + 31) / 32 * 32ull : (unsigned long long)q.Nout;
+  const unsigned long long w_bytes = w_rows * q.wrow * 2ull;
   if (src_bytes >= (1ull << 31) || w_bytes >= (1ull << 31)) return MN_EUNSUPPORTED;
   q.src_bytes = (uint32_t)src_bytes;
   q.w_bytes = (uint32_t)w_bytes;
-  // 32-deep staging: 64-deep tiles (half as many barriers) measured 10 % slower at the
-  // ResNet-50 layer3 shape because their LDS footprint halves the resident workgroups
+  const bool deep = q.Cs % 64 == 0;
   if (q.Nout % 128 == 0) {
     dim3 grid((q.npix + BM - 1) / BM, q.Nout / 128);
-    gather_bf16_kernel<128, 32><<<grid, kThreads, 0, s>>>(q, src, w, bias, dst);
+    if (deep)
+      gather_bf16_kernel<128, 64><<<grid, kThreads, 0, s>>>(q, src, w, bias, dst);
+    else
+      gather_bf16_kernel<128, 32><<<grid, kThreads, 0, s>>>(q, src, w, bias, dst);
   } else {
     dim3 grid((q.npix + BM - 1) / BM, (q.Nout + 63) / 64);
-    gather_bf16_kernel<64, 32><<<grid, kThreads, 0, s>>>(q, src, w, bias, dst);
+    if (deep)
+      gather_bf16_kernel<64, 64><<<grid, kThreads, 0, s>>>(q, src, w, bias, dst);
+    else
+      gather_bf16_kernel<64, 32><<<grid, kThreads, 0, s>>>(q, src, w, bias, dst);
   }
   return MN_OK;
+}
+
+// bytes of the fragment-packed weight operand of a gather direction
+static size_t packed_weight_bytes(const mn_conv2d* g, bool transposed) {
+  const size_t rows = transposed ? g->C : g->K, len = (size_t)g->R * g->S * (transposed ? g->K : g->C);
+  return (rows + 31) / 32 * 32 * len * sizeof(bf16_t);
+}
+
+static void pack_weights(const mn_conv2d* g, const bf16_t* w, bf16_t* wp, bool transposed, hipStream_t s) {
+  const size_t units = packed_weight_bytes(g, transposed) / 16;
+  pack_weights_bf16_kernel<<<(unsigned)((units + kThreads - 1) / kThreads), kThreads, 0, s>>>(
+      w, wp, g->K, g->C, g->R * g->S, transposed ? 1 : 0);
 }
 
 static void wgrad16_tiles(const mn_conv2d* g, int* bm, int* bn) {
@@ -536,15 +639,21 @@ static void wgrad16_split(const mn_conv2d* g, int* splits, int* tiles_per_split)
 }  // namespace mn_conv16
 
 // Entry points used by the dtype dispatch in conv.hip.
-int mn_conv16_ws_bytes(const mn_conv2d* g, int direction, size_t* bytes) {
+int mn_conv16_ws_bytes(const mn_conv2d* g, int direction, int variant, size_t* bytes) {
   using namespace mn_conv16;
   *bytes = 0;
   const int st = check16(g);
   if (st != MN_OK) return st;
-  if (direction == MN_CONV_FWD) return g->C % BK == 0 ? MN_OK : MN_EUNSUPPORTED;
+  if (variant < 0 || variant > 1) return MN_EUNSUPPORTED;
+  if (direction == MN_CONV_FWD) {
+    if (g->C % BK != 0) return MN_EUNSUPPORTED;
+    if (variant == 1) *bytes = packed_weight_bytes(g, false);
+    return MN_OK;
+  }
   if (direction == MN_CONV_BWD_DATA) {
     if (g->K % BK != 0) return MN_EUNSUPPORTED;
-    *bytes = (size_t)g->K * g->C * g->R * g->S * sizeof(bf16_t);
+    *bytes = variant == 1 ? packed_weight_bytes(g, true)
+                          : (size_t)g->K * g->C * g->R * g->S * sizeof(bf16_t);
     return MN_OK;
   }
   if (g->K % 64 != 0 || g->C % 64 != 0) return MN_EUNSUPPORTED;
@@ -555,13 +664,20 @@ int mn_conv16_ws_bytes(const mn_conv2d* g, int direction, size_t* bytes) {
 }
 
 int mn_conv16_fwd(const mn_conv2d* g, const void* x, const void* w, const void* bias, void* y,
-                  hipStream_t s) {
+                  void* ws, size_t ws_bytes, int variant, hipStream_t s) {
   using namespace mn_conv16;
   const int st = check16(g);
   if (st != MN_OK) return st;
-  if (g->C % BK != 0) return MN_EUNSUPPORTED;
+  if (g->C % BK != 0 || variant < 0 || variant > 1) return MN_EUNSUPPORTED;
   if (!mn_aligned(x, 16) || !mn_aligned(w, 16)) return MN_EINVAL;
   GatherH q = {};
+  q.wstep = 32;
+  if (variant == 1) {   // weights in fragment order in the workspace
+    if (!ws || ws_bytes < packed_weight_bytes(g, false) || !mn_aligned(ws, 16)) return MN_EINVAL;
+    pack_weights(g, (const bf16_t*)w, (bf16_t*)ws, false, s);
+    w = ws;
+    q.wstep = 1024;
+  }
   q.npix = (uint32_t)((long long)g->N * g->P * g->Q);
   q.OH = g->P;
   q.OW = g->Q;
@@ -589,17 +705,20 @@ int mn_conv16_fwd(const mn_conv2d* g, const void* x, const void* w, const void* 
 }
 
 int mn_conv16_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void* dx, void* ws,
-                       size_t ws_bytes, hipStream_t s) {
+                       size_t ws_bytes, int variant, hipStream_t s) {
   using namespace mn_conv16;
   const int st = check16(g);
   if (st != MN_OK) return st;
-  if (g->K % BK != 0) return MN_EUNSUPPORTED;
+  if (g->K % BK != 0 || variant < 0 || variant > 1) return MN_EUNSUPPORTED;
   const int T = g->R * g->S;
   const size_t nw = (size_t)g->K * g->C * T;
-  if (!ws || ws_bytes < nw * sizeof(bf16_t) || !mn_aligned(ws, 16) || !mn_aligned(dy, 16))
-    return MN_EINVAL;
-  transpose_weights_bf16_kernel<<<(unsigned)((nw + kThreads - 1) / kThreads), kThreads, 0, s>>>(
-      (const bf16_t*)w, (bf16_t*)ws, g->K, g->C, T);
+  const size_t need = variant == 1 ? packed_weight_bytes(g, true) : nw * sizeof(bf16_t);
+  if (!ws || ws_bytes < need || !mn_aligned(ws, 16) || !mn_aligned(dy, 16)) return MN_EINVAL;
+  if (variant == 1)
+    pack_weights(g, (const bf16_t*)w, (bf16_t*)ws, true, s);
+  else
+    transpose_weights_bf16_kernel<<<(unsigned)((nw + kThreads - 1) / kThreads), kThreads, 0, s>>>(
+        (const bf16_t*)w, (bf16_t*)ws, g->K, g->C, T);
   bool empty_class = false;
   for (int ca = 0; ca < g->sH && !empty_class; ++ca) {
     bool any = false;
@@ -646,6 +765,7 @@ int mn_conv16_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void* 
       q.osh = g->sH;
       q.osw = g->sW;
       q.wrow = (uint32_t)T * g->K;
+      q.wstep = variant == 1 ? 1024 : 32;
       const int lst = launch_gather16(q, (const bf16_t*)dy, (const bf16_t*)ws, nullptr, (bf16_t*)dx, s);
       if (lst != MN_OK) return lst;
     }
@@ -654,7 +774,7 @@ int mn_conv16_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void* 
 }
 
 int mn_conv16_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, void* dw, void* ws,
-                         size_t ws_bytes, hipStream_t s) {
+                         size_t ws_bytes, int variant, hipStream_t s) {
   using namespace mn_conv16;
   const int st = check16(g);
   if (st != MN_OK) return st;

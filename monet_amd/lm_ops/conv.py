@@ -31,9 +31,10 @@ DEFAULT_VARIANT = 0
 def _refused(exc):
     """True when a kernel variant was refused before anything was launched (unknown index,
     shape it does not cover): the only failures the operators answer by running variant 0.
-    Launch failures, host-side shape / dtype errors and allocator failures propagate."""
-    return isinstance(exc, _lib.MonetHipError) and exc.status in (_lib.MN_EUNSUPPORTED,
-                                                                  _lib.MN_EINVAL)
+    Launch failures, invalid arguments (MN_EINVAL: a null or misaligned pointer, a workspace
+    smaller than mn_conv_ws_bytes asked for), host-side shape / dtype errors and allocator
+    failures propagate."""
+    return isinstance(exc, _lib.MonetHipError) and exc.status == _lib.MN_EUNSUPPORTED
 
 
 def _pair(v):

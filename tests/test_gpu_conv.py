@@ -40,6 +40,9 @@ CASES = [
     ((2, 16, 6, 7), (16, 16, 3, 3), 1, 2, 1),          # 3x3 padded by 2: output larger than the input
     ((2, 20, 11, 13), (48, 20, 3, 3), 1, 1, 1),        # Winograd backward-data only (K % 16 == 0, C is not)
     ((3, 48, 5, 5), (32, 48, 3, 3), 1, 1, 1),          # odd planes: ragged 2x2 output tiles
+    ((3, 96, 10, 10), (48, 96, 1, 1), 1, 0, 1),        # 1x1: 48 output channels in a 64-wide tile, pixel tiles across images
+    ((5, 256, 14, 14), (320, 256, 1, 1), 1, 0, 1),     # 1x1: 256-channel tiles with a ragged second one
+    ((2, 144, 12, 12), (128, 144, 1, 1), 1, 0, 1),     # 1x1: nine 16-deep stages (an odd number)
 ]
 
 
@@ -56,6 +59,15 @@ def winograd_applies(ws, st, pad, dil, reduced_channels):
 def winograd_wgrad_applies(xs, ws, st, pad, dil):
     """Variant 2 of backward-weight: 3x3, stride 1, dilation 1, equal padding <= 2, C % 4 == 0."""
     return winograd_applies(ws, st, pad, dil, 16) and xs[1] % 4 == 0
+
+
+def split_applies(xs, ws, st, pad, dil, reduced_channels):
+    """Variant 4 of forward and backward-data (fp32 through three bf16 slices per operand on the
+    bf16 matrix cores): 1x1 filters, stride 1, no padding, planes of a multiple of 4 pixels and
+    a reduction over a multiple of 16 channels; anything else is refused."""
+    pair = lambda v: tuple(v) if isinstance(v, (tuple, list)) else (v, v)
+    return (ws[2] == 1 and ws[3] == 1 and pair(st) == (1, 1) and pair(pad) == (0, 0) and
+            (xs[2] * xs[3]) % 4 == 0 and reduced_channels % 16 == 0)
 
 
 def refused(call):
@@ -97,9 +109,10 @@ def test_conv_forward(cuda, xs, ws, st, pad, dil):
     x, w, b = problem(xs, ws)
     exp = O.conv_fwd(x, w, b, st, pad, dil)
     exp_nobias = O.conv_fwd(x, w, None, st, pad, dil)
-    assert conv_ops.n_fwd_algos() == 4
+    assert conv_ops.n_fwd_algos() == 5
     for v in range(conv_ops.n_fwd_algos()):
-        if v >= 2 and not winograd_applies(ws, st, pad, dil, xs[1]):
+        if (v in (2, 3) and not winograd_applies(ws, st, pad, dil, xs[1])) or \
+                (v == 4 and not split_applies(xs, ws, st, pad, dil, xs[1])):
             assert refused(lambda: conv_ops.conv_forward(dev(x, cuda), dev(w, cuda), None, pad, st,
                                                          dil, 1, v))
             continue
@@ -116,9 +129,10 @@ def test_conv_backward_data(cuda, xs, ws, st, pad, dil):
     yshape = O.conv_fwd(x, w, None, st, pad, dil).shape
     dy = np.random.default_rng(2).standard_normal(yshape).astype(np.float32)
     exp = O.conv_bwd_data(dy, w, xs, st, pad, dil)
-    assert conv_ops.n_bwd_ip_algos() == 4
+    assert conv_ops.n_bwd_ip_algos() == 5
     for v in range(conv_ops.n_bwd_ip_algos()):
-        if v >= 2 and not winograd_applies(ws, st, pad, dil, ws[0]):
+        if (v in (2, 3) and not winograd_applies(ws, st, pad, dil, ws[0])) or \
+                (v == 4 and not split_applies(xs, ws, st, pad, dil, ws[0])):
             assert refused(lambda: conv_ops.conv_backward_input(xs, dev(dy, cuda), dev(w, cuda),
                                                                 pad, st, dil, 1, v))
             continue
@@ -256,8 +270,8 @@ def test_conv_bf16_all_directions(cuda, xs, ws, st, pad, dil):
     exp = O.conv_fwd(x, w, b, st, pad, dil)
     rng = np.random.default_rng(5)
     dy = bf16_round(rng.standard_normal(exp.shape))
-    assert conv_ops.n_fwd_algos(torch.bfloat16) == 1
-    for v in (0, 1):    # index 1 is accepted as an alias of the one bf16 kernel
+    assert conv_ops.n_fwd_algos(torch.bfloat16) == 2
+    for v in (0, 1):    # weights read in place / packed in fragment order in the workspace
         y = conv_ops.conv_forward(dev16(x, cuda), dev16(w, cuda), dev16(b, cuda), pad, st, dil, 1, v)
         assert y.dtype == torch.bfloat16 and y.is_contiguous(memory_format=torch.channels_last)
         assert_rel(host(y.float()), exp, BF16_TOL, f"bf16 forward variant {v}")
@@ -310,7 +324,7 @@ def test_conv_bf16_channel_counts_that_only_fit_the_shallow_tiles(cuda):
     assert e.value.status == _lib.MN_EUNSUPPORTED
 
 
-@pytest.mark.parametrize("xs,ws,st,pad,dil", [CASES[8], CASES[10], CASES[11], CASES[1], CASES[9]])
+@pytest.mark.parametrize("xs,ws,st,pad,dil", [CASES[8], CASES[10], CASES[11], CASES[1], CASES[9], CASES[25]])
 def test_conv_backward_data_accumulates_into_an_existing_gradient(cuda, xs, ws, st, pad, dil):
     """dx += conv_backward_data(dy): every variant, dense and strided (parity-class) outputs,
     positions no tap reaches keep their value, split reductions add onto what is there."""
@@ -320,7 +334,9 @@ def test_conv_backward_data_accumulates_into_an_existing_gradient(cuda, xs, ws, 
     prior = rng.standard_normal(xs).astype(np.float32)
     exp = prior.astype(np.float64) + O.conv_bwd_data(dy, w, xs, st, pad, dil)
     for v in range(conv_ops.n_bwd_ip_algos()):
-        if v >= 2 and not winograd_applies(ws, st, pad, dil, ws[0]):
+        if v in (2, 3) and not winograd_applies(ws, st, pad, dil, ws[0]):
+            continue
+        if v == 4 and not split_applies(xs, ws, st, pad, dil, ws[0]):
             continue
         acc = dev(prior, cuda)
         out = conv_ops.conv_backward_input(xs, dev(dy, cuda), dev(w, cuda), pad, st, dil, 1, v,

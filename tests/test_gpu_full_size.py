@@ -116,17 +116,34 @@ def test_max_pool_indices_at_full_size(cuda):
     assert float((dx.double().view(N, C, H * W) - ref).abs().max()) < 1e-5
 
 
-@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 1e-2)])
-def test_convolution_directions_are_adjoint_at_full_size(cuda, dtype, tol):
-    xs, ws = LAYER3
+POINTWISE3 = ((184, 1024, 14, 14), (256, 1024, 1, 1))   # ResNet-50 layer3, reducing 1x1
+
+
+def _variants(n, run):
+    """(variant, result) for every variant that takes the shape; refusals are skipped."""
+    from monet_amd import _lib
+    for v in range(n):
+        try:
+            yield v, run(v)
+        except _lib.MonetHipError as e:
+            if e.status != _lib.MN_EUNSUPPORTED:
+                raise
+
+
+@pytest.mark.parametrize("shape,pad,dtype,tol", [(LAYER3, 1, torch.float32, 1e-5),
+                                                 (LAYER3, 1, torch.bfloat16, 1e-2),
+                                                 (POINTWISE3, 0, torch.float32, 1e-5)])
+def test_convolution_directions_are_adjoint_at_full_size(cuda, shape, pad, dtype, tol):
+    xs, ws = shape
     x = _randn(xs, cuda, 7)
-    w = _randn(ws, cuda, 8) * (2.0 / (ws[0] * 9)) ** 0.5
+    w = _randn(ws, cuda, 8) * (2.0 / (ws[0] * ws[2] * ws[3])) ** 0.5
     if dtype == torch.bfloat16:
         x = x.to(dtype).contiguous(memory_format=torch.channels_last)
         w = w.to(dtype).contiguous(memory_format=torch.channels_last)
     dy = None
-    for v in range(conv_ops.n_fwd_algos(dtype)):
-        y = conv_ops.conv_forward(x, w, None, 1, 1, 1, 1, v)
+    ran = []
+    for v, y in _variants(conv_ops.n_fwd_algos(dtype), lambda v: conv_ops.conv_forward(x, w, None, pad, 1, 1, 1, v)):
+        ran.append(v)
         if dy is None:
             dy = _randn(tuple(y.shape), cuda, 9)
             if dtype == torch.bfloat16:
@@ -135,22 +152,25 @@ def test_convolution_directions_are_adjoint_at_full_size(cuda, dtype, tol):
         # <conv(x, w), dy> is a sum of 9e6 products of independent values: its natural size is
         # sqrt(n) * rms(y) * rms(dy) (a wrong operand, e.g. transposed weights, is off by ~0.2 of it)
         scale = (y.numel() ** 0.5) * float(y.float().pow(2).mean().sqrt()) * float(dy.float().pow(2).mean().sqrt())
-        for vd in range(conv_ops.n_bwd_ip_algos(dtype)):
-            dx = conv_ops.conv_backward_input(list(xs), dy, w, 1, 1, 1, 1, vd)
+        for vd, dx in _variants(conv_ops.n_bwd_ip_algos(dtype), lambda vd: conv_ops.conv_backward_input(
+                list(xs), dy, w, pad, 1, 1, 1, vd)):
             assert abs(lhs - _dot(dx, x)) < tol * scale, (v, vd)
-        for vw in range(conv_ops.n_bwd_wt_algos(dtype)):
-            dw = conv_ops.conv_backward_weight(list(ws), dy, x, 1, 1, 1, 1, vw)
+        for vw, dw in _variants(conv_ops.n_bwd_wt_algos(dtype), lambda vw: conv_ops.conv_backward_weight(
+                list(ws), dy, x, pad, 1, 1, 1, vw)):
             assert abs(lhs - _dot(dw, w)) < tol * scale, (v, vw)
         # linearity of the forward in x (exact up to rounding of the two results)
         x2 = _randn(xs, cuda, 10)
         if dtype == torch.bfloat16:
             x2 = x2.to(dtype).contiguous(memory_format=torch.channels_last)
-        y2 = conv_ops.conv_forward(x2, w, None, 1, 1, 1, 1, v)
+        y2 = conv_ops.conv_forward(x2, w, None, pad, 1, 1, 1, v)
         ys = conv_ops.conv_forward((x.float() + x2.float()).to(dtype).contiguous(
             memory_format=torch.channels_last if dtype == torch.bfloat16 else torch.contiguous_format),
-            w, None, 1, 1, 1, 1, v)
+            w, None, pad, 1, 1, 1, v)
         lin_tol = (4 if dtype == torch.float32 else 3) * tol * float(ys.float().abs().max())
         assert float((ys.float() - (y.float() + y2.float())).abs().max()) < lin_tol, v
+    # every variant that covers the shape ran: Winograd on the 3x3, three slices on the 1x1
+    expect = {(3, torch.float32): [0, 1, 2, 3], (3, torch.bfloat16): [0, 1], (1, torch.float32): [0, 1, 4]}
+    assert ran == expect[(ws[2], dtype)]
 
 
 @pytest.fixture(scope="module")
