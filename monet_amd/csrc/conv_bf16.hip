@@ -323,6 +323,214 @@ __global__ __launch_bounds__(kThreads) void gather_bf16_kernel(const GatherH g,
   }
 }
 
+// The large-tile form of the same gather GEMM: 64 CMW output channels x 128 TN / CMW positions x 64
+// deep per stage, eight wavefronts with two roles.  Wavefronts 0-3 (one per SIMD) only multiply:
+// CMW of them along the channels (64 each), 4 / CMW along the positions (32 TN each, 2 x TN
+// accumulator tiles); per stage one reads 4 x (2 + TN) fragments from LDS for 8 TN matrix
+// instructions.  Wavefronts 4-7 (the second one of each
+// SIMD) only feed: they fetch the next stages' weight rows and gathered pixel rows into
+// registers two stages ahead and write them to LDS, double buffered, one barrier per stage.
+// With every wavefront doing both (the 128 x 128 kernel above) the phases of a stage run one
+// after the other on all of them, and what a CU pulls through its vector memory path per matrix
+// instruction is twice as much: 0.54 PFLOP/s at the ResNet-50 layer3 shape against the
+// 2.5 PFLOP/s peak.  Workgroups are persistent (at most one per CU) and walk the tile list.
+// Needs Cs % 64 == 0 and Nout % 64 == 0; weights as rows in place (wstep == 32).
+constexpr int kRoleThreads = 512;
+constexpr int kRoleDepth = 64;
+constexpr int kRoleLd = kRoleDepth + 8;   // LDS row: 144 bytes (9 x 16: conflict-free 16-byte reads)
+
+template <int CMW, int TN>
+__global__ __launch_bounds__(kRoleThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void gather_roles_kernel(
+    const GatherH g, const bf16_t* __restrict__ src, const bf16_t* __restrict__ w,
+    const bf16_t* __restrict__ bias, bf16_t* __restrict__ dst) {
+  constexpr int CPW = 4 / CMW;
+  constexpr int BMW = 64 * CMW, BP = 32 * TN * CPW;
+  static_assert(BP <= 256, "one row of the position table per multiplying thread");
+  constexpr int kFeeders = 256;
+  constexpr int kWChunks = BMW * (kRoleDepth / 8) / kFeeders;
+  constexpr int kXChunks = (BP * (kRoleDepth / 8) + kFeeders - 1) / kFeeders;
+  constexpr uint32_t kBeyond = 0x80000000u;   // byte offset past any buffer (tensors are < 2 GB)
+  __shared__ __attribute__((aligned(16))) bf16_t lds_w[2][BMW][kRoleLd];
+  __shared__ __attribute__((aligned(16))) bf16_t lds_x[2][BP][kRoleLd];
+  __shared__ int tdh[kMaxTaps], tdw[kMaxTaps], twoff[kMaxTaps];
+  __shared__ uint32_t row_dst[2][BP];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t slot = xcd_slot();
+  const uint32_t ntiles_n = ((uint32_t)g.Nout + BMW - 1) / BMW;
+  const uint32_t tiles = ((g.npix + BP - 1) / BP) * ntiles_n;
+  const uint32_t plane = (uint32_t)g.OH * g.OW;
+  const int per_tap = g.Cs / kRoleDepth;
+  const int stages = g.T * per_tap;
+  if (tid < g.T) {
+    tdh[tid] = g.dh[tid];
+    tdw[tid] = g.dw[tid];
+    twoff[tid] = g.woff[tid];
+  }
+  __syncthreads();
+
+  if (wave >= 4) {
+    // ------------------------------------------------------------------ feeding wavefronts
+    const int ft = tid - 256;
+    const __amdgpu_buffer_rsrc_t src_buf =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(src), 0, g.src_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t w_buf =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(w), 0, g.w_bytes, 0x00020000);
+    // chunk e = ft + 256 i of an operand tile: row e / 8, 16-byte chunk e % 8 (a row's 128 bytes
+    // are contiguous in memory and across 8 lanes)
+    const int ch = ft & 7, row0 = ft >> 3;
+    uint32_t w_off[kWChunks];
+    int ohs[kXChunks], ows[kXChunks];
+    uint32_t abase[kXChunks];
+    bool aok[kXChunks];
+    uint32_t a_off[kXChunks];
+    constexpr int kSets = 4;   // register sets = stages the loads run ahead of the LDS writes
+    uint4_t rw[kSets][kWChunks], rx[kSets][kXChunks];
+    for (uint32_t tile = slot; tile < tiles; tile += gridDim.x) {
+      const uint32_t p0 = (tile / ntiles_n) * BP;
+      const int n0 = (int)(tile % ntiles_n) * BMW;
+#pragma unroll
+      for (int i = 0; i < kWChunks; ++i) {
+        const int col = n0 + row0 + 32 * i;
+        w_off[i] = col < g.Nout ? ((uint32_t)col * g.wrow + ch * 8) * 2u : kBeyond;
+      }
+#pragma unroll
+      for (int i = 0; i < kXChunks; ++i) {
+        const uint32_t r = row0 + 32 * i, pix = p0 + r;
+        aok[i] = r < BP && pix < g.npix;
+        const uint32_t pp = aok[i] ? pix : 0u;
+        const uint32_t n = pp / plane, rem = pp - n * plane;
+        const uint32_t oh = rem / g.OW, ow = rem - oh * g.OW;
+        ohs[i] = oh * g.ish;
+        ows[i] = ow * g.isw;
+        abase[i] = n * (uint32_t)g.Hs * g.Ws;
+      }
+      int t = -1, c0 = g.Cs;   // position of the next stage to fetch
+      uint32_t so_w = 0;
+      auto fetch = [&](uint4_t (&qw)[kWChunks], uint4_t (&qx)[kXChunks]) {
+        c0 += kRoleDepth;
+        if (c0 >= g.Cs) {   // enter the next tap (uniform)
+          c0 = 0;
+          ++t;
+          const int dh = tdh[t], dw = tdw[t];
+#pragma unroll
+          for (int i = 0; i < kXChunks; ++i) {
+            const int hh = ohs[i] + dh, ww = ows[i] + dw;
+            const bool ok = aok[i] && (unsigned)hh < (unsigned)g.Hs && (unsigned)ww < (unsigned)g.Ws;
+            a_off[i] = ok ? ((abase[i] + hh * g.Ws + ww) * (uint32_t)g.Cs + ch * 8) * 2u : kBeyond;
+          }
+          so_w = (uint32_t)__builtin_amdgcn_readfirstlane(twoff[t]) * 2u;
+        }
+        const int so = __builtin_amdgcn_readfirstlane(c0 * 2);
+        const int sw = __builtin_amdgcn_readfirstlane((int)so_w + c0 * 2);
+#pragma unroll
+        for (int i = 0; i < kWChunks; ++i)
+          qw[i] = __builtin_amdgcn_raw_buffer_load_b128(w_buf, w_off[i], sw, 0);
+#pragma unroll
+        for (int i = 0; i < kXChunks; ++i)
+          qx[i] = __builtin_amdgcn_raw_buffer_load_b128(src_buf, a_off[i], so, 0);
+      };
+      auto stage = [&](int buf, const uint4_t (&qw)[kWChunks], const uint4_t (&qx)[kXChunks]) {
+#pragma unroll
+        for (int i = 0; i < kWChunks; ++i)
+          *reinterpret_cast<uint4_t*>(&lds_w[buf][row0 + 32 * i][ch * 8]) = qw[i];
+#pragma unroll
+        for (int i = 0; i < kXChunks; ++i)
+          if (row0 + 32 * i < BP) *reinterpret_cast<uint4_t*>(&lds_x[buf][row0 + 32 * i][ch * 8]) = qx[i];
+      };
+#pragma unroll
+      for (int k = 0; k < kSets; ++k)
+        if (k < stages) fetch(rw[k], rx[k]);
+      stage(0, rw[0], rx[0]);
+      if (kSets < stages) fetch(rw[0], rx[0]);
+      __syncthreads();
+      for (int s2 = 0; s2 < stages; s2 += kSets) {
+#pragma unroll
+        for (int u = 0; u < kSets; ++u) {
+          if (s2 + u >= stages) break;
+          const int k = (u + 1) % kSets;   // register set of stage s2 + u + 1
+          if (s2 + u + 1 < stages) stage((u + 1) & 1, rw[k], rx[k]);
+          if (s2 + u + 1 + kSets < stages) fetch(rw[k], rx[k]);
+          __syncthreads();
+        }
+      }
+    }
+    return;
+  }
+
+  // -------------------------------------------------------------------- multiplying wavefronts
+  const int wm = wave / CPW, wp = wave % CPW;   // 64 channels x 32 TN positions each
+  const int r = lane & 31, kq = (lane >> 5) * 8;
+  const bf16_t* aw = &lds_w[0][wm * 64 + r][kq];
+  const bf16_t* ax = &lds_x[0][wp * TN * 32 + r][kq];
+  float16_t acc[2][TN];
+  int parity = 0;
+  for (uint32_t tile = slot; tile < tiles; tile += gridDim.x, parity ^= 1) {
+    const uint32_t p0 = (tile / ntiles_n) * BP;
+    const int n0 = (int)(tile % ntiles_n) * BMW;
+    if (tid < BP) {
+      const uint32_t pix = p0 + tid;
+      uint32_t off = kNoRow;
+      if (pix < g.npix) {
+        const uint32_t n = pix / plane, rem = pix - n * plane;
+        const uint32_t oh = rem / g.OW, ow = rem - oh * g.OW;
+        off = ((n * g.DH + oh * g.osh + g.oh0) * (uint32_t)g.DW + ow * g.osw + g.ow0) * (uint32_t)g.Nout;
+      }
+      row_dst[parity][tid] = off;
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    __syncthreads();   // stage 0 is in LDS
+    for (int s2 = 0; s2 < stages; ++s2) {
+      const bf16_t* bw = aw + (s2 & 1) * (BMW * kRoleLd);
+      const bf16_t* bx = ax + (s2 & 1) * (BP * kRoleLd);
+#pragma unroll
+      for (int ks = 0; ks < kRoleDepth; ks += 16) {
+        bf16x8 af[2], bfr[TN];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) af[i] = *reinterpret_cast<const bf16x8*>(bw + 32 * i * kRoleLd + ks);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) bfr[j] = *reinterpret_cast<const bf16x8*>(bx + 32 * j * kRoleLd + ks);
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+      }
+      __syncthreads();
+    }
+    // channels are the rows of the matrix instruction: a lane holds four consecutive channels of
+    // one position in four consecutive registers = one 8-byte store; lanes l and l + 32 write
+    // neighbouring 8 bytes
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+      for (int v4 = 0; v4 < 4; ++v4) {
+        const int col = n0 + wm * 64 + 32 * i + 8 * v4 + 4 * (lane >> 5);
+        if (col >= g.Nout) continue;
+        float b4[4] = {0.f, 0.f, 0.f, 0.f};
+        if (bias) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) b4[e] = bf2f(bias[col + e]);
+        }
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const uint32_t off = row_dst[parity][(wp * TN + j) * 32 + (lane & 31)];
+          if (off == kNoRow) continue;
+          uint32_t lo = (uint32_t)f2bf(acc[i][j][4 * v4] + b4[0]) | ((uint32_t)f2bf(acc[i][j][4 * v4 + 1] + b4[1]) << 16);
+          uint32_t hi = (uint32_t)f2bf(acc[i][j][4 * v4 + 2] + b4[2]) | ((uint32_t)f2bf(acc[i][j][4 * v4 + 3] + b4[3]) << 16);
+          typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+          *reinterpret_cast<u2*>(dst + off + col) = u2{lo, hi};
+        }
+      }
+    }
+  }
+}
+
 // Weight operand in fragment order: wp[(blk * steps + s) * 64 + lane] (16-byte units) = the 8
 // elements rows[blk * 32 + lane % 32][s * 16 + (lane / 32) * 8 ...] of a [rows][len] matrix
 // (rows beyond the matrix are zero).  With transposed == 0 the matrix is the weight tensor
@@ -575,6 +783,13 @@ static int check16(const mn_conv2d* g) {
   return MN_OK;
 }
 
+// Shapes the large-tile kernel (feeding and multiplying wavefronts) takes, given weight rows in
+// place: deep enough channel chunks, at least 128 output channels in whole 64s, enough positions
+// to fill the device.
+static bool roles_shape(int Cs, int Nout, unsigned long long npix) {
+  return Cs % 64 == 0 && Nout % 64 == 0 && Nout >= 128 && npix >= 4096;
+}
+
 static int launch_gather16(GatherH q, const bf16_t* src, const bf16_t* w, const bf16_t* bias,
                            bf16_t* dst, hipStream_t s) {
   if (q.npix == 0 || q.Nout == 0) return MN_OK;
@@ -587,6 +802,38 @@ static int launch_gather16(GatherH q, const bf16_t* src, const bf16_t* w, const 
   q.src_bytes = (uint32_t)src_bytes;
   q.w_bytes = (uint32_t)w_bytes;
   const bool deep = q.Cs % 64 == 0;
+  if (q.wstep == 32 && roles_shape(q.Cs, q.Nout, q.npix)) {
+    // large tiles, feeding and multiplying wavefronts.  256-channel tiles of 128 or 160 positions
+    // (160 where it saves a round of the persistent, one-per-CU workgroups), 128-channel tiles of
+    // 192 or 256 positions when that covers the channels with less padding.
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      cus = 256;
+    struct Cand { int bm, bp; };
+    static const Cand cands[] = {{256, 160}, {256, 128}, {128, 256}, {128, 192}};
+    int best = 0;
+    double best_cost = 1e30;
+    long long best_tiles = 0;
+    for (int i = 0; i < 4; ++i) {
+      const long long tiles = (long long)((q.npix + cands[i].bp - 1) / cands[i].bp) * ((q.Nout + cands[i].bm - 1) / cands[i].bm);
+      // rounds x tile area; the narrower channel tile re-reads the pixels once more per 128 channels
+      const double cost = (double)((tiles + cus - 1) / cus) * cands[i].bp * cands[i].bm * (cands[i].bm == 128 ? 1.1 : 1.0);
+      if (cost < best_cost) {
+        best_cost = cost;
+        best = i;
+        best_tiles = tiles;
+      }
+    }
+    const dim3 grid((unsigned)(best_tiles < cus ? best_tiles : cus));
+    switch (best) {
+      case 0: gather_roles_kernel<4, 5><<<grid, kRoleThreads, 0, s>>>(q, src, w, bias, dst); break;
+      case 1: gather_roles_kernel<4, 4><<<grid, kRoleThreads, 0, s>>>(q, src, w, bias, dst); break;
+      case 2: gather_roles_kernel<2, 4><<<grid, kRoleThreads, 0, s>>>(q, src, w, bias, dst); break;
+      default: gather_roles_kernel<2, 3><<<grid, kRoleThreads, 0, s>>>(q, src, w, bias, dst); break;
+    }
+    return MN_OK;
+  }
   if (q.Nout % 128 == 0) {
     dim3 grid((q.npix + BM - 1) / BM, q.Nout / 128);
     if (deep)
@@ -672,7 +919,9 @@ int mn_conv16_fwd(const mn_conv2d* g, const void* x, const void* w, const void* 
   if (!mn_aligned(x, 16) || !mn_aligned(w, 16)) return MN_EINVAL;
   GatherH q = {};
   q.wstep = 32;
-  if (variant == 1) {   // weights in fragment order in the workspace
+  // variant 1 packs the weights in fragment order for the kernel that loads them straight into
+  // registers; shapes the large-tile kernel takes run that one under either variant
+  if (variant == 1 && !roles_shape(g->C, g->K, (unsigned long long)g->N * g->P * g->Q)) {
     if (!ws || ws_bytes < packed_weight_bytes(g, false) || !mn_aligned(ws, 16)) return MN_EINVAL;
     pack_weights(g, (const bf16_t*)w, (bf16_t*)ws, false, s);
     w = ws;
@@ -714,7 +963,11 @@ int mn_conv16_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void* 
   const size_t nw = (size_t)g->K * g->C * T;
   const size_t need = variant == 1 ? packed_weight_bytes(g, true) : nw * sizeof(bf16_t);
   if (!ws || ws_bytes < need || !mn_aligned(ws, 16) || !mn_aligned(dy, 16)) return MN_EINVAL;
-  if (variant == 1)
+  // variant 1: fragment-packed transposed weights, except where the large-tile kernel runs
+  // (it reads plain transposed rows; the packed size covers them)
+  const bool packed = variant == 1 &&
+                      !roles_shape(g->K, g->C, (unsigned long long)g->N * g->H * g->W / (g->sH * g->sW));
+  if (packed)
     pack_weights(g, (const bf16_t*)w, (bf16_t*)ws, true, s);
   else
     transpose_weights_bf16_kernel<<<(unsigned)((nw + kThreads - 1) / kThreads), kThreads, 0, s>>>(
@@ -765,7 +1018,7 @@ int mn_conv16_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void* 
       q.osh = g->sH;
       q.osw = g->sW;
       q.wrow = (uint32_t)T * g->K;
-      q.wstep = variant == 1 ? 1024 : 32;
+      q.wstep = packed ? 1024 : 32;
       const int lst = launch_gather16(q, (const bf16_t*)dy, (const bf16_t*)ws, nullptr, (bf16_t*)dx, s);
       if (lst != MN_OK) return lst;
     }

@@ -251,6 +251,12 @@ BF16_CASES = [
     ((2, 128, 7, 9), (128, 128, 2, 3), (2, 1), (1, 0), 1),
     ((8, 256, 14, 14), (256, 256, 3, 3), 1, 1, 1),      # ResNet-50 layer3 shape at a small batch
     ((2, 64, 56, 56), (256, 64, 1, 1), 1, 0, 1),
+    # more than 4096 positions and at least 128 output channels: the large-tile kernel (feeding
+    # and multiplying wavefronts), 256- and 128-channel tiles, ragged in both directions
+    ((24, 256, 14, 14), (256, 256, 3, 3), 1, 1, 1),
+    ((80, 64, 15, 15), (192, 64, 3, 3), 2, 1, 1),
+    ((23, 128, 14, 14), (128, 128, 5, 5), 1, 2, 1),
+    ((34, 128, 12, 12), (320, 128, 1, 1), 1, 0, 1),
 ]
 
 

@@ -339,3 +339,59 @@ def test_solver_sizes_follow_the_element_size_of_the_profiled_tensors():
         else:
             assert a.mem == 2 * b.mem
         assert a.fixed_mem == 2 * b.fixed_mem
+
+
+class TinyNet(nn.Module):
+    """Four operators: small enough to enumerate every schedule."""
+    def __init__(self):
+        super().__init__()
+        self.c1 = nn.Conv2d(3, 6, 3, padding=1, bias=False)
+        self.r = nn.ReLU()
+        self.mp = nn.MaxPool2d(2, 2)
+        self.fc = nn.Linear(6 * 4 * 4, 5)
+
+    def forward(self, x):
+        return self.fc(torch.flatten(self.mp(self.r(self.c1(x))), 1))
+
+
+@pytest.mark.parametrize("mode", ["normal", "multiway"])
+def test_ilp_optimum_equals_the_enumerated_optimum_on_a_tiny_graph(mode):
+    """The restated ILP (with its reductions) against the reference's formulation evaluated on
+    every schedule of a 6-node graph: same optimal run time at every budget from generous to the
+    floor, and infeasible at the same budgets."""
+    from brute_force_schedule import optimum
+    torch.manual_seed(0)
+    g = Graph.create(TinyNet(), (3, 8, 8))
+    si = SolverInfo(64, "tiny", mode)
+
+    def cost(n, op, bwd_op):   # uneven costs, so that what is recomputed matters
+        mb = abs(np.prod(n.shape)) * 4 * si.bs / 1e6
+        k = 1.0 + 0.37 * (len(n.op) % 5)
+        # implementations that get by with less stored data are slower
+        name = type(op).__name__
+        k *= 1.25 if name.startswith(("OutputAct", "BinaryAct", "IndicesAct")) else 1.0
+        return ([0.0], [0.0], []), ([k * mb], [0.7 * k * mb], [])
+    si.extract(g, cost_fn=cost)
+    V = si.loss + 1
+    assert V <= 7
+    seen_feasible = seen_infeasible = 0
+    costs = []
+    # (KB) generous, around the point where storing everything stops fitting, just above and just
+    # below the floor of 341 KB
+    for kb in (4096, 365, 342, 335):
+        gb = kb / 1024.0 / 1024.0
+        exact = optimum(si, gb)
+        try:
+            sol = Model(si, budget=gb, time_limit=120, mip_rel_gap=0.0).solve()
+        except ValueError:
+            sol = None
+        if exact is None:
+            assert sol is None, (mode, kb)
+            seen_infeasible += 1
+        else:
+            assert sol is not None, (mode, kb)
+            assert abs(sol.runtime_expected - exact) <= 1e-6 * max(1.0, exact), (mode, kb, sol.runtime_expected, exact)
+            seen_feasible += 1
+            costs.append(exact)
+    assert seen_feasible == 3 and seen_infeasible == 1
+    assert costs[-1] > costs[0]       # a tight budget costs run time: the comparison is not trivial
