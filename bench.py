@@ -267,33 +267,131 @@ def cpu_baseline(sample_n=23, reps=5):
         times.append(time.perf_counter() - t0)
     med = sorted(times)[len(times) // 2]
     nbytes = BYTES_STEP * sample_n / N
+
+    def median_ms(fn, n=3):
+        fn()
+        ts = []
+        for _ in range(n):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        return sorted(ts)[len(ts) // 2] * 1e3
+    # the layer3 convolution of the convolution benchmark, three directions, same slice of the batch
+    g = CONV_SHAPE
+    cx = torch.randn(sample_n, g["C"], g["H"], g["W"])
+    cw = torch.randn(g["K"], g["C"], g["R"], g["S"]) * (2.0 / (g["K"] * 9)) ** 0.5
+    cdy = torch.randn(sample_n, g["K"], g["H"], g["W"])
+    cflops = 2.0 * cdy.numel() * g["C"] * 9
+    conv_legs = {}
+    for i, name in enumerate(("fwd", "bwd_data", "bwd_weight")):
+        if i == 0:
+            ms = median_ms(lambda: cpu_path.conv_forward(cx, cw, g["stride"], g["pad"]))
+        else:
+            mask = [i == 1, i == 2, False]
+            ms = median_ms(lambda: cpu_path.conv_backward(cdy, cx, cw, g["stride"], g["pad"], mask))
+        conv_legs[name] = {"ms": round(ms, 3), "TFLOP/s": round(cflops / ms / 1e9, 3)}
+    # the stem block (7x7/2 convolution, BatchNorm, ReLU, 3x3/2 max-pool; batch 8 of 3x224x224),
+    # forward + backward through stock autograd: 2 warm-up + median of 5
+    stem, sx = cpu_path.stem_block(8)
+    cpu_path.stem_step(stem, sx)
+    stem_ms = median_ms(lambda: cpu_path.stem_step(stem, sx), 5)
     return {"value": round(nbytes / med / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
             "sample": f"{sample_n} of {N} images of the same three operators through stock PyTorch "
-                      f"CPU ops (torch {torch.__version__}), 1 warm-up + median of {reps}"}
+                      f"CPU ops (torch {torch.__version__}), 1 warm-up + median of {reps}",
+            "conv_layer3": {"sample": f"{sample_n} of {N} images, fp32, torch CPU convolution "
+                                      f"(mkldnn {torch.backends.mkldnn.is_available()}), 1 warm-up + median of 3",
+                            **conv_legs},
+            "stem_block": {"sample": "batch 8, forward + backward, 2 warm-up + median of 5",
+                           "ms": round(stem_ms, 2), "images_per_s": round(8 / stem_ms * 1e3, 1)}}
 
 
 MFMA_F32_PEAK_TFLOPS = 157.3   # MI355X published dense fp32 matrix rate
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # ... and dense bf16
 CONV_SHAPE = dict(N=184, C=256, K=256, R=3, S=3, H=14, W=14, stride=1, pad=1)  # ResNet-50 layer3
+# Matrix-core work each entry of the convolution benchmark really issues, from hardware counters
+# (they cannot be read inside this program): one `rocprofv3 --pmc SQ_INSTS_VALU_MFMA_MOPS_F32
+# SQ_INSTS_VALU_MFMA_MOPS_BF16 SQ_VALU_MFMA_BUSY_CYCLES GRBM_GUI_ACTIVE` run of
+# `bench.py --only conv --steps 3 --warmup 1`, turned into this file by
+# `bench.py --mfma-summary PMC_DIR BENCH_STDOUT`.
+MFMA_FILE = ROOT / "profiles" / "conv_bs184_mfma_flops.json"
+MARKER = "spin_kernel"   # torch.cuda._sleep: separates the entries in the counter output
+
+
+def load_mfma():
+    """{entry path: {"flop": issued per call, "mfma": "f32" | "bf16", "busy": ...}}, {} if absent."""
+    try:
+        return json.loads(MFMA_FILE.read_text())["entries"]
+    except (OSError, ValueError, KeyError):
+        return {}
+
+
+def mfma_summary(pmc_dir, bench_stdout):
+    """Write MFMA_FILE.  The benchmark launches one marker kernel before every entry and prints
+    the entries in order (`order`), with the calls each made; the dispatches between two markers
+    are one entry's.  flop = MFMA_MOPS * 512 (one counter unit is 512 floating-point operations
+    on this chip; the direct kernels come out at exactly their algorithmic count)."""
+    import csv
+    line = [l for l in Path(bench_stdout).read_text().splitlines() if l.startswith("{")][-1]
+    conv = json.loads(line)["conv"]
+    order, calls = conv["order"], conv["calls_per_entry"]
+    rows = {}
+    for f in Path(pmc_dir).rglob("*counter_collection.csv"):
+        with open(f, newline="") as fh:
+            for r in csv.DictReader(fh):
+                d = rows.setdefault(int(r["Dispatch_Id"]), {"name": r["Kernel_Name"]})
+                d[r["Counter_Name"]] = d.get(r["Counter_Name"], 0.0) + float(r["Counter_Value"])
+    segments, cur = [], None
+    for did in sorted(rows):
+        if MARKER in rows[did]["name"]:
+            cur = []
+            segments.append(cur)
+        elif cur is not None:
+            cur.append(rows[did])
+    if len(segments) != len(order):
+        raise SystemExit("%d marked segments for %d entries" % (len(segments), len(order)))
+    entries = {}
+    for name, seg in zip(order, segments):
+        f32 = sum(d.get("SQ_INSTS_VALU_MFMA_MOPS_F32", 0.0) for d in seg) * 512.0 / calls
+        b16 = sum(d.get("SQ_INSTS_VALU_MFMA_MOPS_BF16", 0.0) for d in seg) * 512.0 / calls
+        busy = sum(d.get("SQ_VALU_MFMA_BUSY_CYCLES", 0.0) for d in seg)
+        act = sum(d.get("GRBM_GUI_ACTIVE", 0.0) for d in seg if d.get("SQ_VALU_MFMA_BUSY_CYCLES", 0.0) > 0)
+        kernels = sorted({d["name"].split("(")[0][:100] for d in seg if
+                          d.get("SQ_VALU_MFMA_BUSY_CYCLES", 0.0) > 0})
+        entries[name] = {"flop": f32 + b16, "mfma": "bf16" if b16 > f32 else "f32",
+                         # busy cycles of the 1024 SIMDs over the cycles of the kernels that use them
+                         "busy": round(busy / (1024.0 * act / 8.0), 3) if act else None,
+                         "kernels": kernels}
+    doc = {"what": "matrix-core floating-point operations per call of every entry of `python3 bench.py "
+                   "--only conv --steps 3 --warmup 1`, from rocprofv3 --pmc SQ_INSTS_VALU_MFMA_MOPS_F32 "
+                   "SQ_INSTS_VALU_MFMA_MOPS_BF16 SQ_VALU_MFMA_BUSY_CYCLES GRBM_GUI_ACTIVE (flop = MOPS * "
+                   "512; busy = MFMA busy cycles / (1024 SIMDs * GRBM_GUI_ACTIVE / 8 XCDs) over the "
+                   "kernels of the entry that use the matrix cores)",
+           "entries": entries}
+    MFMA_FILE.write_text(json.dumps(doc, indent=1) + "\n")
+    print(json.dumps(doc))
 
 
 def conv_bench(steps, warmup):
     """Forward / backward-data / backward-weight of the ResNet-50 layer3 3x3 convolution at
-    batch 184, fp32, every kernel variant the solver can select; TFLOP/s counts 2*N*K*P*Q*C*R*S
-    per call against the fp32 matrix-core peak."""
+    batch 184, every kernel variant the solver can select, fp32 and bf16; two 1x1 shapes of the
+    same network (where the three-slice variant applies) and one large-plane UNet shape.
+    `TFLOP/s_effective` counts the direct convolution's 2*N*K*P*Q*C*R*S per call whatever the
+    kernel does; `frac_mfma` is the matrix-core work the kernels really issue (hardware counters,
+    MFMA_FILE) per second against the peak of the matrix instruction they use - Winograd issues
+    2.24x fewer operations than the direct form, the three-slice variant six times as many in
+    bf16 - so it never exceeds 1."""
     import torch
 
     from monet_amd.lm_ops import conv as cv
-    c = CONV_SHAPE
+    from monet_amd import _lib
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
-    x = torch.randn(c["N"], c["C"], c["H"], c["W"], device=dev)
-    w = torch.randn(c["K"], c["C"], c["R"], c["S"], device=dev) * (2.0 / (c["K"] * 9)) ** 0.5
-    y = cv.conv_forward(x, w, None, c["pad"], c["stride"], 1, 1, 0)
-    dy = torch.randn_like(y)
-    flops = 2.0 * y.numel() * c["C"] * c["R"] * c["S"]
+    issued = load_mfma()
+    order = []
 
-    def timed(fn, peak):
+    def timed(path, fn, flops):
+        torch.cuda._sleep(1)       # the marker kernel
+        order.append(path)
         for _ in range(warmup):
             fn()
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -304,40 +402,78 @@ def conv_bench(steps, warmup):
         b.record()
         torch.cuda.synchronize()
         ms = a.elapsed_time(b) / steps
-        tf = flops / ms / 1e9
-        return {"ms": round(ms, 4), "TFLOP/s": round(tf, 1), "frac": round(tf / peak, 4)}
-
-    def directions(x, w, dy, peak):
-        out = {}
-        for v in range(cv.n_fwd_algos(x.dtype)):
-            out["fwd_v%d" % v] = timed(
-                lambda: cv.conv_forward(x, w, None, c["pad"], c["stride"], 1, 1, v), peak)
-        for v in range(cv.n_bwd_ip_algos(x.dtype)):
-            out["bwd_data_v%d" % v] = timed(lambda: cv.conv_backward_input(
-                list(x.shape), dy, w, c["pad"], c["stride"], 1, 1, v), peak)
-        for v in range(cv.n_bwd_wt_algos(x.dtype)):
-            out["bwd_weight_v%d" % v] = timed(lambda: cv.conv_backward_weight(
-                list(w.shape), dy, x, c["pad"], c["stride"], 1, 1, v), peak)
+        out = {"ms": round(ms, 4), "TFLOP/s_effective": round(flops / ms / 1e9, 1)}
+        cnt = issued.get(path)
+        if cnt:
+            peak = MFMA_BF16_PEAK_TFLOPS if cnt["mfma"] == "bf16" else MFMA_F32_PEAK_TFLOPS
+            out.update({"mfma": cnt["mfma"], "issued_flop_per_call": cnt["flop"],
+                        "frac_mfma": round(cnt["flop"] / ms / 1e9 / peak, 4)})
+        else:
+            out["frac_mfma"] = None
         return out
 
-    res = {"shape": c, "dtype": "f32", "flops_per_call": flops, "peak_TFLOP/s": MFMA_F32_PEAK_TFLOPS}
-    res.update(directions(x, w, dy, MFMA_F32_PEAK_TFLOPS))
-    # one large-plane shape beside it (UNet batch 11, 128 -> 128 channels at 208 x 304), forward only:
-    # where the one-kernel Winograd variant is the fastest
-    u = dict(N=11, C=128, K=128, H=208, W=304)
-    xu = torch.randn(u["N"], u["C"], u["H"], u["W"], device=dev)
-    wu = torch.randn(u["K"], u["C"], 3, 3, device=dev) * (2.0 / (u["K"] * 9)) ** 0.5
-    flops = 2.0 * u["N"] * u["K"] * u["H"] * u["W"] * u["C"] * 9
-    res["unet_128ch_208x304"] = {"shape": u, "flops_per_call": flops}
-    for v in range(cv.n_fwd_algos(xu.dtype)):
-        res["unet_128ch_208x304"]["fwd_v%d" % v] = timed(
-            lambda: cv.conv_forward(xu, wu, None, 1, 1, 1, 1, v), MFMA_F32_PEAK_TFLOPS)
-    del xu, wu
-    flops = 2.0 * y.numel() * c["C"] * c["R"] * c["S"]
+    def runs(fn, n):
+        """Variants of one direction that take this shape: {variant: callable}."""
+        ok = {}
+        for v in range(n):
+            try:
+                fn(v)
+                ok[v] = (lambda v=v: fn(v))
+            except _lib.MonetHipError as e:
+                if e.status != _lib.MN_EUNSUPPORTED:
+                    raise
+        return ok
+
+    def directions(prefix, g, x, w, dy, which=("fwd", "bwd_data", "bwd_weight")):
+        out = {}
+        flops = 2.0 * dy.numel() * w.shape[1] * w.shape[2] * w.shape[3]
+        table = {
+            "fwd": (cv.n_fwd_algos(x.dtype), lambda v: cv.conv_forward(
+                x, w, None, g["pad"], g["stride"], 1, 1, v)),
+            "bwd_data": (cv.n_bwd_ip_algos(x.dtype), lambda v: cv.conv_backward_input(
+                list(x.shape), dy, w, g["pad"], g["stride"], 1, 1, v)),
+            "bwd_weight": (cv.n_bwd_wt_algos(x.dtype), lambda v: cv.conv_backward_weight(
+                list(w.shape), dy, x, g["pad"], g["stride"], 1, 1, v)),
+        }
+        for d in which:
+            n, fn = table[d]
+            for v, call in runs(fn, n).items():
+                key = "%s_v%d" % (d, v)
+                out[key] = timed(prefix + key, call, flops)
+        out["flops_per_call"] = flops
+        return out
+
+    def problem(g):
+        x = torch.randn(g["N"], g["C"], g["H"], g["W"], device=dev)
+        w = torch.randn(g["K"], g["C"], g["R"], g["S"], device=dev) * (2.0 / (g["K"] * g["R"] * g["S"])) ** 0.5
+        y = cv.conv_forward(x, w, None, g["pad"], g["stride"], 1, 1, 0)
+        return x, w, torch.randn_like(y)
+
+    c = CONV_SHAPE
+    x, w, dy = problem(c)
+    res = {"shape": c, "dtype": "f32", "peak_TFLOP/s": MFMA_F32_PEAK_TFLOPS}
+    res.update(directions("", c, x, w, dy))
     # the same problem on bf16 channels-last tensors (bf16 matrix cores, fp32 accumulation)
     cl = lambda t: t.to(torch.bfloat16).contiguous(memory_format=torch.channels_last)
     res["bf16"] = {"layout": "channels-last", "peak_TFLOP/s": MFMA_BF16_PEAK_TFLOPS}
-    res["bf16"].update(directions(cl(x), cl(w), cl(dy), MFMA_BF16_PEAK_TFLOPS))
+    res["bf16"].update(directions("bf16/", c, cl(x), cl(w), cl(dy)))
+    del x, w, dy
+    # 1x1 convolutions of the same network, fp32: variant 4 splits every operand into three bf16
+    # slices and accumulates the six significant products on the bf16 matrix cores
+    for name, g in (("pointwise_1024_256_14x14", dict(N=184, C=1024, K=256, R=1, S=1, H=14, W=14, stride=1, pad=0)),
+                    ("pointwise_64_256_56x56", dict(N=184, C=64, K=256, R=1, S=1, H=56, W=56, stride=1, pad=0))):
+        x, w, dy = problem(g)
+        res[name] = {"shape": g}
+        res[name].update(directions(name + "/", g, x, w, dy, ("fwd", "bwd_data")))
+        del x, w, dy
+    # one large-plane shape (UNet batch 11, 128 -> 128 channels at 208 x 304), forward only: where
+    # the one-kernel Winograd variant is the fastest
+    u = dict(N=11, C=128, K=128, R=3, S=3, H=208, W=304, stride=1, pad=1)
+    x, w, dy = problem(u)
+    res["unet_128ch_208x304"] = {"shape": u}
+    res["unet_128ch_208x304"].update(directions("unet_128ch_208x304/", u, x, w, dy, ("fwd",)))
+    res["order"] = order
+    res["calls_per_entry"] = steps + warmup + 1   # + the call that finds out whether a variant applies
     return res
 
 
@@ -422,14 +558,13 @@ def _schedules(name, bs, make_model, input_shape, x, loss_fn, modes, iters, warm
     return res
 
 
-def end_to_end(iters=20, warmup=10):
+def end_to_end(iters=20, warmup=100):
     """ResNet-50 (torchvision topology, random init), batch 184, fp32 SGD steps with cross
     entropy over 1000 classes: under the solved 10 GB and 6 GB schedules, under the
     unconstrained schedule (same kernels, nothing recomputed) and with stock PyTorch autograd;
     three operator sets (the reference's; BatchNorm+ReLU and add+ReLU pairs fused; also
     BatchNorm+add+ReLU at the end of a residual block).  Timing protocol of the reference
-    (monet/schedule.py:430-443) with 10 instead of 100 warm-up steps: 20 timed steps between
-    two events."""
+    (monet/schedule.py:430-443): 100 warm-up steps, then 20 timed steps between two events."""
     import torch
 
     from monet_amd.models import resnet50
@@ -446,7 +581,7 @@ def end_to_end(iters=20, warmup=10):
                       warmup, res)
 
 
-def end_to_end_unet(iters=20, warmup=5):
+def end_to_end_unet(iters=20, warmup=100):
     """The reference's UNet (models/unet) with 2 output classes, batch 11, 3 x 416 x 608, fp32
     SGD steps with softmax cross entropy over per-pixel labels, same runs as for ResNet-50."""
     import torch
@@ -479,9 +614,15 @@ def main():
     ap.add_argument("--traffic-summary", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"), default=None,
                     help="no GPU work: turn the output folders of the two counter runs of "
                          "`--only lm_ops` into profiles/lm_ops_bs184_hbm_traffic.json")
+    ap.add_argument("--mfma-summary", nargs=2, metavar=("PMC_DIR", "BENCH_STDOUT"), default=None,
+                    help="no GPU work: turn the output folder of the counter run of `--only conv` and "
+                         "what that run printed into profiles/conv_bs184_mfma_flops.json")
     args = ap.parse_args()
     if args.traffic_summary:
         traffic_summary(*args.traffic_summary)
+        return
+    if args.mfma_summary:
+        mfma_summary(*args.mfma_summary)
         return
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
@@ -523,8 +664,18 @@ def main():
     }
     out["conv"] = conv_bench(args.steps, args.warmup)
     if not args.no_end_to_end:
-        out["end_to_end"] = end_to_end()
+        out["end_to_end"] = e2e = end_to_end()
         out["end_to_end_unet"] = end_to_end_unet()
+        # the reference's own headline (ResNet-50, batch 184, 10 GB budget, its operator set):
+        # throughput of whole training steps and the overhead against the unconstrained schedule
+        head = e2e.get("budget_10GB")
+        if head:
+            out["config"]["resnet50_bs184_10GB"] = {
+                "images_per_s": head["images_per_s"], "ms_per_step": head["ms_per_step"],
+                "overhead_vs_unconstrained": head.get("overhead_vs_unconstrained"),
+                "peak_MB": head["peak_MB"], "within_budget": head.get("within_budget"),
+                "stock_pytorch_images_per_s": e2e["stock_pytorch"]["images_per_s"],
+                "warmup_steps": e2e["warmup_steps"], "timed_steps": e2e["timed_steps"]}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))

@@ -40,6 +40,15 @@ typedef void* mn_stream_t;
 /* ABI version of this header; bumped on any signature change. */
 int mn_abi_version(void);
 const char* mn_status_string(int status);
+/* Optional.  Does now, for the CURRENT device, what a few entry points would
+ * otherwise do on their first call there and what is not a stream operation:
+ * looks up the address of the fixed workspace of mn_bn_bwd_from_y_static_f32
+ * and raises the LDS limit of the one-kernel Winograd convolution.  A caller
+ * that captures HIP graphs calls it once per device before the first capture
+ * (or makes one call of those entry points outside capture); everyone else may
+ * ignore it.  Idempotent, thread-safe; MN_ELAUNCH if a lookup fails.  No
+ * counterpart in the reference. */
+int mn_init(void);
 
 /* ------------------------------------------------------------------ pack --
  * 1-bit pack: n bytes (each 0 or 1) -> (n+7)/8 bytes, first element in bit 7
@@ -149,10 +158,20 @@ int mn_bn_bwd_from_y_f32(const float* dy, const float* y, const float* gamma, co
  * word in the workspace is raised; each launch clears the word first.
  * mn_bn_ws_status waits for `stream`, reads the word left by the LAST launch
  * that used `ws` for a tensor of this shape and returns MN_ELAUNCH if it is
- * raised.  The reference's kernel (one block per channel, lrbn.cu:212-235)
+ * raised; ws == NULL (ws_bytes ignored) asks about the library's own array,
+ * i.e. about the last mn_bn_bwd_from_y_static_f32 call on this device.  The reference's kernel (one block per channel, lrbn.cu:212-235)
  * has no cross-block wait and so no counterpart of this call. */
 int mn_bn_ws_status(const void* ws, size_t ws_bytes, int64_t N, int64_t C, int64_t HW,
                     mn_stream_t stream);
+/* The same question for callers that free a workspace right after the call: a
+ * wait that gives up also raises one word per device, which stays raised.
+ * host_word == NULL: waits for `stream`, returns MN_ELAUNCH if any BatchNorm
+ * launch on the current device gave up a wait since the last such call, and
+ * clears the word.  host_word != NULL (pinned host memory): only enqueues a
+ * copy of the word to *host_word on `stream` and returns at once; the caller
+ * reads it when the stream has passed that point (non-zero = raised) and makes
+ * the synchronous call to clear it.  No counterpart in the reference. */
+int mn_bn_wait_status(uint32_t* host_word, mn_stream_t stream);
 /* mn_bn_bwd_from_y_f32 with its launch parameters given explicitly (0 = the
  * default): `spin_limit` polls before a wait gives up, at most
  * `max_workgroups` persistent workgroups, pieces of `channel_group`

@@ -50,6 +50,7 @@ _SIGNATURES = {
     # name: (restype, argtypes); restype c_int means "status code, checked"
     "mn_abi_version": (c_int, []),
     "mn_status_string": (c_char_p, [c_int]),
+    "mn_init": (c_int, []),
     "mn_pack_bits": (c_int, [_P, _P, c_size_t, _P]),
     "mn_unpack_bits": (c_int, [_P, _P, c_size_t, _P]),
     "mn_unpack_bits_mul_f32": (c_int, [_P, _P, _P, c_size_t, _P]),
@@ -74,6 +75,7 @@ _SIGNATURES = {
                                             c_int64, _P, c_size_t, c_uint32, c_uint32, c_uint32, c_uint32,
                                             _P]),
     "mn_bn_ws_status": (c_int, [_P, c_size_t, c_int64, c_int64, c_int64, _P]),
+    "mn_bn_wait_status": (c_int, [_P, _P]),
     "mn_bn_bwd_from_y_static_f32": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int64,
                                             c_int64, _P]),
     "mn_bn_relu_fwd_train_f32": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64,
@@ -152,8 +154,20 @@ def ptr(t):
     return None if t is None else t.data_ptr()
 
 
+_initialised = set()
+
+
 def stream_ptr(device=None):
-    """hipStream_t of torch's current stream on `device`."""
+    """hipStream_t of torch's current stream on `device`.  The first call for a device also
+    runs the library's per-device set-up (mn_init), so that no entry point has to do it on
+    its first call, which may be under stream capture."""
+    index = torch.cuda.current_device() if device is None else torch.device(device).index
+    if index is None:
+        index = torch.cuda.current_device()
+    if index not in _initialised:
+        with torch.cuda.device(index):
+            call("mn_init")
+        _initialised.add(index)
     return torch.cuda.current_stream(device).cuda_stream
 
 

@@ -5,6 +5,11 @@ extern "C" {
 
 int mn_abi_version(void) { return 1; }
 
+int mn_init(void) {
+  const bool bn = mn_bn_static_init(), wino = mn_wino_init();
+  return bn && wino ? MN_OK : MN_ELAUNCH;
+}
+
 const char* mn_status_string(int status) {
   switch (status) {
     case MN_OK:

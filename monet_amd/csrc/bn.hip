@@ -160,6 +160,7 @@ struct Args {
   float* pivot;         // [C], forward only
   uint32_t* ticket;     // resident launch only
   uint32_t* error;      // set to 1 by a wait that gave up; cleared by every launch
+  uint32_t* sticky;     // the device's own word, set with it and only cleared by mn_bn_wait_status
   uint32_t spin_limit;  // polls of one slot before the wait gives up
   float inv_m, unbias, momentum, eps;
   // Fused ReLU.  Forward: out = max(out, 0).  Backward from the input: the incoming gradient
@@ -464,7 +465,8 @@ constexpr int kMaxResident = 256;  // most pieces per channel in the resident fo
 // a fixed order (lane l takes slots l, l+64, ..; then a lane tree) and hands
 // the totals to the workgroup through `lds`.
 __device__ __forceinline__ void gather_totals(const uint64_t* slots, int S, float* lds, float& t0,
-                                              float& t1, uint32_t spin_limit, uint32_t* error) {
+                                              float& t1, uint32_t spin_limit, uint32_t* error,
+                                              uint32_t* sticky) {
   if (threadIdx.x < MN_WAVE) {
     const int lane = threadIdx.x;
     float p0 = 0.f, p1 = 0.f;
@@ -482,6 +484,7 @@ __device__ __forceinline__ void gather_totals(const uint64_t* slots, int S, floa
       if (w == kEmptySlot) {
         w = 0x7FC000007FC00000ull;
         __hip_atomic_store(error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (sticky) __hip_atomic_store(sticky, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
       p0 += __uint_as_float((uint32_t)w);
       p1 += __uint_as_float((uint32_t)(w >> 32));
@@ -616,7 +619,7 @@ __device__ __forceinline__ void finish_piece(const Args& A, const Held<VEC, KEEP
   if (!SOLO) {
     __syncthreads();  // lds is free again
     gather_totals(reinterpret_cast<uint64_t*>(A.partial) + (size_t)h.c * sh.S, sh.S, lds, t0, t1,
-                  A.spin_limit, A.error);
+                  A.spin_limit, A.error, A.sticky);
   }
   float s_, proj, gmean, gscale;
   coefficients<MODE>(A, h.c, h.piece, t0, t1, h.sft, s_, proj, gmean, gscale);
@@ -777,6 +780,26 @@ static int cache_hints(int64_t HW, int forced = 0) {
     }                                        \
   } while (0)
 
+// One word per device that every wait that gives up raises besides the word in its workspace
+// (workspaces are usually freed right after the call): mn_bn_wait_status reads and clears it.
+// In host code the name is a handle for hipGetSymbolAddress, not a device address.
+static __device__ uint32_t gave_up_word;
+
+static uint32_t* sticky_word() {
+  constexpr int kMaxDevices = 64;
+  static std::mutex lock;
+  static uint32_t* address[kMaxDevices] = {};
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> hold(lock);
+  if (!address[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(gave_up_word)) != hipSuccess) return nullptr;
+    address[dev] = static_cast<uint32_t*>(p);
+  }
+  return address[dev];
+}
+
 template <int MODE>
 static int run(Args& A, int64_t N, int64_t C, int64_t HW, bool aligned16, void* ws,
                const Tuning& t, hipStream_t s) {
@@ -787,6 +810,7 @@ static int run(Args& A, int64_t N, int64_t C, int64_t HW, bool aligned16, void* 
   A.pivot = reinterpret_cast<float*>(counters) - C;  // last C floats of the float area
   A.ticket = counters;
   A.error = counters + 1;
+  A.sticky = sticky_word();
   A.spin_limit = t.spin_limit ? t.spin_limit : 1u;
   int keep = t.keep > 0 ? t.keep : 8, threads = t.threads > 0 ? t.threads : kThreads;
   // The forward holds one tensor per piece: 512-thread workgroups (pieces twice as long, half as
@@ -1208,8 +1232,14 @@ int mn_bn_bwd_from_y_static_f32(const float* dy, const float* y, const float* ga
 int mn_bn_ws_status(const void* ws, size_t ws_bytes, int64_t N, int64_t C, int64_t HW,
                     mn_stream_t stream) {
   if (N <= 0 || C <= 0 || HW <= 0) return (N < 0 || C < 0 || HW < 0) ? MN_EINVAL : MN_OK;
-  if (!ws || !mn_bn::shape_limits(N, C, HW) || ws_bytes < mn_bn::ws_bytes_for(N, C, HW))
+  if (!mn_bn::shape_limits(N, C, HW)) return MN_EINVAL;
+  if (!ws) {   // the array of mn_bn_bwd_from_y_static_f32
+    if (mn_bn::ws_bytes_for(N, C, HW) > (size_t)MN_BN_STATIC_WS_BYTES) return MN_EINVAL;
+    ws = static_workspace();
+    if (!ws) return MN_ELAUNCH;
+  } else if (ws_bytes < mn_bn::ws_bytes_for(N, C, HW)) {
     return MN_EINVAL;
+  }
   const char* word = static_cast<const char*>(ws) + mn_bn::ws_floats(N, C, HW) * sizeof(float) +
                      sizeof(uint32_t);
   uint32_t raised = 0;
@@ -1220,4 +1250,26 @@ int mn_bn_ws_status(const void* ws, size_t ws_bytes, int64_t N, int64_t C, int64
   return raised ? MN_ELAUNCH : MN_OK;
 }
 
+int mn_bn_wait_status(uint32_t* host_word, mn_stream_t stream) {
+  uint32_t* word = mn_bn::sticky_word();
+  if (!word) return MN_ELAUNCH;
+  hipStream_t s = mn_stream(stream);
+  if (host_word)
+    return hipMemcpyAsync(host_word, word, sizeof(uint32_t), hipMemcpyDeviceToHost, s) == hipSuccess
+               ? MN_OK
+               : MN_ELAUNCH;
+  uint32_t raised = 0;
+  if (hipMemcpyAsync(&raised, word, sizeof(raised), hipMemcpyDeviceToHost, s) != hipSuccess ||
+      hipStreamSynchronize(s) != hipSuccess)
+    return MN_ELAUNCH;
+  if (raised && (hipMemsetAsync(word, 0, sizeof(uint32_t), s) != hipSuccess ||
+                 hipStreamSynchronize(s) != hipSuccess))
+    return MN_ELAUNCH;
+  return raised ? MN_ELAUNCH : MN_OK;
+}
+
 }  // extern "C"
+
+// Part of mn_init(): the address lookups of the static workspace and of the word
+// mn_bn_wait_status reads, for the current device.
+bool mn_bn_static_init() { return static_workspace() != nullptr && mn_bn::sticky_word() != nullptr; }

@@ -38,6 +38,12 @@ __device__ __forceinline__ float wave_sum(float v) {
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, MN_WAVE);
   return v;
 }
+
+// Per-device set-up that is not a stream operation (see mn_init); defined in bn.hip and
+// conv_wino.hip.  Both are idempotent and also run lazily from the entry points that need them.
+bool mn_bn_static_init();
+bool mn_wino_init();
+
 // Workgroups are handed to the 8 XCDs (each with its own L2) round-robin in launch order.
 // xcd_slot() turns a workgroup's launch index into a position in a LOGICAL order in which each
 // XCD runs one contiguous range: a kernel that decodes its tile from the slot, neighbours

@@ -772,6 +772,216 @@ __global__ __launch_bounds__(kThreads) void wgrad_reduce_bf16_kernel(
   dw[i] = f2bf(s);
 }
 
+// The large-tile form of backward-weight: eight wavefronts with two roles, as in the gather kernel.
+// A workgroup owns 64 TM output channels (rows, from dy) x 64 TN input channels (columns, from x) of
+// ONE tap and a range of the positions; wavefronts 0-3 multiply (2 x 2 of them, TM x TN accumulator
+// tiles of 32 x 32 each), wavefronts 4-7 feed.  Both tensors hold the channels of a position
+// contiguously while the matrix instruction wants 8 consecutive positions per lane: the feeders
+// copy 16-byte chunks into LDS unchanged ([position][channel], rows padded by 32 bytes) and the
+// multiplying wavefronts read the operands with the transposing LDS load (ds_read_b64_tr_b16: 16
+// lanes give the addresses of a 4-position x 16-channel block and lane i receives the 4 positions of
+// channel i), two per operand fragment.  No shuffles, byte permutes or 4-byte LDS stores, which is
+// what the kernel above spends its time on.  The partial sums of a workgroup go to the workspace in
+// the order the accumulators lie in registers (16 bytes per lane, a whole KB per instruction) and
+// `wgrad_roles_reduce_kernel` adds the ranges in a fixed order (reproducible).
+constexpr int kWrDepth = 64;   // positions per stage
+
+template <int TM, int TN>
+__global__ __launch_bounds__(kRoleThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void wgrad_roles_kernel(
+    const WGradH g, const bf16_t* __restrict__ dy, const bf16_t* __restrict__ x,
+    float* __restrict__ partial, uint32_t tiles, uint32_t stages_per_split) {
+  constexpr int BM = 64 * TM, BN = 64 * TN;
+  constexpr int LDA = BM + 16, LDB = BN + 16;      // elements per LDS row
+  constexpr int kLpr = 256 / kWrDepth;             // feeding threads per position
+  constexpr int kA = BM / 8 / kLpr, kB = BN / 8 / kLpr;   // 16-byte chunks per feeding thread and stage
+  constexpr uint32_t kBeyond = 0x80000000u;
+  typedef short short4_t __attribute__((ext_vector_type(4)));
+  typedef __attribute__((address_space(3))) short4_t* lds_frag_ptr;
+  __shared__ __attribute__((aligned(16))) bf16_t lds_a[2][kWrDepth][LDA];
+  __shared__ __attribute__((aligned(16))) bf16_t lds_b[2][kWrDepth][LDB];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // a contiguous range of slots per XCD: the workgroups of one range of positions (they read the
+  // same dy and x) lie under one L2
+  const uint32_t slot = xcd_slot();
+  const uint32_t split = slot / tiles, tile = slot - split * tiles;
+  const uint32_t tiles_n = (uint32_t)g.C / BN, tiles_m = (uint32_t)g.K / BM;
+  const uint32_t tn = tile % tiles_n, tm = (tile / tiles_n) % tiles_m, tap = tile / (tiles_n * tiles_m);
+  const uint32_t total = (g.depth + kWrDepth - 1) / kWrDepth;
+  const uint32_t t_begin = min(split * stages_per_split, total);
+  const uint32_t t_end = min(t_begin + stages_per_split, total);
+  const int stages = (int)(t_end - t_begin);
+
+  if (wave >= 4) {
+    // ------------------------------------------------------------------ feeding wavefronts
+    if (stages == 0) return;
+    const int ft = tid - 256;
+    const uint32_t row = ft / kLpr, c8 = ft % kLpr;   // position of the stage, first 16-byte chunk
+    const __amdgpu_buffer_rsrc_t dy_buf =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(dy), 0, g.dy_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t x_buf =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(x), 0, g.x_bytes, 0x00020000);
+    const uint32_t r = tap / g.S, sx = tap - r * g.S;
+    const int dh = (int)r * g.dH - g.pH, dw = (int)sx * g.dW - g.pW;
+    const uint32_t PQ = (uint32_t)g.P * g.Q;
+    // dy is [position][K]: a fixed byte offset per thread, the stage in the scalar offset;
+    // positions past the end of the reduction lie past the buffer and read as zero
+    const uint32_t a_off = (row * (uint32_t)g.K + tm * BM + c8 * 8) * 2u;
+    const uint32_t a_stage = kWrDepth * (uint32_t)g.K * 2u;
+    // x: this thread's position (image, p, q), carried from stage to stage by additions
+    uint32_t d = t_begin * kWrDepth + row, bp, bq, img_off;
+    {
+      const uint32_t n = d / PQ, pq = d - n * PQ;
+      bp = pq / g.Q;
+      bq = pq - bp * g.Q;
+      img_off = n * (uint32_t)g.H * g.W * (uint32_t)g.C * 2u;
+    }
+    const uint32_t kq = kWrDepth / (uint32_t)g.Q, rq = kWrDepth - kq * g.Q;
+    const uint32_t img_bytes = (uint32_t)g.H * g.W * (uint32_t)g.C * 2u;
+    const uint32_t b_chan = (tn * BN + c8 * 8) * 2u;
+    uint32_t t = t_begin;
+    constexpr int kSets = kWrDepth == 32 ? 4 : 2;   // register sets = stages the loads run ahead of the LDS writes
+    uint4_t ra[kSets][kA], rb[kSets][kB];
+    auto fetch = [&](uint4_t (&qa)[kA], uint4_t (&qb)[kB]) {
+      const int so = __builtin_amdgcn_readfirstlane((int)(t * a_stage));
+#pragma unroll
+      for (int i = 0; i < kA; ++i)
+        qa[i] = __builtin_amdgcn_raw_buffer_load_b128(dy_buf, a_off + i * (16 * kLpr), so, 0);
+      const int hh = (int)__umul24(bp, (uint32_t)g.sH) + dh, ww = (int)__umul24(bq, (uint32_t)g.sW) + dw;
+      const bool ok = d < g.depth && (unsigned)hh < (unsigned)g.H && (unsigned)ww < (unsigned)g.W;
+      const uint32_t pix = __umul24((uint32_t)hh, (uint32_t)g.W) + (uint32_t)ww;
+      const uint32_t b_off = ok ? img_off + pix * (uint32_t)g.C * 2u + b_chan : kBeyond;
+#pragma unroll
+      for (int i = 0; i < kB; ++i)
+        qb[i] = __builtin_amdgcn_raw_buffer_load_b128(x_buf, b_off + i * (16 * kLpr), 0, 0);
+      ++t;
+      d += kWrDepth;
+      bq += rq;
+      bp += kq;
+      if (bq >= (uint32_t)g.Q) {
+        bq -= g.Q;
+        ++bp;
+      }
+      while (bp >= (uint32_t)g.P) {
+        bp -= g.P;
+        img_off += img_bytes;
+      }
+    };
+    auto stage = [&](int buf, const uint4_t (&qa)[kA], const uint4_t (&qb)[kB]) {
+#pragma unroll
+      for (int i = 0; i < kA; ++i)
+        *reinterpret_cast<uint4_t*>(&lds_a[buf][row][(c8 + kLpr * i) * 8]) = qa[i];
+#pragma unroll
+      for (int i = 0; i < kB; ++i)
+        *reinterpret_cast<uint4_t*>(&lds_b[buf][row][(c8 + kLpr * i) * 8]) = qb[i];
+    };
+#pragma unroll
+    for (int k = 0; k < kSets; ++k)
+      if (k < stages) fetch(ra[k], rb[k]);
+    stage(0, ra[0], rb[0]);
+    if (kSets < stages) fetch(ra[0], rb[0]);
+    __syncthreads();
+    for (int s2 = 0; s2 < stages; s2 += kSets) {
+#pragma unroll
+      for (int u = 0; u < kSets; ++u) {
+        if (s2 + u >= stages) break;
+        const int k = (u + 1) % kSets;   // register set of stage s2 + u + 1
+        if (s2 + u + 1 < stages) stage((u + 1) & 1, ra[k], rb[k]);
+        if (s2 + u + 1 + kSets < stages) fetch(ra[k], rb[k]);
+        __syncthreads();
+      }
+    }
+    return;
+  }
+
+  // -------------------------------------------------------------------- multiplying wavefronts
+  const int wm = wave >> 1, wn = wave & 1;
+  // the lane's address inside a 16-position x 32-channel fragment: 16 lanes cover 4 positions x 16
+  // channels; lanes 32-63 hold the second half of the 16 positions of a matrix step
+  const int l16 = lane & 15, grp = lane >> 4;
+  const int pix0 = 8 * (grp >> 1) + (l16 >> 2), chan0 = 16 * (grp & 1) + 4 * (l16 & 3);
+  const bf16_t* pa = &lds_a[0][pix0][wm * (TM * 32) + chan0];
+  const bf16_t* pb = &lds_b[0][pix0][wn * (TN * 32) + chan0];
+  float16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+  if (stages > 0) __syncthreads();   // stage 0 is in LDS
+  for (int s2 = 0; s2 < stages; ++s2) {
+    const bf16_t* qa = pa + (s2 & 1) * (kWrDepth * LDA);
+    const bf16_t* qb = pb + (s2 & 1) * (kWrDepth * LDB);
+#pragma unroll
+    for (int ks = 0; ks < kWrDepth; ks += 16) {
+      bf16x8 af[TM], bfr[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_frag_ptr)(qa + ks * LDA + 32 * i));
+        const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_frag_ptr)(qa + (ks + 4) * LDA + 32 * i));
+        af[i] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      }
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_frag_ptr)(qb + ks * LDB + 32 * j));
+        const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_frag_ptr)(qb + (ks + 4) * LDB + 32 * j));
+        bfr[j] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+  // registers as they lie: unit ((slot * 4 + wave) * TM * TN * 4 + (i * TN + j) * 4 + a) * 64 + lane
+  // holds acc[i][j][4a .. 4a + 3]
+  float4* out = reinterpret_cast<float4*>(partial) +
+                ((size_t)slot * 4 + wave) * (TM * TN * 4 * 64) + lane;
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+        out[((i * TN + j) * 4 + a) * 64] =
+            make_float4(acc[i][j][4 * a], acc[i][j][4 * a + 1], acc[i][j][4 * a + 2], acc[i][j][4 * a + 3]);
+}
+
+// dw[k][tap][c] = sum over the ranges of positions, in order; one thread per 16-byte unit of a
+// range (four consecutive output channels k of one input channel c)
+template <int TM, int TN>
+__global__ __launch_bounds__(kThreads) void wgrad_roles_reduce_kernel(
+    const float4* __restrict__ partial, bf16_t* __restrict__ dw, uint32_t units, int splits, int K,
+    int C, int T) {
+  constexpr int BM = 64 * TM, BN = 64 * TN;
+  const uint32_t u = blockIdx.x * kThreads + threadIdx.x;
+  if (u >= units) return;
+  float4 s = partial[u];
+  for (int z = 1; z < splits; ++z) {
+    const float4 v = partial[(size_t)z * units + u];
+    s.x += v.x;
+    s.y += v.y;
+    s.z += v.z;
+    s.w += v.w;
+  }
+  const uint32_t lane = u & 63, a = (u >> 6) & 3, ij = (u >> 8) % (TM * TN);
+  const uint32_t wave = (u / (256 * TM * TN)) & 3, tile = u / (1024 * TM * TN);
+  const uint32_t i = ij / TN, j = ij - i * TN;
+  const uint32_t tiles_n = (uint32_t)C / BN, tiles_m = (uint32_t)K / BM;
+  const uint32_t tn = tile % tiles_n, tm = (tile / tiles_n) % tiles_m, tap = tile / (tiles_n * tiles_m);
+  const uint32_t k = tm * BM + (wave >> 1) * (TM * 32) + 32 * i + 8 * a + 4 * (lane >> 5);
+  const uint32_t c = tn * BN + (wave & 1) * (TN * 32) + 32 * j + (lane & 31);
+  const size_t row = (size_t)T * C;
+  bf16_t* o = dw + (size_t)k * row + (size_t)tap * C + c;
+  o[0] = f2bf(s.x);
+  o[row] = f2bf(s.y);
+  o[2 * row] = f2bf(s.z);
+  o[3 * row] = f2bf(s.w);
+}
+
 // ----------------------------------------------------------------------- host
 static int check16(const mn_conv2d* g) {
   // every tensor is addressed with 32-bit element offsets
@@ -883,6 +1093,38 @@ static void wgrad16_split(const mn_conv2d* g, int* splits, int* tiles_per_split)
   if (*splits < 1) *splits = 1;
 }
 
+// The large-tile backward-weight (variant 1): channel counts that are multiples of 128 and a
+// reduction long enough to share out.  tm / tn = accumulator tiles per wavefront along K / C;
+// splits = ranges of positions, one workgroup per (tile, range), about one workgroup per CU.
+struct WgradRoles {
+  int tm, tn;
+  uint32_t tiles, splits, stages_per_split;
+};
+
+static bool wgrad16_roles(const mn_conv2d* g, WgradRoles* r) {
+  if (g->K % 128 != 0 || g->C % 128 != 0) return false;
+  const long long depth = (long long)g->N * g->P * g->Q;
+  if (depth < 4096) return false;
+  // 128 accumulation registers per lane: a wavefront has 256 registers in all at two per SIMD
+  r->tm = g->K % 256 == 0 ? 4 : 2;
+  r->tn = r->tm == 2 && g->C % 256 == 0 ? 4 : 2;
+  const long long tiles = (long long)g->R * g->S * (g->K / (64 * r->tm)) * (g->C / (64 * r->tn));
+  if (tiles > 65535) return false;
+  int dev = 0, cus = 256;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+    cus = 256;
+  const long long total = (depth + kWrDepth - 1) / kWrDepth;
+  long long splits = cus / tiles;
+  if (splits < 1) splits = 1;
+  if (splits > total / 4) splits = total / 4 > 0 ? total / 4 : 1;
+  const long long per = (total + splits - 1) / splits;
+  r->tiles = (uint32_t)tiles;
+  r->stages_per_split = (uint32_t)per;
+  r->splits = (uint32_t)((total + per - 1) / per);
+  return true;
+}
+
 }  // namespace mn_conv16
 
 // Entry points used by the dtype dispatch in conv.hip.
@@ -904,6 +1146,11 @@ int mn_conv16_ws_bytes(const mn_conv2d* g, int direction, int variant, size_t* b
     return MN_OK;
   }
   if (g->K % 64 != 0 || g->C % 64 != 0) return MN_EUNSUPPORTED;
+  WgradRoles wr;
+  if (variant == 1 && wgrad16_roles(g, &wr)) {
+    *bytes = (size_t)wr.splits * g->K * g->C * g->R * g->S * sizeof(float);
+    return MN_OK;
+  }
   int splits, tps;
   wgrad16_split(g, &splits, &tps);
   if (splits > 1) *bytes = (size_t)splits * g->K * g->C * g->R * g->S * sizeof(float);
@@ -1055,6 +1302,26 @@ int mn_conv16_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, void
   if (dy_bytes >= (1ull << 31) || x_bytes >= (1ull << 31)) return MN_EUNSUPPORTED;
   q.dy_bytes = (uint32_t)dy_bytes;
   q.x_bytes = (uint32_t)x_bytes;
+  WgradRoles wr;
+  if (variant == 1 && wgrad16_roles(g, &wr)) {
+    const size_t nw = (size_t)g->K * g->C * q.T;
+    if (!ws || ws_bytes < nw * sizeof(float) * wr.splits || !mn_aligned(ws, 16)) return MN_EINVAL;
+    const unsigned grid = wr.tiles * wr.splits;
+    const uint32_t units = (uint32_t)(nw / 4);
+    const unsigned rgrid = (units + kThreads - 1) / kThreads;
+#define MN_WGRAD_ROLES(TM_, TN_)                                                                  \
+  do {                                                                                            \
+    wgrad_roles_kernel<TM_, TN_><<<grid, kRoleThreads, 0, s>>>(                                   \
+        q, (const bf16_t*)dy, (const bf16_t*)x, (float*)ws, wr.tiles, wr.stages_per_split);       \
+    wgrad_roles_reduce_kernel<TM_, TN_><<<rgrid, kThreads, 0, s>>>(                               \
+        (const float4*)ws, (bf16_t*)dw, units, (int)wr.splits, g->K, g->C, q.T);                  \
+  } while (0)
+    if (wr.tm == 4) MN_WGRAD_ROLES(4, 2);
+    else if (wr.tn == 4) MN_WGRAD_ROLES(2, 4);
+    else MN_WGRAD_ROLES(2, 2);
+#undef MN_WGRAD_ROLES
+    return mn_launch_status();
+  }
   int splits, tps, bm, bn;
   wgrad16_split(g, &splits, &tps);
   wgrad16_tiles(g, &bm, &bn);

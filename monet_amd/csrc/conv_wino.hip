@@ -781,6 +781,9 @@ static bool shape_ok(const mn_conv2d* g) {
 
 }  // namespace mn_wino
 
+// Part of mn_init(): the LDS limit of the one-kernel form, for the current device.
+bool mn_wino_init() { return mn_wino::fused_lds_allowed(); }
+
 // Entry points used by conv.hip (all fp32).  `bytes` = 0 and MN_EUNSUPPORTED when the shape is
 // not a 3x3 / stride 1 / dilation 1 convolution with a reduction over a multiple of 16 channels.
 int mn_wino_ws_bytes(const mn_conv2d* g, bool backward_data, size_t* bytes) {

@@ -47,6 +47,46 @@ def _workspace(N, C, HW, device):
 check_waits = os.environ.get("MONET_AMD_CHECK_BN_WAITS", "0") not in ("", "0")
 
 
+class _WaitMonitor:
+    """Looks, without waiting for the device, whether a BatchNorm wait gave up (the results are
+    NaN then): `poll` enqueues a 4-byte copy of the device's give-up word into pinned host
+    memory and looks at the copy the previous poll enqueued once that has arrived, so a give-up
+    raises one poll late.  One per device; the schedule executor polls once per step."""
+
+    def __init__(self, device):
+        self.device = device
+        self.word = torch.zeros(1, dtype=torch.int32).pin_memory()
+        self.event = None
+
+    def poll(self):
+        if self.event is not None:
+            if not self.event.query():
+                return      # the previous copy is still on its way
+            self.event = None
+            if int(self.word[0]) != 0:
+                self.word.zero_()
+                # the synchronous form clears the device's word (and reports it as MN_ELAUNCH)
+                _lib.load().mn_bn_wait_status(None, _lib.stream_ptr(self.device))
+                raise RuntimeError(
+                    "a BatchNorm kernel gave up waiting for the other workgroups of its channel: "
+                    "the results of that call are NaN (the device ran fewer workgroups at once "
+                    "than the launch relies on)")
+        _lib.call("mn_bn_wait_status", self.word.data_ptr(), _lib.stream_ptr(self.device))
+        self.event = torch.cuda.Event()
+        self.event.record(torch.cuda.current_stream(self.device))
+
+
+_monitors = {}
+
+
+def poll_waits(device):
+    """See _WaitMonitor; `device` is a torch.device of type cuda."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    if index not in _monitors:
+        _monitors[index] = _WaitMonitor(torch.device("cuda", index))
+    _monitors[index].poll()
+
+
 def _ws_call(ws_shape, name, *args):
     _lib.call(name, *args)
     if check_waits:

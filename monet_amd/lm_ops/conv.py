@@ -187,12 +187,19 @@ def _depthwise_forward(input_, weight, bias, stride, padding, dilation, groups):
 def _depthwise_backward(grad, input_, weight, stride, padding, dilation, groups, mask,
                         input_shape=None):
     """(di, dw) of a grouped convolution through aten.  `mask` says which of the two to
-    compute; an input the executor has already dropped (input-gradient step of a split
-    backward) is replaced by a shape-only stand-in, which is all aten reads of it then."""
+    compute.  When the executor has already dropped the input (input-gradient step of a split
+    backward) di is the transposed convolution of the gradient, which reads no input at all:
+    handing aten.convolution_backward a shape-only stand-in would make it materialise a
+    full-size copy of it, memory the schedule counts as free."""
     if input_ is None:
         assert not mask[1] and input_shape is not None
-        input_ = torch.empty(1, dtype=grad.dtype, device=grad.device).expand(
-            [int(d) for d in input_shape])
+        spatial = [int(d) for d in input_shape[2:]]
+        out_pad = [spatial[i] - ((grad.shape[2 + i] - 1) * stride[i] - 2 * padding[i] +
+                                 dilation[i] * (weight.shape[2 + i] - 1) + 1)
+                   for i in range(len(spatial))]
+        di = torch.nn.functional.conv_transpose2d(grad, weight, None, list(stride), list(padding),
+                                                  out_pad, groups, list(dilation))
+        return di, None
     di, dw, _ = torch.ops.aten.convolution_backward(
         grad, input_, weight, None, list(stride), list(padding), list(dilation), False, [0, 0],
         groups, [bool(mask[0]), bool(mask[1]), False])

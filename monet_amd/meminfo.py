@@ -15,6 +15,7 @@ Each returns one entry per kernel variant for convolutions in "conv" modes
 switch in "inplace" modes, first-forward and recompute-forward entries for
 BatchNorm, and a single entry otherwise.
 """
+import gc
 from time import time
 
 import numpy as np
@@ -115,6 +116,7 @@ def _timed(fn, samples=RUNTIME_SAMPLES, rounds=3):
 
 def _peak_over_outputs(fn):
     """(workspace bytes, outputs) of one call: allocator peak minus returned bytes."""
+    gc.collect()   # garbage that is only freed during the call would be taken off its peak
     torch.cuda.empty_cache()
     torch.cuda.reset_peak_memory_stats()
     before = torch.cuda.memory_stats()['allocated_bytes.all.peak']

@@ -29,11 +29,12 @@ to `.grad` directly instead of through the autograd engine.
 """
 import copy
 import pickle
-from collections import defaultdict, namedtuple
+from collections import OrderedDict, defaultdict, namedtuple
 
 import torch
 
 from . import lm_ops
+from .lm_ops import bn as bn_ops
 from .graph import ComputeNode, Graph, is_batch_norm, two_step_backward
 from .solver_info import BwdNode, IntNode, SolverInfo
 
@@ -405,6 +406,10 @@ class Schedule(Graph):
         self._shared.clear()
         for op in self._ops0:
             op.params = None
+        # once per step, without waiting for the device: did a BatchNorm kernel give up a wait
+        # (its results are NaN then)?  Raises one step late.
+        if delta_x.is_cuda:
+            bn_ops.poll_waits(delta_x.device)
 
 
 def disable_dropout(model):
@@ -420,22 +425,49 @@ def load_solution(filename):
     return si, solution
 
 
-# traced graphs by (architecture, parameter shapes, input shape, fusion level): tracing runs the
-# model once on the CPU (tens of seconds for a UNet at full resolution), and a graph holds
-# structure only, so wrappers of the same architecture share it
-_graph_cache = {}
+# Traced graphs by (architecture, parameter shapes, plain attributes of every module, input
+# shape, fusion level, training flags): tracing runs the model once on the CPU (tens of seconds
+# for a UNet at full resolution), and a graph holds structure only, so wrappers of the same
+# architecture share it.  The assumption is that the traced graph depends on nothing else; a
+# model whose forward() branches on state the key does not see (a global, a tensor's value) must
+# not be traced through this cache (`cache=False`).  The eight most recently used graphs are kept.
+_graph_cache = OrderedDict()
+_GRAPH_CACHE_SIZE = 8
 
 
-def _traced_graph(model, input_shape, fuse_level):
-    key = (type(model).__module__, type(model).__qualname__, repr(model),
-           tuple((k, tuple(v.shape)) for k, v in model.state_dict().items()),
-           tuple(input_shape), int(fuse_level),
-           tuple(bool(mod.training) for mod in model.modules()))
-    if key not in _graph_cache:
+def _plain_attributes(model):
+    """(module path, attribute, repr) of every public attribute of a module that is a number, a
+    string, None or a flat tuple / list of those: what repr(model) may leave out and forward()
+    may read (UNet's target height and width, a flag)."""
+    plain = (bool, int, float, str, type(None))
+    out = []
+    for path, mod in model.named_modules():
+        for k, v in sorted(vars(mod).items()):
+            if k.startswith("_") or k == "training":
+                continue
+            if isinstance(v, plain) or (isinstance(v, (tuple, list)) and
+                                        all(isinstance(e, plain) for e in v)):
+                out.append((path, k, repr(v)))
+    return tuple(out)
+
+
+def _traced_graph(model, input_shape, fuse_level, cache=True):
+    def trace():
         m = copy.deepcopy(model)
         m.cpu()
-        _graph_cache[key] = Graph.create(m, input_shape, fuse_bn_relu=fuse_level)
-        del m
+        return Graph.create(m, input_shape, fuse_bn_relu=fuse_level)
+    if not cache:
+        return trace()
+    key = (type(model).__module__, type(model).__qualname__, repr(model),
+           tuple((k, tuple(v.shape)) for k, v in model.state_dict().items()),
+           _plain_attributes(model), tuple(input_shape), int(fuse_level),
+           tuple(bool(mod.training) for mod in model.modules()))
+    if key in _graph_cache:
+        _graph_cache.move_to_end(key)
+    else:
+        _graph_cache[key] = trace()
+        while len(_graph_cache) > _GRAPH_CACHE_SIZE:
+            _graph_cache.popitem(last=False)
     return _graph_cache[key]
 
 

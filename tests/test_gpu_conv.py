@@ -257,6 +257,10 @@ BF16_CASES = [
     ((80, 64, 15, 15), (192, 64, 3, 3), 2, 1, 1),
     ((23, 128, 14, 14), (128, 128, 5, 5), 1, 2, 1),
     ((34, 128, 12, 12), (320, 128, 1, 1), 1, 0, 1),
+    # backward-weight variant 1 with feeding and multiplying wavefronts (both channel counts
+    # multiples of 128, more than 4096 positions): 128 x 256 tiles, and strided with odd planes
+    ((12, 256, 20, 20), (128, 256, 3, 3), 1, 1, 1),
+    ((40, 128, 23, 21), (384, 128, 3, 3), 2, 1, 1),
 ]
 
 
@@ -293,9 +297,9 @@ def test_conv_bf16_all_directions(cuda, xs, ws, st, pad, dil):
         dw = conv_ops.conv_backward_weight(ws, dev16(dy, cuda), dev16(x, cuda), pad, st, dil, 1, v)
         assert dw.dtype == torch.bfloat16 and list(dw.shape) == list(ws)
         assert_rel(host(dw.float()), exp_dw, BF16_TOL, f"bf16 backward-weight variant {v}")
-    # reproducible: fixed-order reduction of the split partials
-    dw2 = conv_ops.conv_backward_weight(ws, dev16(dy, cuda), dev16(x, cuda), pad, st, dil, 1, 0)
-    assert torch.equal(dw, dw2)
+        # reproducible: fixed-order reduction of the split partials
+        dw2 = conv_ops.conv_backward_weight(ws, dev16(dy, cuda), dev16(x, cuda), pad, st, dil, 1, v)
+        assert torch.equal(dw, dw2)
     # there is no bf16 Winograd tier
     assert refused(lambda: conv_ops.conv_forward(dev16(x, cuda), dev16(w, cuda), None, pad, st, dil, 1, 2))
 

@@ -191,6 +191,9 @@ def resnet50_case(cuda):
     return model, x, loss_fn, g64, g32, l64
 
 
+_UNCONSTRAINED = {}   # mode -> (gradients, loss, output, choices) of the 100 GB schedule
+
+
 @pytest.mark.parametrize("budget", [10, 6])
 @pytest.mark.parametrize("mode", ["inplace_conv_multiway_newnode", "fused_inplace_conv_multiway_newnode",
                                   "fused2_inplace_conv_multiway_newnode"])
@@ -202,29 +205,26 @@ def test_resnet50_batch_184_under_the_committed_schedules(cuda, resnet50_case, m
     what stock fp32 autograd is (plus 1e-5): deep-layer gradients of a random-init ResNet-50
     differ by percents between any two fp32 summation orders, so float64 is the only yardstick
     that says anything."""
-    import copy
     import os
-    from grad_check import assert_no_worse_than_stock
-    from monet_amd.monet_wrapper import MONeTWrapper
+    from grad_check import (assert_no_worse_than_stock, assert_same_as_unconstrained,
+                            run_schedule, schedule_choices)
     model, x, loss_fn, g64, g32, l64 = resnet50_case
-    sol = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "data",
-                       "solution_resnet50_184_%s_%d.00.pkl" % (mode, budget))
-    wrapped = MONeTWrapper(copy.deepcopy(model), sol, (3, 224, 224)).to(cuda)
-    wrapped.train()
-    own = sum(t.numel() * t.element_size() for t in wrapped.state_dict().values()) + \
-        x.numel() * x.element_size()
-    torch.cuda.synchronize()
-    torch.cuda.empty_cache()
-    others = torch.cuda.memory_allocated() - own     # what the fixture keeps on the device
-    torch.cuda.reset_peak_memory_stats()
-    loss = loss_fn(wrapped(x))
-    loss.backward()
-    torch.cuda.synchronize()
-    peak_mb = (torch.cuda.max_memory_allocated() - others) / 2 ** 20
-    print("ResNet-50 %s %d GB: peak %.1f MiB, loss %.9f" % (mode, budget, peak_mb, float(loss)),
-          flush=True)
+    data = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "data")
+    if mode not in _UNCONSTRAINED:
+        w0, g0, l0, _, o0 = run_schedule(cuda, model, x, loss_fn, os.path.join(
+            data, "solution_resnet50_184_%s_100.00.pkl" % mode), (3, 224, 224))
+        _UNCONSTRAINED[mode] = ({k: v.cpu() for k, v in g0.items()}, l0, o0, schedule_choices(w0))
+        del w0, g0
+    sol = os.path.join(data, "solution_resnet50_184_%s_%d.00.pkl" % (mode, budget))
+    wrapped, got, loss, peak_mb, out = run_schedule(cuda, model, x, loss_fn, sol, (3, 224, 224))
+    print("ResNet-50 %s %d GB: peak %.1f MiB, loss %.9f" % (mode, budget, peak_mb, loss), flush=True)
     assert peak_mb <= budget * 1024, peak_mb
-    assert abs(float(loss.detach()) - l64) < 1e-5 * max(1.0, abs(l64))
-    got = {k: p.grad.detach() for k, p in wrapped.model.named_parameters()}
+    assert abs(loss - l64) < 1e-5 * max(1.0, abs(l64))
     assert set(got) == set(g64) and all(bool(torch.isfinite(g).all()) for g in got.values())
     assert_no_worse_than_stock(got, g32, g64, "ResNet-50 %s %d GB" % (mode, budget))
+    # the budgeted schedule against the unconstrained one of the same operator set
+    ref_got, ref_loss, ref_out, ref_choices = _UNCONSTRAINED[mode]
+    assert_same_as_unconstrained(
+        (got, loss, out, schedule_choices(wrapped)),
+        ({k: v.to(cuda) for k, v in ref_got.items()}, ref_loss, ref_out, ref_choices), g64,
+        "ResNet-50 %s %d GB" % (mode, budget))

@@ -48,9 +48,12 @@ def test_batchnorm_wait_that_gives_up_is_reported(cuda):
     ws = torch.empty(nbytes, dtype=torch.uint8, device=cuda)
     status = lambda: _lib.load().mn_bn_ws_status(_lib.ptr(ws), nbytes, N, C, HW,
                                                  _lib.stream_ptr(cuda))
+    # the device's own word (for callers whose workspace is gone after the call): clear so far
+    device_word = lambda: _lib.load().mn_bn_wait_status(None, _lib.stream_ptr(cuda))
+    assert device_word() == _lib.MN_OK
     # default limits: everything arrives
     dx0, dg0, db0 = _from_y_with_limits(y, gamma, beta, invstd, dy, ws, 0, 0)
-    assert status() == _lib.MN_OK
+    assert status() == _lib.MN_OK and device_word() == _lib.MN_OK
     ref = bn_ops.bn_backward_from_output(dy, y, gamma, beta, invstd)
     assert torch.equal(dx0, ref[0]) and torch.equal(dg0, ref[1]) and torch.equal(db0, ref[2])
     # two workgroups, eight polls: the wait gives up
@@ -65,6 +68,22 @@ def test_batchnorm_wait_that_gives_up_is_reported(cuda):
     # the next launch on the same workspace starts clean
     dx2, dg2, db2 = _from_y_with_limits(y, gamma, beta, invstd, dy, ws, 0, 0)
     assert status() == _lib.MN_OK
+    # ... while the device's word stays raised until it is asked for: the executor's monitor
+    # (one non-blocking poll per step) raises on the poll after the one that fetched it
+    bn_ops.poll_waits(cuda)
+    torch.cuda.synchronize()
+    with pytest.raises(RuntimeError, match="gave up waiting"):
+        bn_ops.poll_waits(cuda)
+    assert device_word() == _lib.MN_OK          # cleared by the monitor
+    bn_ops.poll_waits(cuda)
+    torch.cuda.synchronize()
+    bn_ops.poll_waits(cuda)                     # and quiet again
+    # the entry point with the library's own array answers the same question with ws == NULL
+    _lib.call("mn_bn_bwd_from_y_static_f32", _lib.ptr(dy), _lib.ptr(y), _lib.ptr(gamma),
+              _lib.ptr(beta), _lib.ptr(invstd), _lib.ptr(dx2), _lib.ptr(dg2), _lib.ptr(db2), N, C, HW,
+              _lib.stream_ptr(cuda))
+    assert _lib.load().mn_bn_ws_status(None, 0, N, C, HW, _lib.stream_ptr(cuda)) == _lib.MN_OK
+    assert torch.equal(dx2, dx0) and torch.equal(dg2, dg0)
     assert torch.equal(dx2, dx0) and torch.equal(dg2, dg0) and torch.equal(db2, db0)
     # the operator classes check after every call when asked to
     bn_ops.check_waits = True

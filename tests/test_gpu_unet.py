@@ -10,7 +10,8 @@ import os
 import pytest
 import torch
 
-from grad_check import assert_no_worse_than_stock, stock_gradients
+from grad_check import (assert_no_worse_than_stock, assert_same_as_unconstrained, run_schedule,
+                        schedule_choices, stock_gradients)
 
 pytestmark = pytest.mark.gpu
 
@@ -37,36 +38,33 @@ def unet_case(cuda):
     return model, shape, x, labels, loss_fn, g64, g32, l64
 
 
+_UNCONSTRAINED = {}   # mode -> (gradients, loss, output, choices) of the 100 GB schedule
+
+
 @pytest.mark.parametrize("budget", [10, 6])
 @pytest.mark.parametrize("mode", ["inplace_conv_multiway_newnode",
                                   "fused_inplace_conv_multiway_newnode"])
 def test_unet_batch_11_under_the_committed_schedules(cuda, unet_case, mode, budget):
-    import copy
     from monet_amd.graph import ComputeNode
-    from monet_amd.monet_wrapper import MONeTWrapper
     model, shape, x, labels, loss_fn, g64, g32, l64 = unet_case
+    if mode not in _UNCONSTRAINED:
+        w0, g0, l0, _, o0 = run_schedule(cuda, model, x, loss_fn, os.path.join(
+            DATA, "solution_unet_%d_%s_100.00.pkl" % (BS, mode)), tuple(shape))
+        _UNCONSTRAINED[mode] = ({k: v.cpu() for k, v in g0.items()}, l0, o0, schedule_choices(w0))
+        del w0, g0
     sol = os.path.join(DATA, "solution_unet_%d_%s_%d.00.pkl" % (BS, mode, budget))
-    wrapped = MONeTWrapper(copy.deepcopy(model), sol, tuple(shape)).to(cuda)
-    wrapped.train()
+    # weights + batch + activations + workspaces + parameter gradients + the loss's own tensors
+    wrapped, got, loss, peak_mb, out = run_schedule(cuda, model, x, loss_fn, sol, tuple(shape))
     ops = {n.op for n in wrapped.schedule[0].nodes if isinstance(n, ComputeNode)}
     assert {"aten::cat", "aten::adaptive_avg_pool2d", "aten::max_pool2d"} <= ops
     assert wrapped.schedule[0].solution.r[1:].sum() > 0 or budget == 10  # 6 GB recomputes
-
-    own = sum(t.numel() * t.element_size() for t in wrapped.state_dict().values()) + \
-        x.numel() * x.element_size()
-    torch.cuda.synchronize()
-    torch.cuda.empty_cache()
-    others = torch.cuda.memory_allocated() - own     # the fixture's references, labels, ...
-    torch.cuda.reset_peak_memory_stats()
-    loss = loss_fn(wrapped(x))
-    loss.backward()
-    torch.cuda.synchronize()
-    # weights + batch + activations + workspaces + parameter gradients + the loss's own tensors
-    peak_mb = (torch.cuda.max_memory_allocated() - others) / 2**20
-    print("UNet %s %d GB: peak %.1f MiB, loss %.9f" % (mode, budget, peak_mb, float(loss)),
-          flush=True)
+    print("UNet %s %d GB: peak %.1f MiB, loss %.9f" % (mode, budget, peak_mb, loss), flush=True)
     assert peak_mb <= budget * 1024, peak_mb
-    assert abs(float(loss.detach()) - l64) < 1e-5 * max(1.0, abs(l64))
-    got = {n: p.grad.detach() for n, p in wrapped.model.named_parameters()}
+    assert abs(loss - l64) < 1e-5 * max(1.0, abs(l64))
     assert set(got) == set(g64) and all(bool(torch.isfinite(g).all()) for g in got.values())
     assert_no_worse_than_stock(got, g32, g64, "UNet %s %d GB" % (mode, budget))
+    ref_got, ref_loss, ref_out, ref_choices = _UNCONSTRAINED[mode]
+    assert_same_as_unconstrained(
+        (got, loss, out, schedule_choices(wrapped)),
+        ({k: v.to(cuda) for k, v in ref_got.items()}, ref_loss, ref_out, ref_choices), g64,
+        "UNet %s %d GB" % (mode, budget))
