@@ -351,6 +351,8 @@ def mfma_summary(pmc_dir, bench_stdout):
         raise SystemExit("%d marked segments for %d entries" % (len(segments), len(order)))
     entries = {}
     for name, seg in zip(order, segments):
+        if name.endswith("/probe"):
+            continue
         f32 = sum(d.get("SQ_INSTS_VALU_MFMA_MOPS_F32", 0.0) for d in seg) * 512.0 / calls
         b16 = sum(d.get("SQ_INSTS_VALU_MFMA_MOPS_BF16", 0.0) for d in seg) * 512.0 / calls
         busy = sum(d.get("SQ_VALU_MFMA_BUSY_CYCLES", 0.0) for d in seg)
@@ -412,8 +414,11 @@ def conv_bench(steps, warmup):
             out["frac_mfma"] = None
         return out
 
-    def runs(fn, n):
-        """Variants of one direction that take this shape: {variant: callable}."""
+    def runs(path, fn, n):
+        """Variants of one direction that take this shape: {variant: callable}.  The trial calls
+        get a marker and an entry of their own ("/probe"), which the counter summary drops."""
+        torch.cuda._sleep(1)
+        order.append(path + "/probe")
         ok = {}
         for v in range(n):
             try:
@@ -437,13 +442,15 @@ def conv_bench(steps, warmup):
         }
         for d in which:
             n, fn = table[d]
-            for v, call in runs(fn, n).items():
+            for v, call in runs(prefix + d, fn, n).items():
                 key = "%s_v%d" % (d, v)
                 out[key] = timed(prefix + key, call, flops)
         out["flops_per_call"] = flops
         return out
 
     def problem(g):
+        torch.cuda._sleep(1)            # the set-up work is nobody's entry
+        order.append("setup/probe")
         x = torch.randn(g["N"], g["C"], g["H"], g["W"], device=dev)
         w = torch.randn(g["K"], g["C"], g["R"], g["S"], device=dev) * (2.0 / (g["K"] * g["R"] * g["S"])) ** 0.5
         y = cv.conv_forward(x, w, None, g["pad"], g["stride"], 1, 1, 0)
@@ -473,7 +480,7 @@ def conv_bench(steps, warmup):
     res["unet_128ch_208x304"] = {"shape": u}
     res["unet_128ch_208x304"].update(directions("unet_128ch_208x304/", u, x, w, dy, ("fwd",)))
     res["order"] = order
-    res["calls_per_entry"] = steps + warmup + 1   # + the call that finds out whether a variant applies
+    res["calls_per_entry"] = steps + warmup
     return res
 
 

@@ -334,12 +334,15 @@ __global__ __launch_bounds__(kThreads) void gather_bf16_kernel(const GatherH g,
 // after the other on all of them, and what a CU pulls through its vector memory path per matrix
 // instruction is twice as much: 0.54 PFLOP/s at the ResNet-50 layer3 shape against the
 // 2.5 PFLOP/s peak.  Workgroups are persistent (at most one per CU) and walk the tile list.
-// Needs Cs % 64 == 0 and Nout % 64 == 0; weights as rows in place (wstep == 32).
+// Needs Cs % 64 == 0 and Nout % 64 == 0.  PACKED = weights in fragment order (wstep == 1024): the
+// multiplying wavefronts load their weight fragments straight into registers, so LDS only carries
+// the pixel rows (a stage moves 52 KB in and 112 KB out of LDS otherwise, as many LDS cycles as
+// the stage has matrix cycles).
 constexpr int kRoleThreads = 512;
 constexpr int kRoleDepth = 64;
 constexpr int kRoleLd = kRoleDepth + 8;   // LDS row: 144 bytes (9 x 16: conflict-free 16-byte reads)
 
-template <int CMW, int TN>
+template <int CMW, int TN, bool PACKED>
 __global__ __launch_bounds__(kRoleThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void gather_roles_kernel(
     const GatherH g, const bf16_t* __restrict__ src, const bf16_t* __restrict__ w,
     const bf16_t* __restrict__ bias, bf16_t* __restrict__ dst) {
@@ -350,7 +353,7 @@ __global__ __launch_bounds__(kRoleThreads) __attribute__((amdgpu_waves_per_eu(2,
   constexpr int kWChunks = BMW * (kRoleDepth / 8) / kFeeders;
   constexpr int kXChunks = (BP * (kRoleDepth / 8) + kFeeders - 1) / kFeeders;
   constexpr uint32_t kBeyond = 0x80000000u;   // byte offset past any buffer (tensors are < 2 GB)
-  __shared__ __attribute__((aligned(16))) bf16_t lds_w[2][BMW][kRoleLd];
+  __shared__ __attribute__((aligned(16))) bf16_t lds_w[PACKED ? 1 : 2][PACKED ? 1 : BMW][kRoleLd];
   __shared__ __attribute__((aligned(16))) bf16_t lds_x[2][BP][kRoleLd];
   __shared__ int tdh[kMaxTaps], tdw[kMaxTaps], twoff[kMaxTaps];
   __shared__ uint32_t row_dst[2][BP];
@@ -389,10 +392,12 @@ __global__ __launch_bounds__(kRoleThreads) __attribute__((amdgpu_waves_per_eu(2,
     for (uint32_t tile = slot; tile < tiles; tile += gridDim.x) {
       const uint32_t p0 = (tile / ntiles_n) * BP;
       const int n0 = (int)(tile % ntiles_n) * BMW;
+      if constexpr (!PACKED) {
 #pragma unroll
-      for (int i = 0; i < kWChunks; ++i) {
-        const int col = n0 + row0 + 32 * i;
-        w_off[i] = col < g.Nout ? ((uint32_t)col * g.wrow + ch * 8) * 2u : kBeyond;
+        for (int i = 0; i < kWChunks; ++i) {
+          const int col = n0 + row0 + 32 * i;
+          w_off[i] = col < g.Nout ? ((uint32_t)col * g.wrow + ch * 8) * 2u : kBeyond;
+        }
       }
 #pragma unroll
       for (int i = 0; i < kXChunks; ++i) {
@@ -423,17 +428,21 @@ __global__ __launch_bounds__(kRoleThreads) __attribute__((amdgpu_waves_per_eu(2,
         }
         const int so = __builtin_amdgcn_readfirstlane(c0 * 2);
         const int sw = __builtin_amdgcn_readfirstlane((int)so_w + c0 * 2);
+        if constexpr (!PACKED) {
 #pragma unroll
-        for (int i = 0; i < kWChunks; ++i)
-          qw[i] = __builtin_amdgcn_raw_buffer_load_b128(w_buf, w_off[i], sw, 0);
+          for (int i = 0; i < kWChunks; ++i)
+            qw[i] = __builtin_amdgcn_raw_buffer_load_b128(w_buf, w_off[i], sw, 0);
+        }
 #pragma unroll
         for (int i = 0; i < kXChunks; ++i)
           qx[i] = __builtin_amdgcn_raw_buffer_load_b128(src_buf, a_off[i], so, 0);
       };
       auto stage = [&](int buf, const uint4_t (&qw)[kWChunks], const uint4_t (&qx)[kXChunks]) {
+        if constexpr (!PACKED) {
 #pragma unroll
-        for (int i = 0; i < kWChunks; ++i)
-          *reinterpret_cast<uint4_t*>(&lds_w[buf][row0 + 32 * i][ch * 8]) = qw[i];
+          for (int i = 0; i < kWChunks; ++i)
+            *reinterpret_cast<uint4_t*>(&lds_w[buf][row0 + 32 * i][ch * 8]) = qw[i];
+        }
 #pragma unroll
         for (int i = 0; i < kXChunks; ++i)
           if (row0 + 32 * i < BP) *reinterpret_cast<uint4_t*>(&lds_x[buf][row0 + 32 * i][ch * 8]) = qx[i];
@@ -461,7 +470,14 @@ __global__ __launch_bounds__(kRoleThreads) __attribute__((amdgpu_waves_per_eu(2,
   // -------------------------------------------------------------------- multiplying wavefronts
   const int wm = wave / CPW, wp = wave % CPW;   // 64 channels x 32 TN positions each
   const int r = lane & 31, kq = (lane >> 5) * 8;
-  const bf16_t* aw = &lds_w[0][wm * 64 + r][kq];
+  const bf16_t* aw = PACKED ? nullptr : &lds_w[0][wm * 64 + r][kq];
+  const __amdgpu_buffer_rsrc_t wq_buf =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(w), 0, g.w_bytes, 0x00020000);
+  // PACKED: this wavefront's weight fragments come straight from memory, one 1 KB load per
+  // fragment, fetched a whole stage ahead into the registers the previous stage has just used
+  constexpr int kSteps = kRoleDepth / 16;
+  uint4_t wreg[kSteps][2];
+  uint32_t wq_off[2];
   const bf16_t* ax = &lds_x[0][wp * TN * 32 + r][kq];
   float16_t acc[2][TN];
   int parity = 0;
@@ -484,15 +500,49 @@ __global__ __launch_bounds__(kRoleThreads) __attribute__((amdgpu_waves_per_eu(2,
       for (int j = 0; j < TN; ++j)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    // position in the reduction of the stage whose weights are fetched next (PACKED)
+    int wt = -1, wc0 = g.Cs;
+    uint32_t wtap = 0;
+    auto next_weights = [&]() -> int {   // scalar byte offset of that stage's first fragment
+      wc0 += kRoleDepth;
+      if (wc0 >= g.Cs) {
+        wc0 = 0;
+        ++wt;
+        wtap = (uint32_t)__builtin_amdgcn_readfirstlane(twoff[wt]);
+      }
+      return __builtin_amdgcn_readfirstlane((int)(((wtap + (uint32_t)wc0) >> 4) * 1024u));
+    };
+    if constexpr (PACKED) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const uint32_t blk = (uint32_t)(n0 + wm * 64 + 32 * i) / 32;
+        wq_off[i] = (blk * (g.wrow / 16) * 64 + lane) * 16u;   // blocks past the rows: past the buffer
+      }
+      const int so = next_weights();
+#pragma unroll
+      for (int q = 0; q < kSteps; ++q)
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+          wreg[q][i] = __builtin_amdgcn_raw_buffer_load_b128(wq_buf, wq_off[i], so + q * 1024, 0);
+    }
     __syncthreads();   // stage 0 is in LDS
+    int so_next = 0;
     for (int s2 = 0; s2 < stages; ++s2) {
       const bf16_t* bw = aw + (s2 & 1) * (BMW * kRoleLd);
       const bf16_t* bx = ax + (s2 & 1) * (BP * kRoleLd);
+      if constexpr (PACKED) {
+        // the last stage fetches its own weights once more instead of branching around the loads
+        if (s2 + 1 < stages) so_next = next_weights();
+        else so_next = __builtin_amdgcn_readfirstlane((int)(((wtap + (uint32_t)wc0) >> 4) * 1024u));
+      }
 #pragma unroll
       for (int ks = 0; ks < kRoleDepth; ks += 16) {
         bf16x8 af[2], bfr[TN];
 #pragma unroll
-        for (int i = 0; i < 2; ++i) af[i] = *reinterpret_cast<const bf16x8*>(bw + 32 * i * kRoleLd + ks);
+        for (int i = 0; i < 2; ++i) {
+          if constexpr (PACKED) af[i] = __builtin_bit_cast(bf16x8, wreg[ks / 16][i]);
+          else af[i] = *reinterpret_cast<const bf16x8*>(bw + 32 * i * kRoleLd + ks);
+        }
 #pragma unroll
         for (int j = 0; j < TN; ++j) bfr[j] = *reinterpret_cast<const bf16x8*>(bx + 32 * j * kRoleLd + ks);
 #pragma unroll
@@ -500,6 +550,11 @@ __global__ __launch_bounds__(kRoleThreads) __attribute__((amdgpu_waves_per_eu(2,
 #pragma unroll
           for (int j = 0; j < TN; ++j)
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+        if constexpr (PACKED) {
+#pragma unroll
+          for (int i = 0; i < 2; ++i)
+            wreg[ks / 16][i] = __builtin_amdgcn_raw_buffer_load_b128(wq_buf, wq_off[i], so_next + (ks / 16) * 1024, 0);
+        }
       }
       __syncthreads();
     }
@@ -1012,7 +1067,7 @@ static int launch_gather16(GatherH q, const bf16_t* src, const bf16_t* w, const 
   q.src_bytes = (uint32_t)src_bytes;
   q.w_bytes = (uint32_t)w_bytes;
   const bool deep = q.Cs % 64 == 0;
-  if (q.wstep == 32 && roles_shape(q.Cs, q.Nout, q.npix)) {
+  if (roles_shape(q.Cs, q.Nout, q.npix)) {
     // large tiles, feeding and multiplying wavefronts.  256-channel tiles of 128 or 160 positions
     // (160 where it saves a round of the persistent, one-per-CU workgroups), 128-channel tiles of
     // 192 or 256 positions when that covers the channels with less padding.
@@ -1036,12 +1091,20 @@ static int launch_gather16(GatherH q, const bf16_t* src, const bf16_t* w, const 
       }
     }
     const dim3 grid((unsigned)(best_tiles < cus ? best_tiles : cus));
+#define MN_ROLES(CMW, TN)                                                                   \
+  do {                                                                                      \
+    if (q.wstep == 1024)                                                                    \
+      gather_roles_kernel<CMW, TN, true><<<grid, kRoleThreads, 0, s>>>(q, src, w, bias, dst);  \
+    else                                                                                    \
+      gather_roles_kernel<CMW, TN, false><<<grid, kRoleThreads, 0, s>>>(q, src, w, bias, dst); \
+  } while (0)
     switch (best) {
-      case 0: gather_roles_kernel<4, 5><<<grid, kRoleThreads, 0, s>>>(q, src, w, bias, dst); break;
-      case 1: gather_roles_kernel<4, 4><<<grid, kRoleThreads, 0, s>>>(q, src, w, bias, dst); break;
-      case 2: gather_roles_kernel<2, 4><<<grid, kRoleThreads, 0, s>>>(q, src, w, bias, dst); break;
-      default: gather_roles_kernel<2, 3><<<grid, kRoleThreads, 0, s>>>(q, src, w, bias, dst); break;
+      case 0: MN_ROLES(4, 5); break;
+      case 1: MN_ROLES(4, 4); break;
+      case 2: MN_ROLES(2, 4); break;
+      default: MN_ROLES(2, 3); break;
     }
+#undef MN_ROLES
     return MN_OK;
   }
   if (q.Nout % 128 == 0) {
@@ -1166,9 +1229,9 @@ int mn_conv16_fwd(const mn_conv2d* g, const void* x, const void* w, const void* 
   if (!mn_aligned(x, 16) || !mn_aligned(w, 16)) return MN_EINVAL;
   GatherH q = {};
   q.wstep = 32;
-  // variant 1 packs the weights in fragment order for the kernel that loads them straight into
-  // registers; shapes the large-tile kernel takes run that one under either variant
-  if (variant == 1 && !roles_shape(g->C, g->K, (unsigned long long)g->N * g->P * g->Q)) {
+  // variant 1 packs the weights in fragment order for the kernels that load them straight into
+  // registers
+  if (variant == 1) {
     if (!ws || ws_bytes < packed_weight_bytes(g, false) || !mn_aligned(ws, 16)) return MN_EINVAL;
     pack_weights(g, (const bf16_t*)w, (bf16_t*)ws, false, s);
     w = ws;
@@ -1210,10 +1273,8 @@ int mn_conv16_bwd_data(const mn_conv2d* g, const void* dy, const void* w, void* 
   const size_t nw = (size_t)g->K * g->C * T;
   const size_t need = variant == 1 ? packed_weight_bytes(g, true) : nw * sizeof(bf16_t);
   if (!ws || ws_bytes < need || !mn_aligned(ws, 16) || !mn_aligned(dy, 16)) return MN_EINVAL;
-  // variant 1: fragment-packed transposed weights, except where the large-tile kernel runs
-  // (it reads plain transposed rows; the packed size covers them)
-  const bool packed = variant == 1 &&
-                      !roles_shape(g->K, g->C, (unsigned long long)g->N * g->H * g->W / (g->sH * g->sW));
+  // variant 1: fragment-packed transposed weights
+  const bool packed = variant == 1;
   if (packed)
     pack_weights(g, (const bf16_t*)w, (bf16_t*)ws, true, s);
   else

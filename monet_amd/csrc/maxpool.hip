@@ -367,9 +367,11 @@ __global__ __launch_bounds__(kThreads) void maxpool_bwd_k3s2p1_flat_kernel(
   const bool col2 = 2 * q + 2 < PW;
   const size_t oA = (size_t)plane * PH * PW + (size_t)r * PW + 2 * q;  // even: PH*PW is even
   const size_t oB = oA + PW;
-  // dy and the indices are read once (streaming loads); dx is written with ordinary stores,
-  // which measured 8 % faster here than streaming ones (0.147 against 0.160 ms at
-  // [184,64,112,112] with operands that come from memory)
+  // Streaming loads for dy and the indices, although a pooled row is read twice (as row B of
+  // patch row r - 1 and as row A of patch row r, one plane row of threads later): an ordinary
+  // load for the first read saves 7 % of the HBM traffic and measured 7 % SLOWER (0.159
+  // against 0.148 ms at [184,64,112,112]).  dx is written with ordinary stores, which measured
+  // 8 % faster here than streaming ones (0.147 against 0.160 ms with operands from memory)
   const uint32_t a01 = ld_stream(idx4 + (oA >> 1));
   const uint32_t b01 = rowB ? ld_stream(idx4 + (oB >> 1)) : 0xFFu;
   const float2_t ga = ld_stream(reinterpret_cast<const float2_t*>(dy + oA));
