@@ -316,16 +316,17 @@ typedef struct mn_conv2d {
  * Needs channel counts that are multiples of 32 on the reduction side
  * (forward: C; backward-data: K) and multiples of 64 for backward-weight (C and
  * K); otherwise MN_EUNSUPPORTED.  Two variants per direction, further ones
- * are fp32 only.  Forward and backward-data multiply pixel tiles staged in
- * LDS with weight fragments that every wavefront loads straight into the
- * registers the matrix instruction reads: variant 0 reads them from the
- * weight rows where they lie (forward: no workspace; backward-data: the
- * transposed weights, K*C*R*S*2 bytes), variant 1 from a copy packed in
- * fragment order in the workspace (rows padded to 32: one contiguous KB per
- * fragment instead of 32 pieces of 32 bytes; 1.6 times faster at the
- * ResNet-50 layer3 shape).  Backward-weight: both variants run one kernel
- * with fp32 split partials in the workspace - ask mn_conv_ws_bytes.  The reference has no reduced-precision path; this dtype
- * serves the bf16 configuration of the layer3 benchmark. */
+ * are fp32 only.  Forward and backward-data: variant 0 reads the weight rows
+ * where they lie (forward: no workspace; backward-data: the transposed
+ * weights, K*C*R*S*2 bytes), variant 1 a copy packed in fragment order in
+ * the workspace (rows padded to 32: one contiguous KB per fragment), which
+ * the multiplying wavefronts load straight into registers.  Backward-weight:
+ * fp32 split partials in the workspace, added in a fixed order; variant 1 is
+ * the large-tile kernel (both channel counts multiples of 128, at least 4096
+ * output positions; other shapes run variant 0's kernel), twice as fast at
+ * the ResNet-50 layer3 shape - ask mn_conv_ws_bytes for either.  The
+ * reference has no reduced-precision path; this dtype serves the bf16
+ * configuration of the layer3 benchmark. */
 #define MN_BF16 1
 
 /* Number of kernel variants ("algorithms") per direction; variant 0 always
@@ -337,7 +338,10 @@ typedef struct mn_conv2d {
  *                    1 same with the weights repacked [tap][c][k] (k padded
  *                      to a multiple of 128) into the workspace, so operand
  *                      tiles load as full 16-byte vectors; channel counts
- *                      that are not a multiple of 16 run it like variant 0.
+ *                      that are not a multiple of 16 run it like variant 0,
+ *                      except the 3 -> 64 channel 7x7 / stride 2 / padding 3
+ *                      stem, which runs a kernel of its own (workspace: the
+ *                      transposed weights, 148 x 64 floats).
  *                      Launches with few, long workgroups split the reduction
  *                      in TWO and add the slices with atomics into a cleared
  *                      output: 0 + a + b and 0 + b + a round identically, so

@@ -48,6 +48,9 @@ int mn_conv16_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, void
                          size_t ws_bytes, int variant, hipStream_t s);
 
 // fp32 through three bf16 slices per operand (conv_split.hip)
+int mn_stem_ws_bytes(const mn_conv2d* g, int direction, size_t* bytes);
+int mn_stem_fwd(const mn_conv2d* g, const float* x, const float* w, const float* bias, float* y,
+                void* ws, size_t ws_bytes, hipStream_t s);
 int mn_split_ws_bytes(const mn_conv2d* g, int direction, size_t* bytes);
 int mn_split_pointwise(const mn_conv2d* g, int direction, const float* in, const float* w,
                        const float* bias, float* out, bool accumulate, void* ws, size_t ws_bytes,
@@ -1414,9 +1417,12 @@ int mn_conv_ws_bytes(const mn_conv2d* g, int direction, int variant, int dtype, 
   if (variant == 3) return mn_wino_fused_ws_bytes(g, direction == MN_CONV_BWD_DATA, bytes);
   if (variant == 4) return mn_split_ws_bytes(g, direction, bytes);
   const size_t wsize = (size_t)g->K * g->C * g->R * g->S * sizeof(float);
-  // variant 1 of the gather directions: the repacked weight operand (rows padded to 128)
-  if (direction == MN_CONV_FWD && variant == 1)
+  // variant 1 of the gather directions: the repacked weight operand (rows padded to 128); the
+  // 3 -> 64 channel 7x7 / 2 stem runs a kernel of its own with transposed weights
+  if (direction == MN_CONV_FWD && variant == 1) {
+    if (mn_stem_ws_bytes(g, direction, bytes) == MN_OK) return MN_OK;
     *bytes = (size_t)g->R * g->S * g->C * packed_rows(g->K) * sizeof(float);
+  }
   if (direction == MN_CONV_BWD_DATA && variant == 1)
     *bytes = (size_t)g->R * g->S * g->K * packed_rows(g->C) * sizeof(float);
   if (direction == MN_CONV_BWD_WEIGHT && variant == 1) {
@@ -1447,6 +1453,12 @@ int mn_conv_fwd(const mn_conv2d* g, const void* x, const void* w, const void* bi
   if (variant == 4)
     return mn_split_pointwise(g, MN_CONV_FWD, (const float*)x, (const float*)w, (const float*)bias,
                               (float*)y, false, ws, ws_bytes, mn_stream(stream));
+  if (variant == 1) {
+    size_t stem_bytes;
+    if (mn_stem_ws_bytes(g, MN_CONV_FWD, &stem_bytes) == MN_OK)
+      return mn_stem_fwd(g, (const float*)x, (const float*)w, (const float*)bias, (float*)y, ws,
+                         ws_bytes, mn_stream(stream));
+  }
   Gather q = {};
   q.M = g->K;
   q.T = g->R * g->S;

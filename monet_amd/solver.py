@@ -96,8 +96,11 @@ class _Builder:
 class Model:
     def __init__(self, si: SolverInfo, budget, time_limit=86400, solver="HIGHS", ablation=False,
                  mip_rel_gap=0.01, verbose=False, presolve=True, recompute_window=None,
-                 excess_price=EXCESS_PRICE, accept_up_to=None):
+                 excess_price=EXCESS_PRICE, accept_up_to=None, cutoff_ms=None):
         self.si = si
+        # run time of a schedule already known (ms): a row keeps the search below it, so the solver
+        # only has to prove that schedule optimal or beat it
+        self.cutoff_ms = cutoff_ms
         self.budget = budget
         self.time_limit = time_limit
         self.solver = solver
@@ -402,6 +405,9 @@ class Model:
             const_cost = 0.0
         else:
             total = sum(abs(c) for v, c in obj) + 1.0
+            if self.cutoff_ms is not None:
+                B.add([(v, c) for v, c in obj if v is not None],
+                      hi=self.cutoff_ms * CPU_GCD_MULTIPLIER - const_cost)
             obj = obj + [(excess, self.excess_price * total / float(self.budget))]
         B.minimise(obj)
 
@@ -529,6 +535,8 @@ def main(argv=None):
                         help="MiB of the budget to leave to what the schedule does not hold "
                              "(optimizer state, loss tensors, allocator rounding): the model is "
                              "solved against BUDGET minus this, the file keeps BUDGET in its name")
+    parser.add_argument("--cutoff_ms", default=None, type=float,
+                        help="run time of a known schedule: only look for schedules at most this slow")
     parser.add_argument("--verbose", action="store_true")
     args = parser.parse_args(argv)
 
@@ -555,7 +563,7 @@ def main(argv=None):
                                    args.solver, args.ablation,
                                    out_file=str(out), rounds=args.rounds, mip_rel_gap=args.gap,
                                    verbose=args.verbose,
-                                   recompute_window=args.window)
+                                   recompute_window=args.window, cutoff_ms=args.cutoff_ms)
     gap = getattr(solution, "mip_gap", float("nan"))
     print("solved in %.1f s, expected run time %.2f ms, gap %.2f %% -> %s" % (
         solution.solve_time, solution.runtime_expected / CPU_GCD_MULTIPLIER, 100.0 * gap, out))

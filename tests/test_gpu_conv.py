@@ -28,7 +28,7 @@ CASES = [
     ((2, 64, 56, 56), (256, 64, 1, 1), 1, 0, 1),       # 1x1 expansion
     ((2, 128, 28, 28), (128, 128, 3, 3), 2, 1, 1),     # strided 3x3
     ((2, 256, 28, 28), (512, 256, 1, 1), 2, 0, 1),     # strided 1x1 (downsample)
-    ((2, 3, 64, 64), (64, 3, 7, 7), 2, 3, 1),          # stem
+    ((2, 3, 64, 64), (64, 3, 7, 7), 2, 3, 1),          # stem (forward variant 1: the kernel of its own)
     ((1, 16, 33, 47), (24, 16, 3, 3), 1, 1, 1),        # odd spatial sizes
     ((5, 128, 7, 7), (128, 128, 3, 3), 1, 1, 1),       # 49-pixel images: no 16-byte alignment along the depth
     ((5, 128, 7, 7), (256, 128, 1, 1), 1, 0, 1),       # the same, 1x1
@@ -43,6 +43,9 @@ CASES = [
     ((3, 96, 10, 10), (48, 96, 1, 1), 1, 0, 1),        # 1x1: 48 output channels in a 64-wide tile, pixel tiles across images
     ((5, 256, 14, 14), (320, 256, 1, 1), 1, 0, 1),     # 1x1: 256-channel tiles with a ragged second one
     ((2, 144, 12, 12), (128, 144, 1, 1), 1, 0, 1),     # 1x1: nine 16-deep stages (an odd number)
+    # the stem again at odd sizes: forward variant 1 (the kernel of its own) stages scalars and
+    # has ragged row blocks
+    ((3, 3, 75, 97), (64, 3, 7, 7), 2, 3, 1),
 ]
 
 

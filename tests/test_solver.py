@@ -395,3 +395,12 @@ def test_ilp_optimum_equals_the_enumerated_optimum_on_a_tiny_graph(mode):
             costs.append(exact)
     assert seen_feasible == 3 and seen_infeasible == 1
     assert costs[-1] > costs[0]       # a tight budget costs run time: the comparison is not trivial
+    # a cutoff row at a known schedule's run time: the optimum is still found when it lies below
+    # the cutoff, and nothing is found when the cutoff is below the optimum
+    from monet_amd.solver import CPU_GCD_MULTIPLIER
+    gb = 342 / 1024.0 / 1024.0
+    best_ms = costs[-1] / CPU_GCD_MULTIPLIER
+    sol = Model(si, budget=gb, time_limit=120, mip_rel_gap=0.0, cutoff_ms=best_ms * 1.0001).solve()
+    assert abs(sol.runtime_expected - costs[-1]) <= 1e-6 * max(1.0, costs[-1])
+    with pytest.raises(ValueError):
+        Model(si, budget=gb, time_limit=120, mip_rel_gap=0.0, cutoff_ms=best_ms * 0.99).solve()
