@@ -473,12 +473,12 @@ def conv_bench(steps, warmup):
         res[name] = {"shape": g}
         res[name].update(directions(name + "/", g, x, w, dy, ("fwd", "bwd_data")))
         del x, w, dy
-    # one large-plane shape (UNet batch 11, 128 -> 128 channels at 208 x 304), forward only: where
-    # the one-kernel Winograd variant is the fastest
+    # one large-plane shape (UNet batch 11, 128 -> 128 channels at 208 x 304), forward and
+    # backward-weight: where the one-kernel Winograd variants are the fastest
     u = dict(N=11, C=128, K=128, R=3, S=3, H=208, W=304, stride=1, pad=1)
     x, w, dy = problem(u)
     res["unet_128ch_208x304"] = {"shape": u}
-    res["unet_128ch_208x304"].update(directions("unet_128ch_208x304/", u, x, w, dy, ("fwd",)))
+    res["unet_128ch_208x304"].update(directions("unet_128ch_208x304/", u, x, w, dy, ("fwd", "bwd_weight")))
     res["order"] = order
     res["calls_per_entry"] = steps + warmup
     return res

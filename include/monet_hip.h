@@ -401,7 +401,14 @@ typedef struct mn_conv2d {
  *                      fp32; workspace of 16 floats per tile and channel for
  *                      dy and x (capped at 512 MB: more tiles are taken in
  *                      passes added in order) plus the partial results;
- *                      reproducible */
+ *                      reproducible
+ *                    3 the same algorithm in one kernel: both transforms are
+ *                      applied on the way into LDS, no transformed tensors in
+ *                      memory; padding 1, even planes with W a multiple of 8,
+ *                      K and C multiples of 64; workspace: the partial
+ *                      results of at most one range of tile rows per CU
+ *                      (16 * ranges * K * C floats); reproducible.  The
+ *                      faster form below 256 channels and on large planes */
 int mn_conv_n_variants(int direction);
 /* The same per dtype: the list above for MN_F32; 2 for MN_BF16 (see MN_BF16);
  * 0 for an unknown dtype.  The reference is fp32 only and has no counterpart. */

@@ -35,6 +35,9 @@ int mn_wino_fused_fwd(const mn_conv2d* g, const float* x, const float* w, const 
 int mn_wino_fused_bwd_data(const mn_conv2d* g, const float* dy, const float* w, float* dx, bool accum,
                            void* ws, size_t ws_bytes, hipStream_t s);
 int mn_wino_bwd_weight_ws_bytes(const mn_conv2d* g, size_t* bytes);
+int mn_wino_fused_bwd_weight_ws_bytes(const mn_conv2d* g, size_t* bytes);
+int mn_wino_fused_bwd_weight(const mn_conv2d* g, const float* dy, const float* x, float* dw, float* db,
+                             void* ws, size_t ws_bytes, hipStream_t s);
 int mn_wino_bwd_weight(const mn_conv2d* g, const float* dy, const float* x, float* dw, float* db,
                        void* ws, size_t ws_bytes, hipStream_t s);
 
@@ -1388,7 +1391,7 @@ int mn_conv_n_variants(int direction) {
     case MN_CONV_BWD_DATA:
       return 5;
     case MN_CONV_BWD_WEIGHT:
-      return 3;
+      return 4;
     default:
       return 0;
   }
@@ -1414,7 +1417,9 @@ int mn_conv_ws_bytes(const mn_conv2d* g, int direction, int variant, int dtype, 
   if (variant == 2)
     return direction == MN_CONV_BWD_WEIGHT ? mn_wino_bwd_weight_ws_bytes(g, bytes)
                                            : mn_wino_ws_bytes(g, direction == MN_CONV_BWD_DATA, bytes);
-  if (variant == 3) return mn_wino_fused_ws_bytes(g, direction == MN_CONV_BWD_DATA, bytes);
+  if (variant == 3)
+    return direction == MN_CONV_BWD_WEIGHT ? mn_wino_fused_bwd_weight_ws_bytes(g, bytes)
+                                           : mn_wino_fused_ws_bytes(g, direction == MN_CONV_BWD_DATA, bytes);
   if (variant == 4) return mn_split_ws_bytes(g, direction, bytes);
   const size_t wsize = (size_t)g->K * g->C * g->R * g->S * sizeof(float);
   // variant 1 of the gather directions: the repacked weight operand (rows padded to 128); the
@@ -1624,9 +1629,15 @@ static int conv_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, vo
   const int st = check(g);
   if (st != MN_OK) return st;
   if (dtype != MN_F32 && dtype != MN_BF16) return MN_EUNSUPPORTED;
-  if (variant < 0 || variant > 2 || (variant == 2 && dtype != MN_F32)) return MN_EUNSUPPORTED;
+  if (variant < 0 || variant > 3 || (variant >= 2 && dtype != MN_F32)) return MN_EUNSUPPORTED;
   if (!dw) return MN_EINVAL;
   hipStream_t s = mn_stream(stream);
+  if (variant == 3) {
+    if (g->N == 0) return MN_EUNSUPPORTED;
+    if (!dy || !x) return MN_EINVAL;
+    return mn_wino_fused_bwd_weight(g, (const float*)dy, (const float*)x, (float*)dw, (float*)db_out,
+                                    ws, ws_bytes, s);
+  }
   if (variant == 2) {
     if (g->N == 0) return MN_EUNSUPPORTED;  // nothing to reduce: variants 0 and 1 clear dw
     if (!dy || !x) return MN_EINVAL;

@@ -430,6 +430,239 @@ __global__ __launch_bounds__(kThreads) void fused_kernel(const Plan p, const flo
   }
 }
 
+// ------------------------------------------ backward weight in one kernel --
+// dW = G^T [ sum over tiles of (A dY A^T) .* (B^T X B) ] G without the transformed tensors in HBM:
+// Z[pos][k][c] = sum_t Ud[pos][t][k] Vx[pos][t][c] is a product over the TILES, so a workgroup owns
+// 64 outputs x 64 inputs x 16 positions (the accumulator shape of the forward kernel above, 256
+// registers per lane) and walks a range of tile rows, four tiles of a row per chunk: per chunk a
+// thread loads one 4x4 patch of x and one 2x2 patch of dy, transforms them and writes one row of
+// Vx and of Ud (the LDS layout, the operand reads and the 32 matrix instructions per chunk are
+// the forward kernel's with "channel of the chunk" read as "tile of the chunk").
+// Lanes: 16 channels x 4 neighbouring tiles per wavefront, so a load touches 16 cache lines and
+// not 64 (a lane per channel plane was measured 1.5-1.7x slower in the forward kernel).  All
+// addresses are scalars per chunk plus byte offsets that never change per lane: the row and the
+// chunk's first column travel in the scalar offset of the buffer loads.  The padding is not
+// addressed: rows beyond the image are read from the nearest row, columns -1 and W from a
+// neighbouring element, and the values are replaced by zero before the transform.
+// The result of a range of tile rows goes to Z[pos][range][k][c]; wgrad_output_kernel adds the
+// ranges in order and applies G^T . G (reproducible).
+// Needs: 3x3, stride 1, padding 1, H and W even, W % 8 == 0, K % 64 == 0, C % 64 == 0.
+struct FWPlan {
+  int N, C, K, H, W;
+  int TH, TW;                 // tiles per image
+  uint32_t rows;              // N * TH tile rows
+  uint32_t rows_per_range;
+  int S;                      // ranges
+  uint32_t x_bytes, dy_bytes;
+};
+
+__global__ __launch_bounds__(kThreads) void fused_wgrad_kernel(const FWPlan p, const float* __restrict__ x,
+                                                               const float* __restrict__ dy,
+                                                               float* __restrict__ Z) {
+  extern __shared__ float4_t fused_lds[];  // [buffer][Ud | Vx][tile of the chunk][channel][LP]
+  float* const lds = reinterpret_cast<float*>(fused_lds);
+  const uint32_t slot = xcd_slot();
+  const uint32_t ncb = (uint32_t)p.C / FT, blocks = ((uint32_t)p.K / FK) * ncb;
+  const uint32_t blk = slot % blocks, range = slot / blocks;  // neighbours read the same tile rows
+  const uint32_t kb = blk / ncb, cb = blk - kb * ncb;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int ci = 16 * wave + (lane >> 2), ti = lane & 3;   // loader role: channel, tile of the chunk
+  const uint32_t r_begin = range * p.rows_per_range;
+  const uint32_t r_end = min(r_begin + p.rows_per_range, p.rows);
+  const int cpr = p.TW >> 2;                                // chunks per tile row
+  const int nchunks = (int)(r_end - r_begin) * cpr;         // real chunks (the loop runs a multiple of 4)
+  const uint32_t plane = (uint32_t)p.H * p.W;
+
+  const __amdgpu_buffer_rsrc_t x_buf =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(x), 0, p.x_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t dy_buf =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(dy), 0, p.dy_bytes, 0x00020000);
+  // byte offsets of this lane inside (image 0, row 0, first chunk): columns 2 ti - 1 .. 2 ti + 2
+  const uint32_t xc = (cb * FT + ci) * plane;
+  const uint32_t x_mid = (xc + 2 * ti) * 4u;                         // columns 2 ti, 2 ti + 1 (8 bytes)
+  const uint32_t x_left0 = (xc + (ti ? 2 * ti - 1 : 0)) * 4u;        // first chunk of a row (column -1 is replaced)
+  const uint32_t x_left = (xc + 2 * ti + 7) * 4u;                    // later chunks, with the scalar offset one chunk back
+  const uint32_t x_right = (xc + 2 * ti + 2) * 4u;
+  const uint32_t x_right_last = (xc + (ti == 3 ? 2 * ti + 1 : 2 * ti + 2)) * 4u;  // last chunk (column W is replaced)
+  const uint32_t dy_off = ((kb * FK + ci) * plane + 2 * ti) * 4u;
+
+  // position of the next chunk to fetch and of the next chunk to stage (all scalar)
+  struct Cursor {
+    int n, th, q;
+  };
+  auto start = [&]() {
+    Cursor c;
+    c.n = (int)(r_begin / (uint32_t)p.TH);
+    c.th = (int)(r_begin - (uint32_t)c.n * p.TH);
+    c.q = 0;
+    return c;
+  };
+  auto advance = [&](Cursor& c) {
+    if (++c.q == cpr) {
+      c.q = 0;
+      if (++c.th == p.TH) {
+        c.th = 0;
+        ++c.n;
+      }
+    }
+  };
+  Cursor cf = start(), cs = start();
+  int fetched = 0, staged = 0;
+
+  // four register sets, as in the forward kernel
+  float d0[4][4], d1[4][4], d2[4][4], d3[4][4];
+  float e0[2][2], e1[2][2], e2[2][2], e3[2][2];
+  auto fetch = [&](float (&d)[4][4], float (&e)[2][2]) {
+    // past the last chunk the last one is loaded again (no branch around the loads) and not used
+    const bool first = cf.q == 0, last = cf.q == cpr - 1;
+    const uint32_t vl = first ? x_left0 : x_left, vr = last ? x_right_last : x_right;
+    const int col = 8 * cf.q;
+    const int colL = first ? 0 : col - 8;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      int row = 2 * cf.th - 1 + a;
+      row = row < 0 ? 0 : (row >= p.H ? p.H - 1 : row);
+      const int base = (cf.n * p.C * p.H + row) * p.W;
+      const int so = __builtin_amdgcn_readfirstlane((base + col) * 4);
+      const int sl = __builtin_amdgcn_readfirstlane((base + colL) * 4);
+      d[a][0] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(x_buf, vl, sl, 0));
+      typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+      const u2 mid = __builtin_amdgcn_raw_buffer_load_b64(x_buf, x_mid, so, 0);
+      d[a][1] = __uint_as_float(mid[0]);
+      d[a][2] = __uint_as_float(mid[1]);
+      d[a][3] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(x_buf, vr, so, 0));
+    }
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+      const int base = (cf.n * p.K * p.H + 2 * cf.th + a) * p.W + col;
+      const int so = __builtin_amdgcn_readfirstlane(base * 4);
+      typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+      const u2 v = __builtin_amdgcn_raw_buffer_load_b64(dy_buf, dy_off, so, 0);
+      e[a][0] = __uint_as_float(v[0]);
+      e[a][1] = __uint_as_float(v[1]);
+    }
+    if (++fetched < nchunks) advance(cf);
+  };
+  float* const vrow = lds + kFusedHalf + (ti * FT + ci) * LP;
+  float* const urow = lds + (ti * FK + ci) * LP;
+  auto stage = [&](int buf, float (&d)[4][4], float (&e)[2][2]) {
+    const bool live = staged < nchunks;
+    const bool top = cs.th == 0, bottom = cs.th == p.TH - 1;
+    const bool left = cs.q == 0 && ti == 0, right = cs.q == cpr - 1 && ti == 3;
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      d[0][b] = top ? 0.f : d[0][b];
+      d[3][b] = bottom ? 0.f : d[3][b];
+    }
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      d[a][0] = left ? 0.f : d[a][0];
+      d[a][3] = right ? 0.f : d[a][3];
+    }
+    float v[16];
+    input_transform(d, v);
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      *reinterpret_cast<float4_t*>(vrow + buf * 2 * kFusedHalf + 4 * q) =
+          float4_t{v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]};
+    // A e A^T, A = [1 0; 1 1; 1 -1; 0 -1]; a chunk past the end contributes nothing
+    const float e00 = live ? e[0][0] : 0.f, e01 = live ? e[0][1] : 0.f;
+    const float e10 = live ? e[1][0] : 0.f, e11 = live ? e[1][1] : 0.f;
+    const float t0[2] = {e00, e01}, t1[2] = {e00 + e10, e01 + e11}, t2[2] = {e00 - e10, e01 - e11},
+                t3[2] = {-e10, -e11};
+    *reinterpret_cast<float4_t*>(urow + buf * 2 * kFusedHalf + 0) = float4_t{t0[0], t0[0] + t0[1], t0[0] - t0[1], -t0[1]};
+    *reinterpret_cast<float4_t*>(urow + buf * 2 * kFusedHalf + 4) = float4_t{t1[0], t1[0] + t1[1], t1[0] - t1[1], -t1[1]};
+    *reinterpret_cast<float4_t*>(urow + buf * 2 * kFusedHalf + 8) = float4_t{t2[0], t2[0] + t2[1], t2[0] - t2[1], -t2[1]};
+    *reinterpret_cast<float4_t*>(urow + buf * 2 * kFusedHalf + 12) = float4_t{t3[0], t3[0] + t3[1], t3[0] - t3[1], -t3[1]};
+    if (++staged < nchunks) advance(cs);
+  };
+
+  float16_t acc[16];
+#pragma unroll
+  for (int pos = 0; pos < 16; ++pos)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[pos][v] = 0.f;
+  const int wk = (wave >> 1) * 32, wc = (wave & 1) * 32;
+  const int r = lane & 31, half = lane >> 5;
+  // operands: row (tile 2 s + half, output wk + r) of Ud and (tile 2 s + half, input wc + r) of Vx
+  const float* const arow = lds + (half * FK + wk + r) * LP;
+  const float* const brow = lds + kFusedHalf + (half * FT + wc + r) * LP;
+  float4_t ca[2], cbv[2];
+#pragma unroll
+  for (int q = 0; q < 2; ++q) ca[q] = cbv[q] = float4_t{0.f, 0.f, 0.f, 0.f};
+  auto tail = [&]() {
+#pragma unroll
+    for (int q = 0; q < 2; ++q)
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        acc[8 + 4 * q + e] = __builtin_amdgcn_mfma_f32_32x32x2f32(ca[q][e], cbv[q][e], acc[8 + 4 * q + e], 0, 0, 0);
+  };
+  auto head = [&](int buf) {
+    float4_t av[FC / 2][4], bv[FC / 2][4];
+#pragma unroll
+    for (int s2 = 0; s2 < FC / 2; ++s2)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        av[s2][q] = *reinterpret_cast<const float4_t*>(arow + buf * 2 * kFusedHalf + 2 * s2 * FK * LP + 4 * q);
+        bv[s2][q] = *reinterpret_cast<const float4_t*>(brow + buf * 2 * kFusedHalf + 2 * s2 * FT * LP + 4 * q);
+      }
+#pragma unroll
+    for (int i = 0; i < 24; ++i) {  // step 0: 16 positions, step 1: positions 0..7
+      const int s2 = i >> 4, pos = i & 15;
+      acc[pos] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[s2][pos >> 2][pos & 3], bv[s2][pos >> 2][pos & 3],
+                                                      acc[pos], 0, 0, 0);
+    }
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      ca[q] = av[1][2 + q];
+      cbv[q] = bv[1][2 + q];
+    }
+  };
+  auto interleave = [&]() {
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);              // one MFMA
+      if (i < 8) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);   // two LDS reads
+      if (i >= 4 && i < 20) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global load
+      __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);              // VALU
+      if (i >= 24) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); // one LDS write
+    }
+  };
+  const int steps = (nchunks + 3) & ~3;
+  fetch(d0, e0);
+  fetch(d1, e1);
+  fetch(d2, e2);
+  fetch(d3, e3);
+  stage(0, d0, e0);
+  __syncthreads();
+#define MN_WINO_WSTEP(buf, dk, ek, dn, en) \
+  fetch(dk, ek);                           \
+  tail();                                  \
+  head(buf);                               \
+  stage((buf) ^ 1, dn, en);                \
+  interleave();                            \
+  __syncthreads();
+  for (int ch = 0; ch < steps; ch += 4) {
+    MN_WINO_WSTEP(0, d0, e0, d1, e1)
+    MN_WINO_WSTEP(1, d1, e1, d2, e2)
+    MN_WINO_WSTEP(0, d2, e2, d3, e3)
+    MN_WINO_WSTEP(1, d3, e3, d0, e0)
+  }
+#undef MN_WINO_WSTEP
+  tail();
+
+  // Z[pos][range][k][c]: a register holds one output for 32 consecutive inputs
+  const size_t kc = (size_t)p.K * p.C;
+  float* zb = Z + (size_t)range * kc + (size_t)(kb * FK + wk) * p.C + cb * FT + wc + r;
+#pragma unroll
+  for (int pos = 0; pos < 16; ++pos)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int k = 8 * (v >> 2) + 4 * half + (v & 3);
+      zb[(size_t)pos * p.S * kc + (size_t)k * p.C] = acc[pos][v];
+    }
+}
+
 // ------------------------------------------------------------ backward weight --
 // dW (3x3) = sum over tiles of G^T [ (A dY A^T) .* (B^T X B) ] G, with dY the 2x2 tile of the
 // output gradient and X the 4x4 input tile the forward used for it (the transposed form of the
@@ -747,6 +980,8 @@ static bool fused_lds_allowed() {
       hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_kernel<true>),
                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)kFusedLds) == hipSuccess &&
       hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_kernel<false>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kFusedLds) == hipSuccess &&
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_wgrad_kernel),
                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)kFusedLds) == hipSuccess;
   done[dev] = ok;
   return ok;
@@ -850,6 +1085,68 @@ int mn_wino_fused_bwd_data(const mn_conv2d* g, const float* dy, const float* w, 
 }
 
 // Weight gradient (fp32) through the Winograd form above; db (optional): the bias gradient.
+namespace mn_wino {
+static bool make_fwplan(const mn_conv2d* g, FWPlan& f) {
+  if (!shape_ok(g) || g->pH != 1 || g->pW != 1) return false;
+  if (g->H != g->P || g->W != g->Q || (g->H & 1) || (g->W & 7) || g->K % FK != 0 || g->C % FT != 0)
+    return false;
+  const unsigned long long xb = (unsigned long long)g->N * g->C * g->H * g->W * 4ull;
+  const unsigned long long yb = (unsigned long long)g->N * g->K * g->H * g->W * 4ull;
+  if (xb >= (1ull << 31) || yb >= (1ull << 31) || g->N == 0) return false;
+  f.N = g->N;
+  f.C = g->C;
+  f.K = g->K;
+  f.H = g->H;
+  f.W = g->W;
+  f.TH = g->H / 2;
+  f.TW = g->W / 2;
+  f.rows = (uint32_t)g->N * f.TH;
+  f.x_bytes = (uint32_t)xb;
+  f.dy_bytes = (uint32_t)yb;
+  // one workgroup per CU (256 accumulation registers per lane, 80 KB of LDS): as many ranges of
+  // tile rows as that leaves per (output, input) block
+  int dev = 0, cus = 256;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+    cus = 256;
+  const long long blocks = (long long)(g->K / FK) * (g->C / FT);
+  long long S = cus / blocks;
+  if (S < 1) S = 1;
+  if (S > f.rows) S = f.rows;
+  f.rows_per_range = (uint32_t)((f.rows + S - 1) / S);
+  f.S = (int)((f.rows + f.rows_per_range - 1) / f.rows_per_range);
+  return true;
+}
+}  // namespace mn_wino
+
+// Backward-weight variant 3: Z only (16 * ranges * K * C floats).
+int mn_wino_fused_bwd_weight_ws_bytes(const mn_conv2d* g, size_t* bytes) {
+  using namespace mn_wino;
+  *bytes = 0;
+  FWPlan f;
+  if (!make_fwplan(g, f)) return MN_EUNSUPPORTED;
+  *bytes = (size_t)16 * f.S * f.K * f.C * sizeof(float);
+  return MN_OK;
+}
+
+int mn_wino_fused_bwd_weight(const mn_conv2d* g, const float* dy, const float* x, float* dw, float* db,
+                             void* ws, size_t ws_bytes, hipStream_t s) {
+  using namespace mn_wino;
+  FWPlan f;
+  if (!make_fwplan(g, f)) return MN_EUNSUPPORTED;
+  if (!fused_lds_allowed()) return MN_EUNSUPPORTED;
+  const size_t need = (size_t)16 * f.S * f.K * f.C * sizeof(float);
+  if (!ws || ws_bytes < need || !mn_aligned(ws, 16) || !mn_aligned(x, 8) || !mn_aligned(dy, 8))
+    return MN_EINVAL;
+  float* Z = static_cast<float*>(ws);
+  const uint32_t grid = (uint32_t)(f.K / FK) * (f.C / FT) * f.S;
+  fused_wgrad_kernel<<<grid, kThreads, kFusedLds, s>>>(f, x, dy, Z);
+  const uint32_t n = (uint32_t)f.K * f.C;
+  wgrad_output_kernel<false><<<(n + 63) / 64, kThreads, 0, s>>>(Z, dw, f.K, f.C, f.S);
+  if (db) bias_grad_kernel<<<f.K, kThreads, 0, s>>>(dy, db, g->N, g->K, g->P * g->Q);
+  return mn_launch_status();
+}
+
 int mn_wino_bwd_weight_ws_bytes(const mn_conv2d* g, size_t* bytes) {
   using namespace mn_wino;
   *bytes = 0;

@@ -46,6 +46,12 @@ CASES = [
     # the stem again at odd sizes: forward variant 1 (the kernel of its own) stages scalars and
     # has ragged row blocks
     ((3, 3, 75, 97), (64, 3, 7, 7), 2, 3, 1),
+    # backward-weight variant 3 (Winograd in one kernel): 64-channel blocks, W % 8 == 0; one and
+    # several chunks per tile row, ranges of one tile row (padded to four chunks), uneven ranges
+    ((2, 64, 16, 16), (64, 64, 3, 3), 1, 1, 1),
+    ((3, 128, 24, 32), (64, 128, 3, 3), 1, 1, 1),
+    ((1, 64, 6, 8), (128, 64, 3, 3), 1, 1, 1),
+    ((37, 64, 18, 24), (64, 64, 3, 3), 1, 1, 1),       # 333 tile rows over 256 ranges
 ]
 
 
@@ -62,6 +68,14 @@ def winograd_applies(ws, st, pad, dil, reduced_channels):
 def winograd_wgrad_applies(xs, ws, st, pad, dil):
     """Variant 2 of backward-weight: 3x3, stride 1, dilation 1, equal padding <= 2, C % 4 == 0."""
     return winograd_applies(ws, st, pad, dil, 16) and xs[1] % 4 == 0
+
+
+def fused_winograd_wgrad_applies(xs, ws, st, pad, dil):
+    """Variant 3 of backward-weight (Winograd in one kernel): 3x3, stride 1, dilation 1, padding 1,
+    even planes with W % 8 == 0, K and C multiples of 64."""
+    pair = lambda v: tuple(v) if isinstance(v, (tuple, list)) else (v, v)
+    return (winograd_applies(ws, st, pad, dil, 16) and pair(pad) == (1, 1) and xs[2] % 2 == 0 and
+            xs[3] % 8 == 0 and xs[1] % 64 == 0 and ws[0] % 64 == 0)
 
 
 def split_applies(xs, ws, st, pad, dil, reduced_channels):
@@ -150,16 +164,17 @@ def test_conv_backward_weight(cuda, xs, ws, st, pad, dil):
     dy = np.random.default_rng(4).standard_normal(yshape).astype(np.float32)
     exp = O.conv_bwd_weight(dy, x, ws, st, pad, dil)
     outs = []
-    assert conv_ops.n_bwd_wt_algos() == 3
+    assert conv_ops.n_bwd_wt_algos() == 4
     for v in range(conv_ops.n_bwd_wt_algos()):
-        if v == 2 and not winograd_wgrad_applies(xs, ws, st, pad, dil):
+        if (v == 2 and not winograd_wgrad_applies(xs, ws, st, pad, dil)) or \
+                (v == 3 and not fused_winograd_wgrad_applies(xs, ws, st, pad, dil)):
             assert refused(lambda: conv_ops.conv_backward_weight(ws, dev(dy, cuda), dev(x, cuda),
                                                                  pad, st, dil, 1, v))
             continue
         dw = conv_ops.conv_backward_weight(ws, dev(dy, cuda), dev(x, cuda), pad, st, dil, 1, v)
         assert_rel(host(dw), exp, TOL, f"backward-weight variant {v}")
         outs.append(dw)
-        if v == 2:   # partial results added in a fixed order: bit-identical run to run
+        if v >= 2:   # partial results added in a fixed order: bit-identical run to run
             assert torch.equal(dw, conv_ops.conv_backward_weight(ws, dev(dy, cuda), dev(x, cuda), pad,
                                                                  st, dil, 1, v))
     # the workspace variant sums its partials in a fixed order: bit-identical run to run
@@ -379,7 +394,8 @@ def test_conv_backward_weight_with_bias_gradient(cuda, xs, ws, st, pad, dil):
     # the largest of K sums
     scale_db = np.sqrt(dy.size / ws[0])
     for v in range(conv_ops.n_bwd_wt_algos()):
-        if v == 2 and not winograd_wgrad_applies(xs, ws, st, pad, dil):
+        if (v == 2 and not winograd_wgrad_applies(xs, ws, st, pad, dil)) or \
+                (v == 3 and not fused_winograd_wgrad_applies(xs, ws, st, pad, dil)):
             continue
         alone = conv_ops.conv_backward_weight(ws, dev(dy, cuda), dev(x, cuda), pad, st, dil, 1, v)
         dw, db = conv_ops.conv_backward_weight(ws, dev(dy, cuda), dev(x, cuda), pad, st, dil, 1, v,

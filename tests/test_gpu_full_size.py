@@ -117,6 +117,8 @@ def test_max_pool_indices_at_full_size(cuda):
 
 
 POINTWISE3 = ((184, 1024, 14, 14), (256, 1024, 1, 1))   # ResNet-50 layer3, reducing 1x1
+LAYER1 = ((184, 64, 56, 56), (64, 64, 3, 3))             # ResNet-50 layer1 3x3: W % 8 == 0, so the
+                                                         # one-kernel Winograd backward-weight runs
 
 
 def _variants(n, run):
@@ -132,7 +134,8 @@ def _variants(n, run):
 
 @pytest.mark.parametrize("shape,pad,dtype,tol", [(LAYER3, 1, torch.float32, 1e-5),
                                                  (LAYER3, 1, torch.bfloat16, 1e-2),
-                                                 (POINTWISE3, 0, torch.float32, 1e-5)])
+                                                 (POINTWISE3, 0, torch.float32, 1e-5),
+                                                 (LAYER1, 1, torch.float32, 1e-5)])
 def test_convolution_directions_are_adjoint_at_full_size(cuda, shape, pad, dtype, tol):
     xs, ws = shape
     x = _randn(xs, cuda, 7)
@@ -155,9 +158,13 @@ def test_convolution_directions_are_adjoint_at_full_size(cuda, shape, pad, dtype
         for vd, dx in _variants(conv_ops.n_bwd_ip_algos(dtype), lambda vd: conv_ops.conv_backward_input(
                 list(xs), dy, w, pad, 1, 1, 1, vd)):
             assert abs(lhs - _dot(dx, x)) < tol * scale, (v, vd)
+        ran_w = []
         for vw, dw in _variants(conv_ops.n_bwd_wt_algos(dtype), lambda vw: conv_ops.conv_backward_weight(
                 list(ws), dy, x, pad, 1, 1, 1, vw)):
             assert abs(lhs - _dot(dw, w)) < tol * scale, (v, vw)
+            ran_w.append(vw)
+        if shape is LAYER1:
+            assert ran_w == [0, 1, 2, 3]      # the one-kernel Winograd backward-weight included
         # linearity of the forward in x (exact up to rounding of the two results)
         x2 = _randn(xs, cuda, 10)
         if dtype == torch.bfloat16:
