@@ -407,7 +407,9 @@ typedef struct mn_conv2d {
  *                      memory; padding 1, even planes with W a multiple of 8,
  *                      K and C multiples of 64; workspace: the partial
  *                      results of at most one range of tile rows per CU
- *                      (16 * ranges * K * C floats); reproducible.  The
+ *                      (16 * ranges * K * C floats, and ranges * K for the
+ *                      bias gradient, which the same kernel sums from the
+ *                      tiles it stages); reproducible.  The
  *                      faster form below 256 channels and on large planes */
 int mn_conv_n_variants(int direction);
 /* The same per dtype: the list above for MN_F32; 2 for MN_BF16 (see MN_BF16);
