@@ -52,6 +52,8 @@ int mn_conv16_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, void
 
 // fp32 through three bf16 slices per operand (conv_split.hip)
 int mn_stem_ws_bytes(const mn_conv2d* g, int direction, size_t* bytes);
+int mn_stem_bwd_weight(const mn_conv2d* g, const float* dy, const float* x, float* dw, float* db,
+                       void* ws, size_t ws_bytes, hipStream_t s);
 int mn_stem_fwd(const mn_conv2d* g, const float* x, const float* w, const float* bias, float* y,
                 void* ws, size_t ws_bytes, hipStream_t s);
 int mn_split_ws_bytes(const mn_conv2d* g, int direction, size_t* bytes);
@@ -1435,6 +1437,9 @@ int mn_conv_ws_bytes(const mn_conv2d* g, int direction, int variant, int dtype, 
     wgrad_split(g, 1, &splits, &tiles);
     // one partial weight gradient and one partial bias gradient (K floats) per split
     *bytes = splits > 1 ? (wsize + (size_t)g->K * sizeof(float)) * splits : 0;
+    // the stem runs a kernel of its own (one partial result per workgroup)
+    size_t stem_bytes = 0;
+    if (mn_stem_ws_bytes(g, direction, &stem_bytes) == MN_OK && stem_bytes > *bytes) *bytes = stem_bytes;
   }
   return MN_OK;
 }
@@ -1660,6 +1665,12 @@ static int conv_bwd_weight(const mn_conv2d* g, const void* dy, const void* x, vo
     return mn_launch_status();
   }
   if (!dy || !x) return MN_EINVAL;
+  if (variant == 1) {
+    size_t stem_bytes = 0;
+    if (mn_stem_ws_bytes(g, MN_CONV_BWD_WEIGHT, &stem_bytes) == MN_OK && ws && ws_bytes >= stem_bytes &&
+        mn_aligned(ws, 16))
+      return mn_stem_bwd_weight(g, (const float*)dy, (const float*)x, (float*)dw, db, ws, ws_bytes, s);
+  }
   WGrad q = {};
   q.K = g->K;
   q.C = g->C;

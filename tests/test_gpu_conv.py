@@ -52,6 +52,10 @@ CASES = [
     ((3, 128, 24, 32), (64, 128, 3, 3), 1, 1, 1),
     ((1, 64, 6, 8), (128, 64, 3, 3), 1, 1, 1),
     ((37, 64, 18, 24), (64, 64, 3, 3), 1, 1, 1),       # 333 tile rows over 256 ranges
+    # the stem's backward-weight kernel (variant 1): 112 output columns (the group count the kernel
+    # is specialised for) with a ragged last row block; more items than workgroups
+    ((2, 3, 42, 224), (64, 3, 7, 7), 2, 3, 1),
+    ((150, 3, 32, 32), (64, 3, 7, 7), 2, 3, 1),
 ]
 
 
