@@ -479,6 +479,13 @@ def conv_bench(steps, warmup):
     x, w, dy = problem(u)
     res["unet_128ch_208x304"] = {"shape": u}
     res["unet_128ch_208x304"].update(directions("unet_128ch_208x304/", u, x, w, dy, ("fwd", "bwd_weight")))
+    del x, w, dy
+    # the stem (3 -> 64 channels, 7x7, stride 2): variant 1 of forward and backward-weight are
+    # kernels of their own
+    st = dict(N=184, C=3, K=64, R=7, S=7, H=224, W=224, stride=2, pad=3)
+    x, w, dy = problem(st)
+    res["stem_3_64_224x224"] = {"shape": st}
+    res["stem_3_64_224x224"].update(directions("stem_3_64_224x224/", st, x, w, dy, ("fwd", "bwd_weight")))
     res["order"] = order
     res["calls_per_entry"] = steps + warmup
     return res

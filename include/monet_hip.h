@@ -394,7 +394,9 @@ typedef struct mn_conv2d {
  *                      are split)
  *   backward-weight  0 split reduction combined with atomics into a cleared dw
  *                    1 split reduction through per-split partials in the
- *                      workspace, then a fixed-order sum (reproducible)
+ *                      workspace, then a fixed-order sum (reproducible); the
+ *                      3 -> 64 channel 7x7 / 2 stem runs a kernel of its own
+ *                      (workspace: one 64 x 148 partial result per workgroup)
  *                    2 Winograd (the transposed form of F(2x2, 3x3): the 16
  *                      transform-domain products reduced over the 2x2 output
  *                      tiles): 3x3, stride 1, dilation 1, C a multiple of 4,
