@@ -447,6 +447,10 @@ __global__ __launch_bounds__(kThreads) void fused_kernel(const Plan p, const flo
 // The result of a range of tile rows goes to Z[pos][range][k][c]; wgrad_output_kernel adds the
 // ranges in order and applies G^T . G (reproducible).
 // Needs: 3x3, stride 1, padding 1, H and W even, W % 8 == 0, K % 64 == 0, C % 64 == 0.
+constexpr int kWgTile = FK * LP + 16;                   // floats of one tile's 64 rows (FK == FT), padded
+constexpr int kWgHalf = FC * kWgTile;                   // floats of Ud (or Vx) in one buffer
+constexpr size_t kWgLds = (size_t)4 * kWgHalf * sizeof(float);  // 81 KB
+static_assert(FK == FT, "one row count for both operands");
 struct FWPlan {
   int N, C, K, H, W;
   int TH, TW;                 // tiles per image
@@ -513,42 +517,68 @@ __global__ __launch_bounds__(kThreads) void fused_wgrad_kernel(const FWPlan p, c
   int fetched = 0, staged = 0;
   float bsum = 0.f;
 
-  // four register sets, as in the forward kernel
-  float d0[4][4], d1[4][4], d2[4][4], d3[4][4];
-  float e0[2][2], e1[2][2], e2[2][2], e3[2][2];
-  auto fetch = [&](float (&d)[4][4], float (&e)[2][2]) {
+  // Eight register sets in two banks of four consecutive chunks.  The loads of a bank are issued
+  // row by row for its four chunks together: four chunks of a tile row cover the same 128-byte
+  // lines (a chunk is 32 bytes of each row), and a CU's chunk touches 384 lines = 48 KB, more than
+  // the L1 holds, so loaded chunk by chunk every line came from L2 four times (with the same
+  // load instructions on cache-resident addresses the kernel ran 1.37 -> 0.94 ms).
+  float p0[4][4], p1[4][4], p2[4][4], p3[4][4], q0[4][4], q1[4][4], q2[4][4], q3[4][4];
+  float f0[2][2], f1[2][2], f2[2][2], f3[2][2], g0[2][2], g1[2][2], g2[2][2], g3[2][2];
+  Cursor gc[4] = {cf, cf, cf, cf};  // the four chunks of the bank being loaded
+  auto group_begin = [&]() {
     // past the last chunk the last one is loaded again (no branch around the loads) and not used
-    const bool first = cf.q == 0, last = cf.q == cpr - 1;
-    const uint32_t vl = first ? x_left0 : x_left, vr = last ? x_right_last : x_right;
-    const int col = 8 * cf.q;
-    const int colL = first ? 0 : col - 8;
 #pragma unroll
-    for (int a = 0; a < 4; ++a) {
-      int row = 2 * cf.th - 1 + a;
-      row = row < 0 ? 0 : (row >= p.H ? p.H - 1 : row);
-      const int base = (cf.n * p.C * p.H + row) * p.W;
-      const int so = __builtin_amdgcn_readfirstlane((base + col) * 4);
-      const int sl = __builtin_amdgcn_readfirstlane((base + colL) * 4);
-      d[a][0] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(x_buf, vl, sl, 0));
-      typedef uint32_t u2 __attribute__((ext_vector_type(2)));
-      const u2 mid = __builtin_amdgcn_raw_buffer_load_b64(x_buf, x_mid, so, 0);
-      d[a][1] = __uint_as_float(mid[0]);
-      d[a][2] = __uint_as_float(mid[1]);
-      d[a][3] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(x_buf, vr, so, 0));
+    for (int i = 0; i < 4; ++i) {
+      gc[i] = cf;
+      if (++fetched < nchunks) advance(cf);
     }
-#pragma unroll
-    for (int a = 0; a < 2; ++a) {
-      const int base = (cf.n * p.K * p.H + 2 * cf.th + a) * p.W + col;
-      const int so = __builtin_amdgcn_readfirstlane(base * 4);
-      typedef uint32_t u2 __attribute__((ext_vector_type(2)));
-      const u2 v = __builtin_amdgcn_raw_buffer_load_b64(dy_buf, dy_off, so, 0);
-      e[a][0] = __uint_as_float(v[0]);
-      e[a][1] = __uint_as_float(v[1]);
-    }
-    if (++fetched < nchunks) advance(cf);
   };
-  float* const vrow = lds + kFusedHalf + (ti * FT + ci) * LP;
-  float* const urow = lds + (ti * FK + ci) * LP;
+  auto fetch_x = [&](int a, const Cursor& c, float (&d)[4][4]) {  // row a of chunk c's patches
+    const bool first = c.q == 0, last = c.q == cpr - 1;
+    const uint32_t vl = first ? x_left0 : x_left, vr = last ? x_right_last : x_right;
+    const int col = 8 * c.q;
+    const int colL = first ? 0 : col - 8;
+    int row = 2 * c.th - 1 + a;
+    row = row < 0 ? 0 : (row >= p.H ? p.H - 1 : row);
+    const int base = (c.n * p.C * p.H + row) * p.W;
+    const int so = __builtin_amdgcn_readfirstlane((base + col) * 4);
+    const int sl = __builtin_amdgcn_readfirstlane((base + colL) * 4);
+    d[a][0] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(x_buf, vl, sl, 0));
+    typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+    const u2 mid = __builtin_amdgcn_raw_buffer_load_b64(x_buf, x_mid, so, 0);
+    d[a][1] = __uint_as_float(mid[0]);
+    d[a][2] = __uint_as_float(mid[1]);
+    d[a][3] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(x_buf, vr, so, 0));
+  };
+  auto fetch_dy = [&](int a, const Cursor& c, float (&e)[2][2]) {
+    const int base = (c.n * p.K * p.H + 2 * c.th + a) * p.W + 8 * c.q;
+    const int so = __builtin_amdgcn_readfirstlane(base * 4);
+    typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+    const u2 v = __builtin_amdgcn_raw_buffer_load_b64(dy_buf, dy_off, so, 0);
+    e[a][0] = __uint_as_float(v[0]);
+    e[a][1] = __uint_as_float(v[1]);
+  };
+  // the four parts of a bank's loads, one per step: rows 0 and 1 of all four chunks (with the
+  // gradient rows), then rows 2 and 3 of the first two and of the last two chunks
+#define MN_WINO_PART01(a, A, B, C, D, EA, EB, EC, ED) \
+  fetch_x(a, gc[0], A);                               \
+  fetch_x(a, gc[1], B);                               \
+  fetch_x(a, gc[2], C);                               \
+  fetch_x(a, gc[3], D);                               \
+  fetch_dy(a, gc[0], EA);                             \
+  fetch_dy(a, gc[1], EB);                             \
+  fetch_dy(a, gc[2], EC);                             \
+  fetch_dy(a, gc[3], ED);
+#define MN_WINO_PART23(i, j, A, B) \
+  fetch_x(2, gc[i], A);            \
+  fetch_x(2, gc[j], B);            \
+  fetch_x(3, gc[i], A);            \
+  fetch_x(3, gc[j], B);
+  // row (tile ti, channel ci): the four tiles of a channel are written by neighbouring lanes, so
+  // a tile's block of 64 rows is padded by 16 floats (64 * LP is a multiple of the 64 banks: the
+  // four lanes of a channel would hit the same banks, a 4-way conflict on every staging write)
+  float* const vrow = lds + kWgHalf + ti * kWgTile + ci * LP;
+  float* const urow = lds + ti * kWgTile + ci * LP;
   auto stage = [&](int buf, float (&d)[4][4], float (&e)[2][2]) {
     const bool live = staged < nchunks;
     const bool top = cs.th == 0, bottom = cs.th == p.TH - 1;
@@ -567,7 +597,7 @@ __global__ __launch_bounds__(kThreads) void fused_wgrad_kernel(const FWPlan p, c
     input_transform(d, v);
 #pragma unroll
     for (int q = 0; q < 4; ++q)
-      *reinterpret_cast<float4_t*>(vrow + buf * 2 * kFusedHalf + 4 * q) =
+      *reinterpret_cast<float4_t*>(vrow + buf * 2 * kWgHalf + 4 * q) =
           float4_t{v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]};
     // A e A^T, A = [1 0; 1 1; 1 -1; 0 -1]; a chunk past the end contributes nothing
     const float e00 = live ? e[0][0] : 0.f, e01 = live ? e[0][1] : 0.f;
@@ -575,10 +605,10 @@ __global__ __launch_bounds__(kThreads) void fused_wgrad_kernel(const FWPlan p, c
     const float t0[2] = {e00, e01}, t1[2] = {e00 + e10, e01 + e11}, t2[2] = {e00 - e10, e01 - e11},
                 t3[2] = {-e10, -e11};
     if (BIAS) bsum += t1[0] + t1[1];
-    *reinterpret_cast<float4_t*>(urow + buf * 2 * kFusedHalf + 0) = float4_t{t0[0], t0[0] + t0[1], t0[0] - t0[1], -t0[1]};
-    *reinterpret_cast<float4_t*>(urow + buf * 2 * kFusedHalf + 4) = float4_t{t1[0], t1[0] + t1[1], t1[0] - t1[1], -t1[1]};
-    *reinterpret_cast<float4_t*>(urow + buf * 2 * kFusedHalf + 8) = float4_t{t2[0], t2[0] + t2[1], t2[0] - t2[1], -t2[1]};
-    *reinterpret_cast<float4_t*>(urow + buf * 2 * kFusedHalf + 12) = float4_t{t3[0], t3[0] + t3[1], t3[0] - t3[1], -t3[1]};
+    *reinterpret_cast<float4_t*>(urow + buf * 2 * kWgHalf + 0) = float4_t{t0[0], t0[0] + t0[1], t0[0] - t0[1], -t0[1]};
+    *reinterpret_cast<float4_t*>(urow + buf * 2 * kWgHalf + 4) = float4_t{t1[0], t1[0] + t1[1], t1[0] - t1[1], -t1[1]};
+    *reinterpret_cast<float4_t*>(urow + buf * 2 * kWgHalf + 8) = float4_t{t2[0], t2[0] + t2[1], t2[0] - t2[1], -t2[1]};
+    *reinterpret_cast<float4_t*>(urow + buf * 2 * kWgHalf + 12) = float4_t{t3[0], t3[0] + t3[1], t3[0] - t3[1], -t3[1]};
     if (++staged < nchunks) advance(cs);
   };
 
@@ -590,8 +620,8 @@ __global__ __launch_bounds__(kThreads) void fused_wgrad_kernel(const FWPlan p, c
   const int wk = (wave >> 1) * 32, wc = (wave & 1) * 32;
   const int r = lane & 31, half = lane >> 5;
   // operands: row (tile 2 s + half, output wk + r) of Ud and (tile 2 s + half, input wc + r) of Vx
-  const float* const arow = lds + (half * FK + wk + r) * LP;
-  const float* const brow = lds + kFusedHalf + (half * FT + wc + r) * LP;
+  const float* const arow = lds + half * kWgTile + (wk + r) * LP;
+  const float* const brow = lds + kWgHalf + half * kWgTile + (wc + r) * LP;
   float4_t ca[2], cbv[2];
 #pragma unroll
   for (int q = 0; q < 2; ++q) ca[q] = cbv[q] = float4_t{0.f, 0.f, 0.f, 0.f};
@@ -608,8 +638,8 @@ __global__ __launch_bounds__(kThreads) void fused_wgrad_kernel(const FWPlan p, c
     for (int s2 = 0; s2 < FC / 2; ++s2)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        av[s2][q] = *reinterpret_cast<const float4_t*>(arow + buf * 2 * kFusedHalf + 2 * s2 * FK * LP + 4 * q);
-        bv[s2][q] = *reinterpret_cast<const float4_t*>(brow + buf * 2 * kFusedHalf + 2 * s2 * FT * LP + 4 * q);
+        av[s2][q] = *reinterpret_cast<const float4_t*>(arow + buf * 2 * kWgHalf + 2 * s2 * kWgTile + 4 * q);
+        bv[s2][q] = *reinterpret_cast<const float4_t*>(brow + buf * 2 * kWgHalf + 2 * s2 * kWgTile + 4 * q);
       }
 #pragma unroll
     for (int i = 0; i < 24; ++i) {  // step 0: 16 positions, step 1: positions 0..7
@@ -623,37 +653,58 @@ __global__ __launch_bounds__(kThreads) void fused_wgrad_kernel(const FWPlan p, c
       cbv[q] = bv[1][2 + q];
     }
   };
-  auto interleave = [&]() {
+  auto interleave = [&](int nloads) {
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);              // one MFMA
       if (i < 8) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);   // two LDS reads
-      if (i >= 4 && i < 20) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global load
+      if (i >= 4 && i < 4 + nloads) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global load
       __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);              // VALU
       if (i >= 24) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); // one LDS write
     }
   };
-  const int steps = (nchunks + 3) & ~3;
-  fetch(d0, e0);
-  fetch(d1, e1);
-  fetch(d2, e2);
-  fetch(d3, e3);
-  stage(0, d0, e0);
+  const int steps = (nchunks + 7) & ~7;
+  // chunks 0..3 whole, and the first part of chunks 4..7 (which step 7 of the loop body issues
+  // for the following pass)
+  group_begin();
+  MN_WINO_PART01(0, p0, p1, p2, p3, f0, f1, f2, f3)
+  MN_WINO_PART01(1, p0, p1, p2, p3, f0, f1, f2, f3)
+  MN_WINO_PART23(0, 1, p0, p1)
+  MN_WINO_PART23(2, 3, p2, p3)
+  group_begin();
+  MN_WINO_PART01(0, q0, q1, q2, q3, g0, g1, g2, g3)
+  stage(0, p0, f0);
   __syncthreads();
-#define MN_WINO_WSTEP(buf, dk, ek, dn, en) \
-  fetch(dk, ek);                           \
+  // one step: a part of the other bank's loads, multiply chunk c, stage chunk c + 1
+#define MN_WINO_WSTEP(buf, nloads, dn, en) \
   tail();                                  \
   head(buf);                               \
   stage((buf) ^ 1, dn, en);                \
-  interleave();                            \
+  interleave(nloads);                      \
   __syncthreads();
-  for (int ch = 0; ch < steps; ch += 4) {
-    MN_WINO_WSTEP(0, d0, e0, d1, e1)
-    MN_WINO_WSTEP(1, d1, e1, d2, e2)
-    MN_WINO_WSTEP(0, d2, e2, d3, e3)
-    MN_WINO_WSTEP(1, d3, e3, d0, e0)
+  for (int ch = 0; ch < steps; ch += 8) {
+    MN_WINO_PART01(1, q0, q1, q2, q3, g0, g1, g2, g3)
+    MN_WINO_WSTEP(0, 16, p1, f1)
+    MN_WINO_PART23(0, 1, q0, q1)
+    MN_WINO_WSTEP(1, 12, p2, f2)
+    MN_WINO_PART23(2, 3, q2, q3)
+    MN_WINO_WSTEP(0, 12, p3, f3)
+    group_begin();  // chunks ch + 8 .. ch + 11: bank p is free (its last chunk was staged a step ago)
+    MN_WINO_PART01(0, p0, p1, p2, p3, f0, f1, f2, f3)
+    MN_WINO_WSTEP(1, 16, q0, g0)
+    MN_WINO_PART01(1, p0, p1, p2, p3, f0, f1, f2, f3)
+    MN_WINO_WSTEP(0, 16, q1, g1)
+    MN_WINO_PART23(0, 1, p0, p1)
+    MN_WINO_WSTEP(1, 12, q2, g2)
+    MN_WINO_PART23(2, 3, p2, p3)
+    MN_WINO_WSTEP(0, 12, q3, g3)
+    group_begin();  // chunks ch + 12 .. ch + 15 into bank q
+    MN_WINO_PART01(0, q0, q1, q2, q3, g0, g1, g2, g3)
+    MN_WINO_WSTEP(1, 16, p0, f0)
   }
 #undef MN_WINO_WSTEP
+#undef MN_WINO_PART01
+#undef MN_WINO_PART23
   tail();
 
   if (BIAS && cb == 0) {
@@ -1023,9 +1074,9 @@ static bool fused_lds_allowed() {
       hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_kernel<false>),
                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)kFusedLds) == hipSuccess &&
       hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_wgrad_kernel<true>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kFusedLds) == hipSuccess &&
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWgLds) == hipSuccess &&
       hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_wgrad_kernel<false>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kFusedLds) == hipSuccess;
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWgLds) == hipSuccess;
   done[dev] = ok;
   return ok;
 }
@@ -1186,9 +1237,9 @@ int mn_wino_fused_bwd_weight(const mn_conv2d* g, const float* dy, const float* x
   float* dbp = Z + zf;
   const uint32_t grid = (uint32_t)(f.K / FK) * (f.C / FT) * f.S;
   if (db)
-    fused_wgrad_kernel<true><<<grid, kThreads, kFusedLds, s>>>(f, x, dy, Z, dbp);
+    fused_wgrad_kernel<true><<<grid, kThreads, kWgLds, s>>>(f, x, dy, Z, dbp);
   else
-    fused_wgrad_kernel<false><<<grid, kThreads, kFusedLds, s>>>(f, x, dy, Z, dbp);
+    fused_wgrad_kernel<false><<<grid, kThreads, kWgLds, s>>>(f, x, dy, Z, dbp);
   const uint32_t n = (uint32_t)f.K * f.C;
   wgrad_output_kernel<false><<<(n + 63) / 64, kThreads, 0, s>>>(Z, dw, f.K, f.C, f.S);
   if (db) bias_ranges_kernel<<<(f.K + kThreads - 1) / kThreads, kThreads, 0, s>>>(dbp, db, f.K, f.S);
