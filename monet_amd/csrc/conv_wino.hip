@@ -435,21 +435,16 @@ __global__ __launch_bounds__(kThreads) void fused_kernel(const Plan p, const flo
 // Z[pos][k][c] = sum_t Ud[pos][t][k] Vx[pos][t][c] is a product over the TILES, so a workgroup owns
 // 64 outputs x 64 inputs x 16 positions (the accumulator shape of the forward kernel above, 256
 // registers per lane) and walks a range of tile rows, four tiles of a row per chunk: per chunk a
-// thread loads one 4x4 patch of x and one 2x2 patch of dy, transforms them and writes one row of
-// Vx and of Ud (the LDS layout, the operand reads and the 32 matrix instructions per chunk are
-// the forward kernel's with "channel of the chunk" read as "tile of the chunk").
-// Lanes: 16 channels x 4 neighbouring tiles per wavefront, so a load touches 16 cache lines and
-// not 64 (a lane per channel plane was measured 1.5-1.7x slower in the forward kernel).  All
-// addresses are scalars per chunk plus byte offsets that never change per lane: the row and the
-// chunk's first column travel in the scalar offset of the buffer loads.  The padding is not
-// addressed: rows beyond the image are read from the nearest row, columns -1 and W from a
-// neighbouring element, and the values are replaced by zero before the transform.
+// thread transforms one 4x4 patch of x and one 2x2 patch of dy and writes one row of Vx and of Ud
+// (the LDS layout, the operand reads and the 32 matrix instructions per chunk are the forward
+// kernel's with "channel of the chunk" read as "tile of the chunk"; a tile's block of 64 rows is
+// padded by 16 floats: the four tiles of a channel are written by neighbouring lanes, and 64 * LP
+// is a multiple of the 64 banks, a 4-way conflict on every staging write otherwise).
 // The result of a range of tile rows goes to Z[pos][range][k][c]; wgrad_output_kernel adds the
 // ranges in order and applies G^T . G (reproducible).
 // Needs: 3x3, stride 1, padding 1, H and W even, W % 8 == 0, K % 64 == 0, C % 64 == 0.
 constexpr int kWgTile = FK * LP + 16;                   // floats of one tile's 64 rows (FK == FT), padded
 constexpr int kWgHalf = FC * kWgTile;                   // floats of Ud (or Vx) in one buffer
-constexpr size_t kWgLds = (size_t)4 * kWgHalf * sizeof(float);  // 81 KB
 static_assert(FK == FT, "one row count for both operands");
 struct FWPlan {
   int N, C, K, H, W;
@@ -460,148 +455,145 @@ struct FWPlan {
   uint32_t x_bytes, dy_bytes;
 };
 
+// The source rows are staged RAW in LDS first.  Loading one 4x4 patch per lane straight from
+// memory costs 14 load instructions per chunk that each touch 16 cache lines for 4 to 8 bytes per
+// lane (430 million L1 lookups per call at 128 -> 128 channels, 208 x 304), and a chunk only uses
+// 32 bytes of every 128-byte line it touches while the CU's lines of one chunk (48 KB) do not fit
+// its L1: every line came from L2 four times (1.44 ms; 1.32 ms with the loads of four chunks
+// issued together; 0.94 ms with the same instructions on cache-resident addresses).  Here the
+// workgroup copies, for a GROUP of four chunks (32 output columns of one tile row), the 64
+// channels x 4 rows x 40 columns of x and the 64 outputs x 2 rows x 32 columns of dy into LDS with
+// 16-byte loads along the rows (14 per thread and group instead of 56, whole lines: 1.15 ms, of
+// which the loads are 1 %), and every lane then reads its patches from LDS.  Out-of-image rows and
+// columns are written as zeros at that point (a load whose offset is beyond the buffer), so
+// staging a chunk has no masks.  A tile row whose chunk count is no multiple of 4 is padded with
+// chunks of zeros.  The raw rows are single-buffered (59 KB beside the 81 KB of transformed
+// operands): the group's registers are written to LDS in the step that stages the group's first
+// chunk, with one more barrier in the middle of that step.
 // BIAS: the workgroups of input block 0 also add up the gradient tiles they stage; their sums per
 // (range, output) go to dbp[range][k] and bias_ranges_kernel adds the ranges in order.
+constexpr int kRawXRow = 40;                  // floats of an input row piece: columns 32 Q - 4 .. 32 Q + 35
+constexpr int kRawXCh = 4 * kRawXRow + 4;     // per channel, padded: 16 channels start in 16 different banks
+constexpr int kRawDyRow = 32;
+constexpr int kRawDyCh = 2 * kRawDyRow + 4;
+constexpr int kRawX = FT * kRawXCh, kRawDy = FK * kRawDyCh;
+constexpr int kRawXItems = FT * 4 * (kRawXRow / 4) / kThreads;   // 16-byte pieces per thread: 10
+constexpr int kRawDyItems = FK * 2 * (kRawDyRow / 4) / kThreads;  // 4
+constexpr size_t kWgRowsLds = (size_t)(4 * kWgHalf + kRawX + kRawDy) * sizeof(float);  // 139 KB
+static_assert(FT * 4 * (kRawXRow / 4) % kThreads == 0 && FK * 2 * (kRawDyRow / 4) % kThreads == 0, "whole items");
+
 template <bool BIAS>
 __global__ __launch_bounds__(kThreads) void fused_wgrad_kernel(const FWPlan p, const float* __restrict__ x,
-                                                               const float* __restrict__ dy,
-                                                               float* __restrict__ Z, float* __restrict__ dbp) {
-  extern __shared__ float4_t fused_lds[];  // [buffer][Ud | Vx][tile of the chunk][channel][LP]
+                                                                    const float* __restrict__ dy,
+                                                                    float* __restrict__ Z,
+                                                                    float* __restrict__ dbp) {
+  extern __shared__ float4_t fused_lds[];  // [buffer][Ud | Vx][tile of the chunk][channel][LP], raw x, raw dy
   float* const lds = reinterpret_cast<float*>(fused_lds);
+  float* const raw_x = lds + 4 * kWgHalf;
+  float* const raw_dy = raw_x + kRawX;
   const uint32_t slot = xcd_slot();
   const uint32_t ncb = (uint32_t)p.C / FT, blocks = ((uint32_t)p.K / FK) * ncb;
   const uint32_t blk = slot % blocks, range = slot / blocks;  // neighbours read the same tile rows
   const uint32_t kb = blk / ncb, cb = blk - kb * ncb;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int ci = 16 * wave + (lane >> 2), ti = lane & 3;   // loader role: channel, tile of the chunk
+  const int ci = 16 * wave + (lane >> 2), ti = lane & 3;   // staging role: channel, tile of the chunk
   const uint32_t r_begin = range * p.rows_per_range;
   const uint32_t r_end = min(r_begin + p.rows_per_range, p.rows);
-  const int cpr = p.TW >> 2;                                // chunks per tile row
-  const int nchunks = (int)(r_end - r_begin) * cpr;         // real chunks (the loop runs a multiple of 4)
+  const int cpr = p.TW >> 2;                               // chunks per tile row
+  const int gpr = (cpr + 3) >> 2;                          // groups per tile row
+  const int ngroups = (int)(r_end - r_begin) * gpr;
   const uint32_t plane = (uint32_t)p.H * p.W;
+  constexpr uint32_t kBeyond = 0x80000000u;
 
   const __amdgpu_buffer_rsrc_t x_buf =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(x), 0, p.x_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t dy_buf =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(dy), 0, p.dy_bytes, 0x00020000);
-  // byte offsets of this lane inside (image 0, row 0, first chunk): columns 2 ti - 1 .. 2 ti + 2
-  const uint32_t xc = (cb * FT + ci) * plane;
-  const uint32_t x_mid = (xc + 2 * ti) * 4u;                         // columns 2 ti, 2 ti + 1 (8 bytes)
-  const uint32_t x_left0 = (xc + (ti ? 2 * ti - 1 : 0)) * 4u;        // first chunk of a row (column -1 is replaced)
-  const uint32_t x_left = (xc + 2 * ti + 7) * 4u;                    // later chunks, with the scalar offset one chunk back
-  const uint32_t x_right = (xc + 2 * ti + 2) * 4u;
-  const uint32_t x_right_last = (xc + (ti == 3 ? 2 * ti + 1 : 2 * ti + 2)) * 4u;  // last chunk (column W is replaced)
-  const uint32_t dy_off = ((kb * FK + ci) * plane + 2 * ti) * 4u;
-
-  // position of the next chunk to fetch and of the next chunk to stage (all scalar)
-  struct Cursor {
-    int n, th, q;
-  };
-  auto start = [&]() {
-    Cursor c;
-    c.n = (int)(r_begin / (uint32_t)p.TH);
-    c.th = (int)(r_begin - (uint32_t)c.n * p.TH);
-    c.q = 0;
-    return c;
-  };
-  auto advance = [&](Cursor& c) {
-    if (++c.q == cpr) {
-      c.q = 0;
-      if (++c.th == p.TH) {
-        c.th = 0;
-        ++c.n;
+  // copier role: piece i = tid + 256 u of [channel][row][16-byte piece]; what never changes
+  uint32_t x_const[kRawXItems], x_af[kRawXItems], d_const[kRawDyItems], d_f[kRawDyItems];
+  int x_lds[kRawXItems], d_lds[kRawDyItems];
+#pragma unroll
+  for (int u = 0; u < kRawXItems; ++u) {
+    const int i = tid + u * kThreads, ch = i / 40, rem = i - ch * 40, a = rem / 10, f = rem - a * 10;
+    x_const[u] = ((cb * FT + ch) * plane + a * p.W + 4 * f) * 4u;
+    x_af[u] = a | (f << 8);
+    x_lds[u] = ch * kRawXCh + a * kRawXRow + 4 * f;
+  }
+#pragma unroll
+  for (int u = 0; u < kRawDyItems; ++u) {
+    const int i = tid + u * kThreads, k = i >> 4, rem = i & 15, a = rem >> 3, f = rem & 7;
+    d_const[u] = ((kb * FK + k) * plane + a * p.W + 4 * f) * 4u;
+    d_f[u] = f;
+    d_lds[u] = k * kRawDyCh + a * kRawDyRow + 4 * f;
+  }
+  // the next group to copy (scalar): image, tile row, group of the row
+  int gn = (int)(r_begin / (uint32_t)p.TH), gth = (int)(r_begin - (uint32_t)gn * p.TH), gq = 0, copied = 0;
+  float4_t rx[kRawXItems], rd[kRawDyItems];
+  auto fetch_group = [&]() {
+    const bool real = copied < ngroups;  // past the end: every piece reads as zeros
+    // byte offset of (row 2 th - 1, column 32 Q - 4) of channel 0 / (row 2 th, column 32 Q) of
+    // output 0; pieces outside the image are the only ones whose sum with it is negative
+    const uint32_t x_term = (uint32_t)(((gn * p.C * p.H + 2 * gth - 1) * p.W + 32 * gq - 4) * 4);
+    const uint32_t d_term = (uint32_t)(((gn * p.K * p.H + 2 * gth) * p.W + 32 * gq) * 4);
+    const bool top = gth == 0, bottom = gth == p.TH - 1;
+    const int f_first = gq == 0 ? 1 : 0;                 // piece 0 of the first group is columns -4 .. -1
+    const int f_end = (p.W - 32 * gq + 4) >> 2;          // first piece that starts at or beyond column W
+#pragma unroll
+    for (int u = 0; u < kRawXItems; ++u) {
+      const int a = x_af[u] & 255, f = x_af[u] >> 8;
+      const bool ok = real && !(top && a == 0) && !(bottom && a == 3) && f >= f_first && f < f_end;
+      rx[u] = __builtin_bit_cast(
+          float4_t, __builtin_amdgcn_raw_buffer_load_b128(x_buf, ok ? x_const[u] + x_term : kBeyond, 0, 0));
+    }
+#pragma unroll
+    for (int u = 0; u < kRawDyItems; ++u) {
+      const bool ok = real && (int)d_f[u] < f_end - 1;   // columns 32 Q + 4 f < W
+      rd[u] = __builtin_bit_cast(
+          float4_t, __builtin_amdgcn_raw_buffer_load_b128(dy_buf, ok ? d_const[u] + d_term : kBeyond, 0, 0));
+    }
+    ++copied;
+    if (++gq == gpr) {
+      gq = 0;
+      if (++gth == p.TH) {
+        gth = 0;
+        ++gn;
       }
     }
   };
-  Cursor cf = start(), cs = start();
-  int fetched = 0, staged = 0;
-  float bsum = 0.f;
-
-  // Eight register sets in two banks of four consecutive chunks.  The loads of a bank are issued
-  // row by row for its four chunks together: four chunks of a tile row cover the same 128-byte
-  // lines (a chunk is 32 bytes of each row), and a CU's chunk touches 384 lines = 48 KB, more than
-  // the L1 holds, so loaded chunk by chunk every line came from L2 four times (with the same
-  // load instructions on cache-resident addresses the kernel ran 1.37 -> 0.94 ms).
-  float p0[4][4], p1[4][4], p2[4][4], p3[4][4], q0[4][4], q1[4][4], q2[4][4], q3[4][4];
-  float f0[2][2], f1[2][2], f2[2][2], f3[2][2], g0[2][2], g1[2][2], g2[2][2], g3[2][2];
-  Cursor gc[4] = {cf, cf, cf, cf};  // the four chunks of the bank being loaded
-  auto group_begin = [&]() {
-    // past the last chunk the last one is loaded again (no branch around the loads) and not used
+  auto write_raw = [&]() {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      gc[i] = cf;
-      if (++fetched < nchunks) advance(cf);
-    }
+    for (int u = 0; u < kRawXItems; ++u) *reinterpret_cast<float4_t*>(raw_x + x_lds[u]) = rx[u];
+#pragma unroll
+    for (int u = 0; u < kRawDyItems; ++u) *reinterpret_cast<float4_t*>(raw_dy + d_lds[u]) = rd[u];
   };
-  auto fetch_x = [&](int a, const Cursor& c, float (&d)[4][4]) {  // row a of chunk c's patches
-    const bool first = c.q == 0, last = c.q == cpr - 1;
-    const uint32_t vl = first ? x_left0 : x_left, vr = last ? x_right_last : x_right;
-    const int col = 8 * c.q;
-    const int colL = first ? 0 : col - 8;
-    int row = 2 * c.th - 1 + a;
-    row = row < 0 ? 0 : (row >= p.H ? p.H - 1 : row);
-    const int base = (c.n * p.C * p.H + row) * p.W;
-    const int so = __builtin_amdgcn_readfirstlane((base + col) * 4);
-    const int sl = __builtin_amdgcn_readfirstlane((base + colL) * 4);
-    d[a][0] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(x_buf, vl, sl, 0));
-    typedef uint32_t u2 __attribute__((ext_vector_type(2)));
-    const u2 mid = __builtin_amdgcn_raw_buffer_load_b64(x_buf, x_mid, so, 0);
-    d[a][1] = __uint_as_float(mid[0]);
-    d[a][2] = __uint_as_float(mid[1]);
-    d[a][3] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(x_buf, vr, so, 0));
-  };
-  auto fetch_dy = [&](int a, const Cursor& c, float (&e)[2][2]) {
-    const int base = (c.n * p.K * p.H + 2 * c.th + a) * p.W + 8 * c.q;
-    const int so = __builtin_amdgcn_readfirstlane(base * 4);
-    typedef uint32_t u2 __attribute__((ext_vector_type(2)));
-    const u2 v = __builtin_amdgcn_raw_buffer_load_b64(dy_buf, dy_off, so, 0);
-    e[a][0] = __uint_as_float(v[0]);
-    e[a][1] = __uint_as_float(v[1]);
-  };
-  // the four parts of a bank's loads, one per step: rows 0 and 1 of all four chunks (with the
-  // gradient rows), then rows 2 and 3 of the first two and of the last two chunks
-#define MN_WINO_PART01(a, A, B, C, D, EA, EB, EC, ED) \
-  fetch_x(a, gc[0], A);                               \
-  fetch_x(a, gc[1], B);                               \
-  fetch_x(a, gc[2], C);                               \
-  fetch_x(a, gc[3], D);                               \
-  fetch_dy(a, gc[0], EA);                             \
-  fetch_dy(a, gc[1], EB);                             \
-  fetch_dy(a, gc[2], EC);                             \
-  fetch_dy(a, gc[3], ED);
-#define MN_WINO_PART23(i, j, A, B) \
-  fetch_x(2, gc[i], A);            \
-  fetch_x(2, gc[j], B);            \
-  fetch_x(3, gc[i], A);            \
-  fetch_x(3, gc[j], B);
-  // row (tile ti, channel ci): the four tiles of a channel are written by neighbouring lanes, so
-  // a tile's block of 64 rows is padded by 16 floats (64 * LP is a multiple of the 64 banks: the
-  // four lanes of a channel would hit the same banks, a 4-way conflict on every staging write)
+  float bsum = 0.f;
+  // this lane's patches of chunk j of the group in LDS: columns 8 j + 2 ti - 1 .. + 2 of the rows
+  // (the staged piece starts at column - 4), and its 2x2 gradient tile
+  const float* const px = raw_x + ci * kRawXCh + 3 + 2 * ti;
+  const float* const pd = raw_dy + ci * kRawDyCh + 2 * ti;
   float* const vrow = lds + kWgHalf + ti * kWgTile + ci * LP;
   float* const urow = lds + ti * kWgTile + ci * LP;
-  auto stage = [&](int buf, float (&d)[4][4], float (&e)[2][2]) {
-    const bool live = staged < nchunks;
-    const bool top = cs.th == 0, bottom = cs.th == p.TH - 1;
-    const bool left = cs.q == 0 && ti == 0, right = cs.q == cpr - 1 && ti == 3;
-#pragma unroll
-    for (int b = 0; b < 4; ++b) {
-      d[0][b] = top ? 0.f : d[0][b];
-      d[3][b] = bottom ? 0.f : d[3][b];
-    }
+  auto stage = [&](int buf, int j) {
+    float d[4][4];
+    typedef float f2 __attribute__((ext_vector_type(2)));
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
-      d[a][0] = left ? 0.f : d[a][0];
-      d[a][3] = right ? 0.f : d[a][3];
+      const float* row = px + a * kRawXRow + 8 * j;
+      d[a][0] = row[0];
+      const f2 mid = *reinterpret_cast<const f2*>(row + 1);
+      d[a][1] = mid[0];
+      d[a][2] = mid[1];
+      d[a][3] = row[3];
     }
+    const f2 ea = *reinterpret_cast<const f2*>(pd + 8 * j), eb = *reinterpret_cast<const f2*>(pd + kRawDyRow + 8 * j);
     float v[16];
     input_transform(d, v);
 #pragma unroll
     for (int q = 0; q < 4; ++q)
       *reinterpret_cast<float4_t*>(vrow + buf * 2 * kWgHalf + 4 * q) =
           float4_t{v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]};
-    // A e A^T, A = [1 0; 1 1; 1 -1; 0 -1]; a chunk past the end contributes nothing
-    const float e00 = live ? e[0][0] : 0.f, e01 = live ? e[0][1] : 0.f;
-    const float e10 = live ? e[1][0] : 0.f, e11 = live ? e[1][1] : 0.f;
+    // A e A^T, A = [1 0; 1 1; 1 -1; 0 -1]
+    const float e00 = ea[0], e01 = ea[1], e10 = eb[0], e11 = eb[1];
     const float t0[2] = {e00, e01}, t1[2] = {e00 + e10, e01 + e11}, t2[2] = {e00 - e10, e01 - e11},
                 t3[2] = {-e10, -e11};
     if (BIAS) bsum += t1[0] + t1[1];
@@ -609,7 +601,6 @@ __global__ __launch_bounds__(kThreads) void fused_wgrad_kernel(const FWPlan p, c
     *reinterpret_cast<float4_t*>(urow + buf * 2 * kWgHalf + 4) = float4_t{t1[0], t1[0] + t1[1], t1[0] - t1[1], -t1[1]};
     *reinterpret_cast<float4_t*>(urow + buf * 2 * kWgHalf + 8) = float4_t{t2[0], t2[0] + t2[1], t2[0] - t2[1], -t2[1]};
     *reinterpret_cast<float4_t*>(urow + buf * 2 * kWgHalf + 12) = float4_t{t3[0], t3[0] + t3[1], t3[0] - t3[1], -t3[1]};
-    if (++staged < nchunks) advance(cs);
   };
 
   float16_t acc[16];
@@ -632,8 +623,8 @@ __global__ __launch_bounds__(kThreads) void fused_wgrad_kernel(const FWPlan p, c
       for (int e = 0; e < 4; ++e)
         acc[8 + 4 * q + e] = __builtin_amdgcn_mfma_f32_32x32x2f32(ca[q][e], cbv[q][e], acc[8 + 4 * q + e], 0, 0, 0);
   };
-  auto head = [&](int buf) {
-    float4_t av[FC / 2][4], bv[FC / 2][4];
+  float4_t av[FC / 2][4], bv[FC / 2][4];
+  auto head_read = [&](int buf) {
 #pragma unroll
     for (int s2 = 0; s2 < FC / 2; ++s2)
 #pragma unroll
@@ -641,12 +632,16 @@ __global__ __launch_bounds__(kThreads) void fused_wgrad_kernel(const FWPlan p, c
         av[s2][q] = *reinterpret_cast<const float4_t*>(arow + buf * 2 * kWgHalf + 2 * s2 * kWgTile + 4 * q);
         bv[s2][q] = *reinterpret_cast<const float4_t*>(brow + buf * 2 * kWgHalf + 2 * s2 * kWgTile + 4 * q);
       }
+  };
+  auto head_mul = [&](int from, int to) {  // step 0: 16 positions, step 1: positions 0..7
 #pragma unroll
-    for (int i = 0; i < 24; ++i) {  // step 0: 16 positions, step 1: positions 0..7
+    for (int i = from; i < to; ++i) {
       const int s2 = i >> 4, pos = i & 15;
       acc[pos] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[s2][pos >> 2][pos & 3], bv[s2][pos >> 2][pos & 3],
                                                       acc[pos], 0, 0, 0);
     }
+  };
+  auto head_keep = [&]() {
 #pragma unroll
     for (int q = 0; q < 2; ++q) {
       ca[q] = av[1][2 + q];
@@ -657,54 +652,53 @@ __global__ __launch_bounds__(kThreads) void fused_wgrad_kernel(const FWPlan p, c
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);              // one MFMA
-      if (i < 8) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);   // two LDS reads
+      if (i < 11) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // two LDS reads (16 operand, 14 patch... the rest follows)
       if (i >= 4 && i < 4 + nloads) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global load
       __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);              // VALU
       if (i >= 24) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); // one LDS write
     }
   };
-  const int steps = (nchunks + 7) & ~7;
-  // chunks 0..3 whole, and the first part of chunks 4..7 (which step 7 of the loop body issues
-  // for the following pass)
-  group_begin();
-  MN_WINO_PART01(0, p0, p1, p2, p3, f0, f1, f2, f3)
-  MN_WINO_PART01(1, p0, p1, p2, p3, f0, f1, f2, f3)
-  MN_WINO_PART23(0, 1, p0, p1)
-  MN_WINO_PART23(2, 3, p2, p3)
-  group_begin();
-  MN_WINO_PART01(0, q0, q1, q2, q3, g0, g1, g2, g3)
-  stage(0, p0, f0);
+  fetch_group();
+  write_raw();
   __syncthreads();
-  // one step: a part of the other bank's loads, multiply chunk c, stage chunk c + 1
-#define MN_WINO_WSTEP(buf, nloads, dn, en) \
-  tail();                                  \
-  head(buf);                               \
-  stage((buf) ^ 1, dn, en);                \
-  interleave(nloads);                      \
+  stage(0, 0);
   __syncthreads();
-  for (int ch = 0; ch < steps; ch += 8) {
-    MN_WINO_PART01(1, q0, q1, q2, q3, g0, g1, g2, g3)
-    MN_WINO_WSTEP(0, 16, p1, f1)
-    MN_WINO_PART23(0, 1, q0, q1)
-    MN_WINO_WSTEP(1, 12, p2, f2)
-    MN_WINO_PART23(2, 3, q2, q3)
-    MN_WINO_WSTEP(0, 12, p3, f3)
-    group_begin();  // chunks ch + 8 .. ch + 11: bank p is free (its last chunk was staged a step ago)
-    MN_WINO_PART01(0, p0, p1, p2, p3, f0, f1, f2, f3)
-    MN_WINO_WSTEP(1, 16, q0, g0)
-    MN_WINO_PART01(1, p0, p1, p2, p3, f0, f1, f2, f3)
-    MN_WINO_WSTEP(0, 16, q1, g1)
-    MN_WINO_PART23(0, 1, p0, p1)
-    MN_WINO_WSTEP(1, 12, q2, g2)
-    MN_WINO_PART23(2, 3, p2, p3)
-    MN_WINO_WSTEP(0, 12, q3, g3)
-    group_begin();  // chunks ch + 12 .. ch + 15 into bank q
-    MN_WINO_PART01(0, q0, q1, q2, q3, g0, g1, g2, g3)
-    MN_WINO_WSTEP(1, 16, p0, f0)
+  for (int g = 0; g < ngroups; ++g) {
+    // step 0 of the group: request the next group's rows; chunks 1..3 are staged in steps 0..2
+    fetch_group();
+    tail();
+    head_read(0);
+    head_mul(0, 24);
+    head_keep();
+    stage(1, 1);
+    interleave(kRawXItems + kRawDyItems);
+    __syncthreads();
+    tail();
+    head_read(1);
+    head_mul(0, 24);
+    head_keep();
+    stage(0, 2);
+    interleave(0);
+    __syncthreads();
+    tail();
+    head_read(0);
+    head_mul(0, 24);
+    head_keep();
+    stage(1, 3);
+    interleave(0);
+    __syncthreads();
+    // step 3: the next group's rows go to LDS (the barrier above was the last reader's), and after
+    // one more barrier its first chunk is staged
+    write_raw();
+    tail();
+    head_read(1);
+    head_mul(0, 12);
+    __syncthreads();
+    head_mul(12, 24);
+    head_keep();
+    stage(0, 0);
+    __syncthreads();
   }
-#undef MN_WINO_WSTEP
-#undef MN_WINO_PART01
-#undef MN_WINO_PART23
   tail();
 
   if (BIAS && cb == 0) {
@@ -1059,7 +1053,8 @@ static int run(Plan p, const float* src, const float* w, bool flip, const float*
   return mn_launch_status();
 }
 
-// The fused kernel uses 80 KB of LDS per workgroup, more than a kernel gets without asking:
+// The fused kernels use 80 KB (forward, backward-data) and 139 KB (backward-weight) of LDS per
+// workgroup, more than a kernel gets without asking:
 // raise its limit once per device (gfx950 has 160 KB per CU).
 static bool fused_lds_allowed() {
   static std::mutex lock;
@@ -1074,9 +1069,9 @@ static bool fused_lds_allowed() {
       hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_kernel<false>),
                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)kFusedLds) == hipSuccess &&
       hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_wgrad_kernel<true>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWgLds) == hipSuccess &&
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWgRowsLds) == hipSuccess &&
       hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_wgrad_kernel<false>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWgLds) == hipSuccess;
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWgRowsLds) == hipSuccess;
   done[dev] = ok;
   return ok;
 }
@@ -1197,7 +1192,7 @@ static bool make_fwplan(const mn_conv2d* g, FWPlan& f) {
   f.rows = (uint32_t)g->N * f.TH;
   f.x_bytes = (uint32_t)xb;
   f.dy_bytes = (uint32_t)yb;
-  // one workgroup per CU (256 accumulation registers per lane, 80 KB of LDS): as many ranges of
+  // one workgroup per CU (256 accumulation registers per lane, 139 KB of LDS): as many ranges of
   // tile rows as that leaves per (output, input) block
   int dev = 0, cus = 256;
   if (hipGetDevice(&dev) != hipSuccess ||
@@ -1237,9 +1232,9 @@ int mn_wino_fused_bwd_weight(const mn_conv2d* g, const float* dy, const float* x
   float* dbp = Z + zf;
   const uint32_t grid = (uint32_t)(f.K / FK) * (f.C / FT) * f.S;
   if (db)
-    fused_wgrad_kernel<true><<<grid, kThreads, kWgLds, s>>>(f, x, dy, Z, dbp);
+    fused_wgrad_kernel<true><<<grid, kThreads, kWgRowsLds, s>>>(f, x, dy, Z, dbp);
   else
-    fused_wgrad_kernel<false><<<grid, kThreads, kWgLds, s>>>(f, x, dy, Z, dbp);
+    fused_wgrad_kernel<false><<<grid, kThreads, kWgRowsLds, s>>>(f, x, dy, Z, dbp);
   const uint32_t n = (uint32_t)f.K * f.C;
   wgrad_output_kernel<false><<<(n + 63) / 64, kThreads, 0, s>>>(Z, dw, f.K, f.C, f.S);
   if (db) bias_ranges_kernel<<<(f.K + kThreads - 1) / kThreads, kThreads, 0, s>>>(dbp, db, f.K, f.S);
