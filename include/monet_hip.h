@@ -406,7 +406,7 @@ typedef struct mn_conv2d {
  *                      reproducible
  *                    3 the same algorithm in one kernel: both transforms are
  *                      applied on the way into LDS, no transformed tensors in
- *                      memory; padding 1, even planes with W a multiple of 8,
+ *                      memory; padding 1, even height, W a multiple of 4,
  *                      K and C multiples of 64; workspace: the partial
  *                      results of at most one range of tile rows per CU
  *                      (16 * ranges * K * C floats, and ranges * K for the

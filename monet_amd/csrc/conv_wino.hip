@@ -442,7 +442,8 @@ __global__ __launch_bounds__(kThreads) void fused_kernel(const Plan p, const flo
 // is a multiple of the 64 banks, a 4-way conflict on every staging write otherwise).
 // The result of a range of tile rows goes to Z[pos][range][k][c]; wgrad_output_kernel adds the
 // ranges in order and applies G^T . G (reproducible).
-// Needs: 3x3, stride 1, padding 1, H and W even, W % 8 == 0, K % 64 == 0, C % 64 == 0.
+// Needs: 3x3, stride 1, padding 1, H even, W % 4 == 0 (16-byte pieces of a row; a last chunk with
+// fewer than four tiles multiplies zeros), K % 64 == 0, C % 64 == 0.
 constexpr int kWgTile = FK * LP + 16;                   // floats of one tile's 64 rows (FK == FT), padded
 constexpr int kWgHalf = FC * kWgTile;                   // floats of Ud (or Vx) in one buffer
 static_assert(FK == FT, "one row count for both operands");
@@ -499,7 +500,7 @@ __global__ __launch_bounds__(kThreads) void fused_wgrad_kernel(const FWPlan p, c
   const int ci = 16 * wave + (lane >> 2), ti = lane & 3;   // staging role: channel, tile of the chunk
   const uint32_t r_begin = range * p.rows_per_range;
   const uint32_t r_end = min(r_begin + p.rows_per_range, p.rows);
-  const int cpr = p.TW >> 2;                               // chunks per tile row
+  const int cpr = (p.TW + 3) >> 2;                         // chunks per tile row (the last may be ragged)
   const int gpr = (cpr + 3) >> 2;                          // groups per tile row
   const int ngroups = (int)(r_end - r_begin) * gpr;
   const uint32_t plane = (uint32_t)p.H * p.W;
@@ -1177,7 +1178,7 @@ int mn_wino_fused_bwd_data(const mn_conv2d* g, const float* dy, const float* w, 
 namespace mn_wino {
 static bool make_fwplan(const mn_conv2d* g, FWPlan& f) {
   if (!shape_ok(g) || g->pH != 1 || g->pW != 1) return false;
-  if (g->H != g->P || g->W != g->Q || (g->H & 1) || (g->W & 7) || g->K % FK != 0 || g->C % FT != 0)
+  if (g->H != g->P || g->W != g->Q || (g->H & 1) || (g->W & 3) || g->K % FK != 0 || g->C % FT != 0)
     return false;
   const unsigned long long xb = (unsigned long long)g->N * g->C * g->H * g->W * 4ull;
   const unsigned long long yb = (unsigned long long)g->N * g->K * g->H * g->W * 4ull;

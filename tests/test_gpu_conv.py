@@ -46,7 +46,7 @@ CASES = [
     # the stem again at odd sizes: forward variant 1 (the kernel of its own) stages scalars and
     # has ragged row blocks
     ((3, 3, 75, 97), (64, 3, 7, 7), 2, 3, 1),
-    # backward-weight variant 3 (Winograd in one kernel): 64-channel blocks, W % 8 == 0; one and
+    # backward-weight variant 3 (Winograd in one kernel): 64-channel blocks, W % 4 == 0; one and
     # several chunks per tile row, ranges of one tile row (padded to four chunks), uneven ranges
     ((2, 64, 16, 16), (64, 64, 3, 3), 1, 1, 1),
     ((3, 128, 24, 32), (64, 128, 3, 3), 1, 1, 1),
@@ -56,6 +56,10 @@ CASES = [
     # is specialised for) with a ragged last row block; more items than workgroups
     ((2, 3, 42, 224), (64, 3, 7, 7), 2, 3, 1),
     ((150, 3, 32, 32), (64, 3, 7, 7), 2, 3, 1),
+    # backward-weight variant 3 with a ragged last chunk (14 and 22 tiles per row) and rows that
+    # need one group and two
+    ((3, 64, 10, 28), (64, 64, 3, 3), 1, 1, 1),
+    ((2, 64, 6, 44), (128, 64, 3, 3), 1, 1, 1),
 ]
 
 
@@ -76,10 +80,10 @@ def winograd_wgrad_applies(xs, ws, st, pad, dil):
 
 def fused_winograd_wgrad_applies(xs, ws, st, pad, dil):
     """Variant 3 of backward-weight (Winograd in one kernel): 3x3, stride 1, dilation 1, padding 1,
-    even planes with W % 8 == 0, K and C multiples of 64."""
+    even height, W % 4 == 0, K and C multiples of 64."""
     pair = lambda v: tuple(v) if isinstance(v, (tuple, list)) else (v, v)
     return (winograd_applies(ws, st, pad, dil, 16) and pair(pad) == (1, 1) and xs[2] % 2 == 0 and
-            xs[3] % 8 == 0 and xs[1] % 64 == 0 and ws[0] % 64 == 0)
+            xs[3] % 4 == 0 and xs[1] % 64 == 0 and ws[0] % 64 == 0)
 
 
 def split_applies(xs, ws, st, pad, dil, reduced_channels):
