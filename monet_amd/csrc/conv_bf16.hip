@@ -832,7 +832,9 @@ __global__ __launch_bounds__(kThreads) void wgrad_reduce_bf16_kernel(
 // ONE tap and a range of the positions; wavefronts 0-3 multiply (2 x 2 of them, TM x TN accumulator
 // tiles of 32 x 32 each), wavefronts 4-7 feed.  Both tensors hold the channels of a position
 // contiguously while the matrix instruction wants 8 consecutive positions per lane: the feeders
-// copy 16-byte chunks into LDS unchanged ([position][channel], rows padded by 32 bytes) and the
+// copy 16-byte chunks into LDS unchanged ([position][channel], rows padded by 64 bytes: four lanes
+// write the 64 bytes of a row piece, so consecutive rows must start 16 banks apart; with 32 bytes
+// of padding the writes of two rows met in 8 banks) and the
 // multiplying wavefronts read the operands with the transposing LDS load (ds_read_b64_tr_b16: 16
 // lanes give the addresses of a 4-position x 16-channel block and lane i receives the 4 positions of
 // channel i), two per operand fragment.  No shuffles, byte permutes or 4-byte LDS stores, which is
@@ -846,7 +848,7 @@ __global__ __launch_bounds__(kRoleThreads) __attribute__((amdgpu_waves_per_eu(2,
     const WGradH g, const bf16_t* __restrict__ dy, const bf16_t* __restrict__ x,
     float* __restrict__ partial, uint32_t tiles, uint32_t stages_per_split) {
   constexpr int BM = 64 * TM, BN = 64 * TN;
-  constexpr int LDA = BM + 16, LDB = BN + 16;      // elements per LDS row
+  constexpr int LDA = BM + 32, LDB = BN + 32;      // elements per LDS row (64 bytes of padding)
   constexpr int kLpr = 256 / kWrDepth;             // feeding threads per position
   constexpr int kA = BM / 8 / kLpr, kB = BN / 8 / kLpr;   // 16-byte chunks per feeding thread and stage
   constexpr uint32_t kBeyond = 0x80000000u;
