@@ -117,8 +117,10 @@ def test_max_pool_indices_at_full_size(cuda):
 
 
 POINTWISE3 = ((184, 1024, 14, 14), (256, 1024, 1, 1))   # ResNet-50 layer3, reducing 1x1
-LAYER1 = ((184, 64, 56, 56), (64, 64, 3, 3))             # ResNet-50 layer1 3x3: W % 8 == 0, so the
-                                                         # one-kernel Winograd backward-weight runs
+LAYER1 = ((184, 64, 56, 56), (64, 64, 3, 3))             # ResNet-50 layer1 3x3: the one-kernel Winograd
+LAYER2 = ((184, 128, 28, 28), (128, 128, 3, 3))          # backward-weight runs; layer2: 14 tiles per row,
+                                                         # a ragged last chunk
+STEM = ((184, 3, 224, 224), (64, 3, 7, 7))               # stride 2: variant 1 = the stem's own kernels
 
 
 def _variants(n, run):
@@ -135,9 +137,12 @@ def _variants(n, run):
 @pytest.mark.parametrize("shape,pad,dtype,tol", [(LAYER3, 1, torch.float32, 1e-5),
                                                  (LAYER3, 1, torch.bfloat16, 1e-2),
                                                  (POINTWISE3, 0, torch.float32, 1e-5),
-                                                 (LAYER1, 1, torch.float32, 1e-5)])
+                                                 (LAYER1, 1, torch.float32, 1e-5),
+                                                 (LAYER2, 1, torch.float32, 1e-5),
+                                                 (STEM, 3, torch.float32, 1e-5)])
 def test_convolution_directions_are_adjoint_at_full_size(cuda, shape, pad, dtype, tol):
     xs, ws = shape
+    st = 2 if shape is STEM else 1
     x = _randn(xs, cuda, 7)
     w = _randn(ws, cuda, 8) * (2.0 / (ws[0] * ws[2] * ws[3])) ** 0.5
     if dtype == torch.bfloat16:
@@ -145,7 +150,7 @@ def test_convolution_directions_are_adjoint_at_full_size(cuda, shape, pad, dtype
         w = w.to(dtype).contiguous(memory_format=torch.channels_last)
     dy = None
     ran = []
-    for v, y in _variants(conv_ops.n_fwd_algos(dtype), lambda v: conv_ops.conv_forward(x, w, None, pad, 1, 1, 1, v)):
+    for v, y in _variants(conv_ops.n_fwd_algos(dtype), lambda v: conv_ops.conv_forward(x, w, None, pad, st, 1, 1, v)):
         ran.append(v)
         if dy is None:
             dy = _randn(tuple(y.shape), cuda, 9)
@@ -156,27 +161,30 @@ def test_convolution_directions_are_adjoint_at_full_size(cuda, shape, pad, dtype
         # sqrt(n) * rms(y) * rms(dy) (a wrong operand, e.g. transposed weights, is off by ~0.2 of it)
         scale = (y.numel() ** 0.5) * float(y.float().pow(2).mean().sqrt()) * float(dy.float().pow(2).mean().sqrt())
         for vd, dx in _variants(conv_ops.n_bwd_ip_algos(dtype), lambda vd: conv_ops.conv_backward_input(
-                list(xs), dy, w, pad, 1, 1, 1, vd)):
+                list(xs), dy, w, pad, st, 1, 1, vd)):
             assert abs(lhs - _dot(dx, x)) < tol * scale, (v, vd)
         ran_w = []
         for vw, dw in _variants(conv_ops.n_bwd_wt_algos(dtype), lambda vw: conv_ops.conv_backward_weight(
-                list(ws), dy, x, pad, 1, 1, 1, vw)):
+                list(ws), dy, x, pad, st, 1, 1, vw)):
             assert abs(lhs - _dot(dw, w)) < tol * scale, (v, vw)
             ran_w.append(vw)
-        if shape is LAYER1:
+        if shape is LAYER1 or shape is LAYER2:
             assert ran_w == [0, 1, 2, 3]      # the one-kernel Winograd backward-weight included
+        if shape is STEM:
+            assert ran_w == [0, 1]
         # linearity of the forward in x (exact up to rounding of the two results)
         x2 = _randn(xs, cuda, 10)
         if dtype == torch.bfloat16:
             x2 = x2.to(dtype).contiguous(memory_format=torch.channels_last)
-        y2 = conv_ops.conv_forward(x2, w, None, pad, 1, 1, 1, v)
+        y2 = conv_ops.conv_forward(x2, w, None, pad, st, 1, 1, v)
         ys = conv_ops.conv_forward((x.float() + x2.float()).to(dtype).contiguous(
             memory_format=torch.channels_last if dtype == torch.bfloat16 else torch.contiguous_format),
-            w, None, pad, 1, 1, 1, v)
+            w, None, pad, st, 1, 1, v)
         lin_tol = (4 if dtype == torch.float32 else 3) * tol * float(ys.float().abs().max())
         assert float((ys.float() - (y.float() + y2.float())).abs().max()) < lin_tol, v
     # every variant that covers the shape ran: Winograd on the 3x3, three slices on the 1x1
-    expect = {(3, torch.float32): [0, 1, 2, 3], (3, torch.bfloat16): [0, 1], (1, torch.float32): [0, 1, 4]}
+    expect = {(3, torch.float32): [0, 1, 2, 3], (3, torch.bfloat16): [0, 1], (1, torch.float32): [0, 1, 4],
+              (7, torch.float32): [0, 1]}
     assert ran == expect[(ws[2], dtype)]
 
 
