@@ -401,29 +401,66 @@ __global__ __launch_bounds__(kThreads) void fused_kernel(const Plan p, const flo
 
   // output transform: this lane's tile is t0 + wt + r, its outputs k0 + wk + row(v)
   const uint32_t etile = t0 + wt + r;
-  if (etile >= p.T) return;
-  const uint32_t en = etile / per_img, er = etile - en * per_img;
+  const bool e_ok = etile < p.T;
+  const uint32_t en = e_ok ? etile / per_img : 0u, er = e_ok ? etile - en * per_img : 0u;
   const int eth = er / p.TW, etw = er - eth * p.TW;
   const int oh = 2 * eth, ow = 2 * etw;
   const bool row1 = oh + 1 < p.OH, col1 = ow + 1 < p.OW;
+  // output k0 + wk + 4 half + kofs(v), kofs(v) = 8 (v / 4) + v % 4: the lane's part of the address
+  // once, the rest a compile-time multiple of the plane size
+  const int kl = k0 + wk + 4 * half;
+  const size_t oplane = (size_t)p.OH * p.OW;
+  float* const obase = dst + ((size_t)en * p.M + kl) * oplane + (size_t)oh * p.OW + ow;
+  // the bias values of this lane's 16 outputs in one go (a load per output inside the loop below
+  // waited for each before it went on)
+  float bvs[16];
 #pragma unroll
   for (int v = 0; v < 16; ++v) {
-    const int k = k0 + wk + 8 * (v >> 2) + 4 * half + (v & 3);
+    const int k = kl + 8 * (v >> 2) + (v & 3);
+    bvs[v] = bias ? bias[k < p.M ? k : p.M - 1] : 0.f;
+  }
+  // Interior blocks (every lane has a whole 2x2 tile and all 64 outputs exist) store without
+  // predicates: four stores per output behind no branch.
+  const bool whole = __all(e_ok && row1 && col1) && k0 + FK <= p.M;
+  if (whole) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      float t[2][4];  // t = A^T m, m[a][b] = acc[4a + b][v]
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        t[0][b] = acc[b][v] + acc[4 + b][v] + acc[8 + b][v];
+        t[1][b] = acc[4 + b][v] - acc[8 + b][v] - acc[12 + b][v];
+      }
+      float* o = obase + (size_t)(8 * (v >> 2) + (v & 3)) * oplane;
+#pragma unroll
+      for (int a = 0; a < 2; ++a) {
+        float* q = o + (size_t)a * p.OW;
+        const float y0 = t[a][0] + t[a][1] + t[a][2] + bvs[v];
+        const float y1 = t[a][1] - t[a][2] - t[a][3] + bvs[v];
+        q[0] = ACCUM ? q[0] + y0 : y0;
+        q[1] = ACCUM ? q[1] + y1 : y1;
+      }
+    }
+    return;
+  }
+  if (!e_ok) return;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const int k = kl + 8 * (v >> 2) + (v & 3);
     if (k >= p.M) continue;
-    float t[2][4];  // t = A^T m, m[a][b] = acc[4a + b][v]
+    float t[2][4];
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
       t[0][b] = acc[b][v] + acc[4 + b][v] + acc[8 + b][v];
       t[1][b] = acc[4 + b][v] - acc[8 + b][v] - acc[12 + b][v];
     }
-    const float bv = bias ? bias[k] : 0.f;
-    float* o = dst + (((size_t)en * p.M + k) * p.OH + oh) * p.OW + ow;
+    float* o = obase + (size_t)(8 * (v >> 2) + (v & 3)) * oplane;
 #pragma unroll
     for (int a = 0; a < 2; ++a) {
       if (a == 1 && !row1) break;
       float* q = o + (size_t)a * p.OW;
-      const float y0 = t[a][0] + t[a][1] + t[a][2] + bv;
-      const float y1 = t[a][1] - t[a][2] - t[a][3] + bv;
+      const float y0 = t[a][0] + t[a][1] + t[a][2] + bvs[v];
+      const float y1 = t[a][1] - t[a][2] - t[a][3] + bvs[v];
       q[0] = ACCUM ? q[0] + y0 : y0;
       if (col1) q[1] = ACCUM ? q[1] + y1 : y1;
     }
